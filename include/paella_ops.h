@@ -1,0 +1,138 @@
+/*
+ * paella_ops.h -- C-ABI of the hand-written gfx950 operator kernels (fp32, NCHW, batch 1).
+ *
+ * These entry points replace the kernels that the reference obtains from its custom TVM build: in the
+ * reference the only call site is `run_()` inside every job adapter (reference
+ * jobs/tvm_mnist/tvm_mnist.cpp:24-33,41 and the ten sibling adapters), which executes one generated CUDA
+ * kernel per scheduler stage.  Here each of those kernels is an explicit launch function.
+ *
+ * Conventions
+ *   - all tensor pointers are DEVICE pointers to contiguous fp32 NCHW data with N == 1; a channel slice
+ *     of a larger tensor is contiguous for N == 1, so "write into channels [off, off+K) of a concat
+ *     buffer" is expressed by offsetting the pointer;
+ *   - `stream` is a hipStream_t passed as void*;
+ *   - `notifier` is a device pointer to an llis::job::FinishedBlockNotifier (or NULL for un-instrumented
+ *     launches); when non-NULL every workgroup calls notifier->start(job_id) on entry and
+ *     notifier->end(job_id) on exit (reference include/llis/job/finished_block_notifier.h:18-94);
+ *   - every function returns 0 on success, a negative PAELLA_E* code for a rejected argument and a
+ *     positive hipError_t for a runtime failure.  Nothing falls back to the CPU.
+ */
+#ifndef PAELLA_OPS_H
+#define PAELLA_OPS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PAELLA_EINVAL (-1)   /* malformed descriptor */
+#define PAELLA_ENOSUP (-2)   /* shape class not implemented (e.g. grouped conv that is not depthwise) */
+
+enum paella_act { PAELLA_ACT_NONE = 0, PAELLA_ACT_RELU = 1, PAELLA_ACT_RELU6 = 2, PAELLA_ACT_PRELU = 3, PAELLA_ACT_CLIP = 4 };
+
+/* Resources of one launch, in the units the block-level scheduler accounts in
+ * (reference include/llis/job/job.h:62-76, src/server/sm_resources.cpp:36-66). */
+typedef struct paella_launch_dims {
+    unsigned grid;        /* number of workgroups */
+    unsigned block;       /* threads per workgroup */
+    unsigned lds_bytes;   /* LDS per workgroup */
+    unsigned vgprs;       /* vector registers per thread */
+} paella_launch_dims;
+
+/* ---------------------------------------------------------------- conv2d (O1 dense, O2 depthwise) */
+
+typedef struct paella_conv_desc {
+    int C, H, W;                 /* input */
+    int K, R, S;                 /* output channels, kernel */
+    int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+    int groups;                  /* 1 (implicit GEMM on MFMA) or C == K (depthwise) */
+    int act;                     /* enum paella_act, applied after bias and residual */
+    float act_lo, act_hi;        /* PAELLA_ACT_CLIP bounds */
+} paella_conv_desc;
+
+typedef struct paella_conv_plan {
+    paella_conv_desc d;
+    int P, Q;                    /* output extent */
+    int kind;                    /* 0 = MFMA implicit GEMM, 1 = depthwise */
+    int mi, ni, kw;              /* per-wave tile = (32*mi) x (32*ni) outputs, kw waves split the reduction */
+    int m_pad, k_pad;            /* padded GEMM dims of the packed weight blob */
+    size_t blob_bytes;           /* size of the packed weight blob (table + weights) */
+    paella_launch_dims dims;
+    double flops;                /* algorithmic: 2*K*(C/g)*R*S*P*Q */
+    double bytes;                /* algorithmic: 4*(C*H*W + K*(C/g)*R*S + K + K*P*Q [+K*P*Q residual]) */
+} paella_conv_plan;
+
+/* Pure host arithmetic: picks the kernel variant and launch shape.  tile_hint = 0 lets the library
+ * choose; otherwise mi<<8 | ni<<4 | log2(kw) forces a tile (used by the tuning sweeps and tests). */
+int paella_conv2d_plan(const paella_conv_desc* desc, int has_residual, int tile_hint, paella_conv_plan* plan);
+
+/* Re-lays out OIHW weights [K][C/g][R][S] into the blob the kernel reads (host memory to host memory). */
+int paella_conv2d_pack(const paella_conv_plan* plan, const float* w_oihw, void* blob_host);
+
+/* y = act(conv(x, w) + bias + residual); bias, residual, slope may be NULL (slope: PReLU, per channel). */
+int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
+                         const float* residual, const float* slope, float* y,
+                         void* stream, uint32_t job_id, void* notifier);
+
+/* ---------------------------------------------------------------- dense (O3) */
+
+/* y[o] = act(bias[o] + sum_i x[i] * w[o][i]); w is the plain [O][I] row-major matrix. */
+int paella_dense_dims(int I, int O, paella_launch_dims* dims);
+int paella_dense_launch(const float* x, const float* w, const float* bias, float* y, int I, int O, int act,
+                        void* stream, uint32_t job_id, void* notifier);
+
+/* ---------------------------------------------------------------- pooling (O4, O5) */
+
+typedef struct paella_pool_desc {
+    int C, H, W;
+    int R, S, stride_h, stride_w, pad_h, pad_w;
+    int ceil_mode;
+    int is_avg;                  /* 0 = max (padding never selected), 1 = average */
+    int count_include_pad;       /* average only */
+} paella_pool_desc;
+
+int paella_pool_out(int in, int k, int stride, int pad, int ceil_mode);
+int paella_pool2d_dims(const paella_pool_desc* d, paella_launch_dims* dims);
+int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y,
+                         void* stream, uint32_t job_id, void* notifier);
+
+/* y[c] = mean over HW of x[c][:] */
+int paella_global_avgpool_dims(int C, int HW, paella_launch_dims* dims);
+int paella_global_avgpool_launch(const float* x, float* y, int C, int HW,
+                                 void* stream, uint32_t job_id, void* notifier);
+
+/* ---------------------------------------------------------------- elementwise (O6), copy (O7) */
+
+/* y = act(a*scale[c] + shift[c] + b): b, scale, shift may be NULL.  Covers residual add(+ReLU),
+ * standalone per-channel scale-shift(+ReLU), ReLU, clip and PReLU (slope per channel). */
+int paella_eltwise_dims(int C, int HW, paella_launch_dims* dims);
+int paella_eltwise_launch(const float* a, const float* b, const float* scale, const float* shift,
+                          const float* slope, float* y, int C, int HW, int act, float lo, float hi,
+                          void* stream, uint32_t job_id, void* notifier);
+
+/* Plain device copy of n floats (only used where a concat cannot be elided). */
+int paella_copy_dims(size_t n, paella_launch_dims* dims);
+int paella_copy_launch(const float* x, float* y, size_t n, void* stream, uint32_t job_id, void* notifier);
+
+/* ---------------------------------------------------------------- softmax, LRN (O8) */
+
+int paella_softmax_dims(int rows, int cols, paella_launch_dims* dims);
+int paella_softmax_launch(const float* x, float* y, int rows, int cols,
+                          void* stream, uint32_t job_id, void* notifier);
+
+int paella_lrn_dims(int C, int HW, paella_launch_dims* dims);
+int paella_lrn_launch(const float* x, float* y, int C, int HW, int size, float alpha, float beta, float k,
+                      void* stream, uint32_t job_id, void* notifier);
+
+/* Vector registers per thread of a kernel, read from the loaded code object (needs a GPU).
+ * family: "dense", "pool", "gap", "eltwise", "copy", "softmax", "lrn". */
+int paella_kernel_vgprs(const char* family, unsigned* vgprs);
+/* Same for a conv variant: kind 0 = MFMA implicit GEMM with tile (mi, ni, kw), kind 1 = depthwise. */
+int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

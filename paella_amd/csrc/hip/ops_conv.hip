@@ -1,0 +1,426 @@
+// conv2d for gfx950 (fp32, NCHW, batch 1): implicit GEMM on the fp32 MFMA pipe and a depthwise kernel.
+//
+// GEMM view:  Y[m][n] = sum_k Wt[m][k] * X~[k][n]   with m = output channel, n = output pixel (p*Q+q),
+// k = (c, r, s).  Output pixels of one channel are contiguous in NCHW, so the MFMA "column" index is the
+// pixel: operand loads of X~ and stores of Y are unit-stride across the 32 lanes of a half wave.
+//
+// One wave owns a (32*MI) x (32*NI) output tile and a contiguous slice of the reduction; the KW waves of a
+// workgroup share the tile and split k, then add their partial tiles through LDS in fixed wave order
+// (deterministic) before the fused epilogue bias -> residual -> activation -> store.
+//
+// Operand feeding (v_mfma_f32_32x32x2_f32; lane l supplies A[l%32][l/32] and B[l/32][l%32]):
+//   * weights are pre-packed on the host as float4 groups [k/4][m][4], so lane (i, kk) fetches the four
+//     k values {8c + 4kk + t} of row i with one 16-byte load and a half wave reads 512 contiguous bytes;
+//   * the im2col operand is gathered straight from the activation tensor with raw buffer loads whose
+//     out-of-range offsets return 0: padding taps, the k tail and the pixel tail need no branches.  A
+//     per-layer table maps k -> {byte offset c*H*W + r*dil*W + s*dil, (r*dil) << 16 | (s*dil)}.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "paella_ops.h"
+#include <llis/job/finished_block_notifier.h>
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct ConvArgs {
+    const float* x;
+    const int2* table;
+    const float4* wpk;
+    const float* bias;
+    const float* residual;
+    const float* slope;
+    float* y;
+    int H, W, Q, PQ;
+    int sh, sw, ph, pw;
+    int K, m_pad, nchunks;
+    unsigned x_bytes;
+    int act;
+    float lo, hi;
+    uint32_t job_id;
+    llis::job::FinishedBlockNotifier* notifier;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act, float slope, float lo, float hi) {
+    switch (act) {
+        case PAELLA_ACT_RELU:  return fmaxf(v, 0.f);
+        case PAELLA_ACT_RELU6: return fminf(fmaxf(v, 0.f), 6.f);
+        case PAELLA_ACT_PRELU: return v > 0.f ? v : v * slope;
+        case PAELLA_ACT_CLIP:  return fminf(fmaxf(v, lo), hi);
+        default:               return v;
+    }
+}
+
+template <int MI, int NI>
+struct Frag {
+    float4 a[MI];
+    float b[NI][4];
+};
+
+template <int MI, int NI, int KW>
+__global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
+    if (p.notifier) p.notifier->start(p.job_id);
+
+    extern __shared__ float red[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 31;
+    const int kk = lane >> 5;
+    const int m0 = blockIdx.y * (32 * MI);
+    const int n0 = blockIdx.x * (32 * NI);
+
+    __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, p.x_bytes, 0x00027000);
+
+    int hb[NI], wb[NI], base[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int pix = n0 + ni * 32 + j;
+        const int ho = pix / p.Q;
+        const int wo = pix - ho * p.Q;
+        hb[ni] = (pix < p.PQ) ? ho * p.sh - p.ph : -0x10000000;
+        wb[ni] = wo * p.sw - p.pw;
+        base[ni] = (hb[ni] * p.W + wb[ni]) * 4;
+    }
+
+    const int cpw = (p.nchunks + KW - 1) / KW;
+    const int c_begin = wave * cpw;
+    const int c_end = min(p.nchunks, c_begin + cpw);
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+
+    auto load_tab = [&](int c, int4& t0, int4& t1) {
+        const int4* t = reinterpret_cast<const int4*>(p.table + c * 8 + kk * 4);
+        t0 = t[0];
+        t1 = t[1];
+    };
+    auto load_frag = [&](int c, const int4& t0, const int4& t1, Frag<MI, NI>& f) {
+        const float4* wrow = p.wpk + (size_t)(c * 2 + kk) * p.m_pad + m0 + j;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) f.a[mi] = wrow[mi * 32];
+        const int off[4] = {t0.x, t0.z, t1.x, t1.z};
+        const int rs[4] = {t0.y, t0.w, t1.y, t1.w};
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int h = hb[ni] + (rs[t] >> 16);
+                const int w = wb[ni] + (rs[t] & 0xFFFF);
+                const bool ok = ((unsigned)h < (unsigned)p.H) & ((unsigned)w < (unsigned)p.W);
+                const int voff = ok ? base[ni] + off[t] : -1;
+                f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, voff, 0, 0));
+            }
+        }
+    };
+
+    if (c_begin < c_end) {
+        int4 tc0, tc1, tn0, tn1;
+        Frag<MI, NI> cur, nxt;
+        load_tab(c_begin, tc0, tc1);
+        load_tab(c_begin + 1, tn0, tn1);  // the table carries two chunks of slack past k_pad
+        load_frag(c_begin, tc0, tc1, cur);
+        for (int c = c_begin; c < c_end; ++c) {
+            int4 tf0, tf1;
+            load_tab(c + 2, tf0, tf1);
+            if (c + 1 < c_end) load_frag(c + 1, tn0, tn1, nxt);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) {
+                    const float av = t == 0 ? cur.a[mi].x : t == 1 ? cur.a[mi].y : t == 2 ? cur.a[mi].z : cur.a[mi].w;
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, cur.b[ni][t], acc[mi][ni], 0, 0, 0);
+                    }
+                }
+            }
+            cur = nxt;
+            tn0 = tf0;
+            tn1 = tf1;
+        }
+    }
+
+    constexpr int NACC = MI * NI * 16;
+    auto epilogue = [&](int r, float v) {
+        const int tile = r >> 4;
+        const int e = r & 15;
+        const int mi = tile / NI;
+        const int ni = tile - mi * NI;
+        const int m = m0 + mi * 32 + (e >> 2) * 8 + kk * 4 + (e & 3);
+        const int pix = n0 + ni * 32 + j;
+        if (m < p.K && pix < p.PQ) {
+            if (p.bias) v += p.bias[m];
+            const size_t o = (size_t)m * p.PQ + pix;
+            if (p.residual) v += p.residual[o];
+            const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
+            p.y[o] = apply_act(v, p.act, sl, p.lo, p.hi);
+        }
+    };
+
+    if (KW == 1) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) epilogue((mi * NI + ni) * 16 + e, acc[mi][ni][e]);
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    red[((wave * NACC) + (mi * NI + ni) * 16 + e) * 64 + lane] = acc[mi][ni][e];
+        __syncthreads();
+        constexpr int RPW = NACC / KW;
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {
+            const int r = wave * RPW + rr;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < KW; ++w) v += red[((w * NACC) + r) * 64 + lane];
+            epilogue(r, v);
+        }
+    }
+
+    if (p.notifier) p.notifier->end(p.job_id);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Depthwise conv (groups == C == K): HBM-bound, one thread per output pixel, taps from L1/L2.
+
+struct DwArgs {
+    const float* x;
+    const float* w;  // [C][R][S]
+    const float* bias;
+    const float* residual;
+    const float* slope;
+    float* y;
+    int C, H, W, P, Q, R, S;
+    int sh, sw, ph, pw, dh, dw;
+    int act;
+    float lo, hi;
+    uint32_t job_id;
+    llis::job::FinishedBlockNotifier* notifier;
+};
+
+__global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
+    if (p.notifier) p.notifier->start(p.job_id);
+    const int c = blockIdx.y;
+    const int pix = blockIdx.x * 256 + threadIdx.x;
+    const int PQ = p.P * p.Q;
+    if (pix < PQ) {
+        const int ho = pix / p.Q;
+        const int wo = pix - ho * p.Q;
+        const float* xc = p.x + (size_t)c * p.H * p.W;
+        const float* wc = p.w + (size_t)c * p.R * p.S;
+        float acc = p.bias ? p.bias[c] : 0.f;
+        for (int r = 0; r < p.R; ++r) {
+            const int h = ho * p.sh - p.ph + r * p.dh;
+            if ((unsigned)h >= (unsigned)p.H) continue;
+            for (int s = 0; s < p.S; ++s) {
+                const int w = wo * p.sw - p.pw + s * p.dw;
+                if ((unsigned)w >= (unsigned)p.W) continue;
+                acc = fmaf(xc[(size_t)h * p.W + w], wc[r * p.S + s], acc);
+            }
+        }
+        const size_t o = (size_t)c * PQ + pix;
+        if (p.residual) acc += p.residual[o];
+        const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
+        p.y[o] = apply_act(acc, p.act, sl, p.lo, p.hi);
+    }
+    if (p.notifier) p.notifier->end(p.job_id);
+}
+
+typedef void (*ConvKernel)(ConvArgs);
+
+template <int MI, int NI>
+ConvKernel pick_kw(int kw) {
+    switch (kw) {
+        case 1: return conv_mfma_kernel<MI, NI, 1>;
+        case 2: return conv_mfma_kernel<MI, NI, 2>;
+        case 4: return conv_mfma_kernel<MI, NI, 4>;
+        case 8: return conv_mfma_kernel<MI, NI, 8>;
+        default: return nullptr;
+    }
+}
+
+ConvKernel pick_kernel(int mi, int ni, int kw) {
+    if (mi == 1 && ni == 1) return pick_kw<1, 1>(kw);
+    if (mi == 1 && ni == 2) return pick_kw<1, 2>(kw);
+    if (mi == 2 && ni == 1) return pick_kw<2, 1>(kw);
+    if (mi == 2 && ni == 2) return pick_kw<2, 2>(kw);
+    return nullptr;
+}
+
+int conv_out(int in, int k, int stride, int pad, int dil) { return (in + 2 * pad - dil * (k - 1) - 1) / stride + 1; }
+
+int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+}  // namespace
+
+extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, int tile_hint, paella_conv_plan* plan) {
+    if (!d || !plan) return PAELLA_EINVAL;
+    if (d->C <= 0 || d->H <= 0 || d->W <= 0 || d->K <= 0 || d->R <= 0 || d->S <= 0 || d->stride_h <= 0 ||
+        d->stride_w <= 0 || d->pad_h < 0 || d->pad_w < 0 || d->dil_h <= 0 || d->dil_w <= 0 || d->groups <= 0)
+        return PAELLA_EINVAL;
+    if (d->act < PAELLA_ACT_NONE || d->act > PAELLA_ACT_CLIP) return PAELLA_EINVAL;
+    const int P = conv_out(d->H, d->R, d->stride_h, d->pad_h, d->dil_h);
+    const int Q = conv_out(d->W, d->S, d->stride_w, d->pad_w, d->dil_w);
+    if (P <= 0 || Q <= 0) return PAELLA_EINVAL;
+    // Offsets are 32-bit byte offsets and (r*dil, s*dil) are packed into 16 bits each.
+    if ((double)d->C * d->H * d->W * 4 >= 2147483648.0 || (d->R - 1) * d->dil_h >= 0x7000 || (d->S - 1) * d->dil_w >= 0x7000)
+        return PAELLA_ENOSUP;
+
+    std::memset(plan, 0, sizeof(*plan));
+    plan->d = *d;
+    plan->P = P;
+    plan->Q = Q;
+    const int PQ = P * Q;
+    const int cg = d->C / d->groups;
+    plan->flops = 2.0 * d->K * cg * d->R * d->S * PQ;
+    plan->bytes = 4.0 * ((double)d->C * d->H * d->W + (double)d->K * cg * d->R * d->S + d->K + (double)d->K * PQ * (has_residual ? 2 : 1));
+
+    if (d->groups == 1) {
+        plan->kind = 0;
+        const int kdim = d->C * d->R * d->S;
+        const int k_pad = round_up(kdim, 8);
+        const int nchunks = k_pad / 8;
+        int mi, ni, kw;
+        if (tile_hint > 0) {
+            mi = (tile_hint >> 8) & 0xF;
+            ni = (tile_hint >> 4) & 0xF;
+            kw = 1 << (tile_hint & 0xF);
+            if (!pick_kernel(mi, ni, kw)) return PAELLA_EINVAL;
+        } else {
+            // Largest tile that still yields at least one workgroup per CU; otherwise the smallest.
+            const int target = 256;
+            auto tiles = [&](int a, int b) { return ((d->K + 32 * a - 1) / (32 * a)) * ((PQ + 32 * b - 1) / (32 * b)); };
+            if (d->K > 32 && tiles(2, 2) >= target) { mi = 2; ni = 2; }
+            else if (tiles(1, 2) >= target) { mi = 1; ni = 2; }
+            else if (d->K > 32 && tiles(2, 1) >= target && PQ <= 32) { mi = 2; ni = 1; }
+            else { mi = 1; ni = 1; }
+            kw = 4;
+            while (kw > 1 && nchunks / kw < 4) kw >>= 1;
+            if (tiles(mi, ni) * kw < 512 && nchunks / 8 >= 8) kw = 8;
+        }
+        plan->mi = mi;
+        plan->ni = ni;
+        plan->kw = kw;
+        plan->m_pad = round_up(d->K, 32 * mi);
+        plan->k_pad = k_pad;
+        const size_t table_bytes = (size_t)(k_pad + 16) * sizeof(int2);
+        plan->blob_bytes = table_bytes + (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
+        plan->dims.grid = (unsigned)(((PQ + 32 * ni - 1) / (32 * ni)) * (plan->m_pad / (32 * mi)));
+        plan->dims.block = 64u * kw;
+        plan->dims.lds_bytes = kw > 1 ? (unsigned)(kw * mi * ni * 16 * 64 * sizeof(float)) : 0u;
+        plan->dims.vgprs = 128;
+        return 0;
+    }
+    if (d->groups == d->C && d->K == d->C) {
+        plan->kind = 1;
+        plan->blob_bytes = (size_t)d->C * d->R * d->S * sizeof(float);
+        plan->dims.grid = (unsigned)(((PQ + 255) / 256) * d->C);
+        plan->dims.block = 256;
+        plan->dims.lds_bytes = 0;
+        plan->dims.vgprs = 32;
+        return 0;
+    }
+    return PAELLA_ENOSUP;
+}
+
+extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, void* blob_host) {
+    if (!plan || !w || !blob_host) return PAELLA_EINVAL;
+    const paella_conv_desc& d = plan->d;
+    if (plan->kind == 1) {
+        std::memcpy(blob_host, w, plan->blob_bytes);
+        return 0;
+    }
+    const int kdim = d.C * d.R * d.S;
+    int2* table = reinterpret_cast<int2*>(blob_host);
+    for (int k = 0; k < plan->k_pad + 16; ++k) {
+        if (k < kdim) {
+            const int c = k / (d.R * d.S);
+            const int r = (k / d.S) % d.R;
+            const int s = k % d.S;
+            table[k].x = (c * d.H * d.W + r * d.dil_h * d.W + s * d.dil_w) * 4;
+            table[k].y = ((r * d.dil_h) << 16) | (s * d.dil_w);
+        } else {
+            table[k].x = 0;
+            table[k].y = 0x7FFF0000;  // row far outside the image: the tap always reads as zero
+        }
+    }
+    float* wp = reinterpret_cast<float*>(reinterpret_cast<char*>(blob_host) + (size_t)(plan->k_pad + 16) * sizeof(int2));
+    std::memset(wp, 0, (size_t)(plan->k_pad / 4) * plan->m_pad * sizeof(float4));
+    for (int m = 0; m < d.K; ++m)
+        for (int k = 0; k < kdim; ++k) wp[((size_t)(k / 4) * plan->m_pad + m) * 4 + (k % 4)] = w[(size_t)m * kdim + k];
+    return 0;
+}
+
+extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
+                                    const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
+                                    void* notifier) {
+    if (!plan || !x || !blob_dev || !y) return PAELLA_EINVAL;
+    const paella_conv_desc& d = plan->d;
+    if (d.act == PAELLA_ACT_PRELU && !slope) return PAELLA_EINVAL;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
+    const int PQ = plan->P * plan->Q;
+    if (plan->kind == 0) {
+        ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw);
+        if (!kern) return PAELLA_EINVAL;
+        ConvArgs a;
+        a.x = x;
+        a.table = reinterpret_cast<const int2*>(blob_dev);
+        a.wpk = reinterpret_cast<const float4*>(reinterpret_cast<const char*>(blob_dev) + (size_t)(plan->k_pad + 16) * sizeof(int2));
+        a.bias = bias;
+        a.residual = residual;
+        a.slope = slope;
+        a.y = y;
+        a.H = d.H; a.W = d.W; a.Q = plan->Q; a.PQ = PQ;
+        a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
+        a.K = d.K; a.m_pad = plan->m_pad; a.nchunks = plan->k_pad / 8;
+        a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
+        a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
+        a.job_id = job_id;
+        a.notifier = nf;
+        dim3 grid((PQ + 32 * plan->ni - 1) / (32 * plan->ni), plan->m_pad / (32 * plan->mi));
+        if (plan->dims.lds_bytes > 65536) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->dims.lds_bytes);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
+        return (int)hipGetLastError();
+    }
+    DwArgs a;
+    a.x = x; a.w = reinterpret_cast<const float*>(blob_dev); a.bias = bias; a.residual = residual; a.slope = slope; a.y = y;
+    a.C = d.C; a.H = d.H; a.W = d.W; a.P = plan->P; a.Q = plan->Q; a.R = d.R; a.S = d.S;
+    a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w; a.dh = d.dil_h; a.dw = d.dil_w;
+    a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
+    a.job_id = job_id;
+    a.notifier = nf;
+    dim3 grid((PQ + 255) / 256, d.C);
+    hipLaunchKernelGGL(dwconv_kernel, grid, dim3(256), 0, st, a);
+    return (int)hipGetLastError();
+}
+
+extern "C" int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs) {
+    const void* fn = kind == 1 ? reinterpret_cast<const void*>(dwconv_kernel) : reinterpret_cast<const void*>(pick_kernel(mi, ni, kw));
+    if (!fn || !vgprs) return PAELLA_EINVAL;
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, fn);
+    if (e != hipSuccess) return (int)e;
+    *vgprs = (unsigned)attr.numRegs;
+    return 0;
+}

@@ -1,0 +1,408 @@
+// Memory-bound operators for gfx950 (fp32, NCHW, batch 1): dense (batch-1 GEMV), pooling, global average
+// pool, fused elementwise, copy, softmax, LRN.  Each is bounded by HBM traffic, so the kernels aim at
+// coalesced 16-byte accesses and wavefront (64-lane) reductions rather than at the matrix pipe.
+
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cstring>
+
+#include "paella_ops.h"
+#include <llis/job/finished_block_notifier.h>
+
+namespace {
+
+using Notifier = llis::job::FinishedBlockNotifier;
+
+__device__ __forceinline__ float act_apply(float v, int act, float slope, float lo, float hi) {
+    switch (act) {
+        case PAELLA_ACT_RELU:  return fmaxf(v, 0.f);
+        case PAELLA_ACT_RELU6: return fminf(fmaxf(v, 0.f), 6.f);
+        case PAELLA_ACT_PRELU: return v > 0.f ? v : v * slope;
+        case PAELLA_ACT_CLIP:  return fminf(fmaxf(v, lo), hi);
+        default:               return v;
+    }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------ dense
+// One wave per output row; lanes stride the row with float4 loads (x stays in L1/L2).
+__global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                    const float* __restrict__ bias, float* __restrict__ y, int I, int O,
+                                                    int act, uint32_t job_id, Notifier* notifier) {
+    if (notifier) notifier->start(job_id);
+    const int lane = threadIdx.x & 63;
+    const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (o < O) {
+        const float* wr = w + (size_t)o * I;
+        float acc = 0.f;
+        if ((I & 3) == 0) {
+            const float4* w4 = reinterpret_cast<const float4*>(wr);
+            const float4* x4 = reinterpret_cast<const float4*>(x);
+            for (int i = lane; i < I / 4; i += 64) {
+                const float4 a = w4[i], b = x4[i];
+                acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+            }
+        } else {
+            for (int i = lane; i < I; i += 64) acc += wr[i] * x[i];
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) y[o] = act_apply(acc + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f);
+    }
+    if (notifier) notifier->end(job_id);
+}
+
+// ------------------------------------------------------------------------------------------ pooling
+struct PoolArgs {
+    const float* x;
+    float* y;
+    int C, H, W, P, Q, R, S, sh, sw, ph, pw;
+    int is_avg, count_include_pad;
+    uint32_t job_id;
+    Notifier* notifier;
+};
+
+__global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
+    if (p.notifier) p.notifier->start(p.job_id);
+    const int PQ = p.P * p.Q;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx < p.C * PQ) {
+        const int c = idx / PQ;
+        const int pix = idx - c * PQ;
+        const int po = pix / p.Q;
+        const int qo = pix - po * p.Q;
+        const float* xc = p.x + (size_t)c * p.H * p.W;
+        const int h0 = po * p.sh - p.ph, w0 = qo * p.sw - p.pw;
+        if (p.is_avg) {
+            float acc = 0.f;
+            int valid = 0;
+            for (int r = 0; r < p.R; ++r) {
+                const int h = h0 + r;
+                if ((unsigned)h >= (unsigned)p.H) continue;
+                for (int s = 0; s < p.S; ++s) {
+                    const int w = w0 + s;
+                    if ((unsigned)w >= (unsigned)p.W) continue;
+                    acc += xc[(size_t)h * p.W + w];
+                    ++valid;
+                }
+            }
+            int div = valid;
+            if (p.count_include_pad) {
+                // window clipped to the padded extent [-pad, in + pad)
+                const int he = min(h0 + p.R, p.H + p.ph), we = min(w0 + p.S, p.W + p.pw);
+                div = (he - h0) * (we - w0);
+            }
+            p.y[idx] = div ? acc / (float)div : 0.f;
+        } else {
+            float m = -FLT_MAX;
+            for (int r = 0; r < p.R; ++r) {
+                const int h = h0 + r;
+                if ((unsigned)h >= (unsigned)p.H) continue;
+                for (int s = 0; s < p.S; ++s) {
+                    const int w = w0 + s;
+                    if ((unsigned)w >= (unsigned)p.W) continue;
+                    m = fmaxf(m, xc[(size_t)h * p.W + w]);
+                }
+            }
+            p.y[idx] = m;
+        }
+    }
+    if (p.notifier) p.notifier->end(p.job_id);
+}
+
+// One wave per channel.
+__global__ __launch_bounds__(256) void gap_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW,
+                                                  uint32_t job_id, Notifier* notifier) {
+    if (notifier) notifier->start(job_id);
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (c < C) {
+        const float* xc = x + (size_t)c * HW;
+        float acc = 0.f;
+        for (int i = lane; i < HW; i += 64) acc += xc[i];
+        acc = wave_sum(acc);
+        if (lane == 0) y[c] = acc / (float)HW;
+    }
+    if (notifier) notifier->end(job_id);
+}
+
+// ------------------------------------------------------------------------------------------ elementwise
+struct EltArgs {
+    const float* a;
+    const float* b;
+    const float* scale;
+    const float* shift;
+    const float* slope;
+    float* y;
+    int C, HW;
+    int act;
+    float lo, hi;
+    uint32_t job_id;
+    Notifier* notifier;
+};
+
+__device__ __forceinline__ float elt_one(const EltArgs& p, float a, float b, int c) {
+    float v = a;
+    if (p.scale) v *= p.scale[c];
+    if (p.shift) v += p.shift[c];
+    v += b;
+    return act_apply(v, p.act, p.act == PAELLA_ACT_PRELU ? p.slope[c] : 0.f, p.lo, p.hi);
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(256) void eltwise_kernel(EltArgs p) {
+    if (p.notifier) p.notifier->start(p.job_id);
+    const size_t n = (size_t)p.C * p.HW;
+    if (VEC4) {
+        const size_t i4 = (size_t)blockIdx.x * 256 + threadIdx.x;
+        if (i4 * 4 < n) {
+            const int c = (int)((i4 * 4) / p.HW);  // HW % 4 == 0: the four lanes share a channel
+            const float4 a = reinterpret_cast<const float4*>(p.a)[i4];
+            float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p.b) b = reinterpret_cast<const float4*>(p.b)[i4];
+            float4 r;
+            r.x = elt_one(p, a.x, b.x, c);
+            r.y = elt_one(p, a.y, b.y, c);
+            r.z = elt_one(p, a.z, b.z, c);
+            r.w = elt_one(p, a.w, b.w, c);
+            reinterpret_cast<float4*>(p.y)[i4] = r;
+        }
+    } else {
+        const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+        if (i < n) p.y[i] = elt_one(p, p.a[i], p.b ? p.b[i] : 0.f, (int)(i / p.HW));
+    }
+    if (p.notifier) p.notifier->end(p.job_id);
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n,
+                                                   uint32_t job_id, Notifier* notifier) {
+    if (notifier) notifier->start(job_id);
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < n && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
+        *reinterpret_cast<float4*>(y + i) = *reinterpret_cast<const float4*>(x + i);
+    } else {
+        for (size_t k = i; k < n && k < i + 4; ++k) y[k] = x[k];
+    }
+    if (notifier) notifier->end(job_id);
+}
+
+// ------------------------------------------------------------------------------------------ softmax / LRN
+// One workgroup per row.
+__global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ x, float* __restrict__ y, int cols,
+                                                      uint32_t job_id, Notifier* notifier) {
+    if (notifier) notifier->start(job_id);
+    __shared__ float part[4];
+    const float* xr = x + (size_t)blockIdx.x * cols;
+    float* yr = y + (size_t)blockIdx.x * cols;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float m = -FLT_MAX;
+    for (int i = threadIdx.x; i < cols; i += 256) m = fmaxf(m, xr[i]);
+    m = wave_max(m);
+    if (lane == 0) part[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    __syncthreads();
+    float s = 0.f;
+    for (int i = threadIdx.x; i < cols; i += 256) s += expf(xr[i] - m);
+    s = wave_sum(s);
+    if (lane == 0) part[wave] = s;
+    __syncthreads();
+    s = (part[0] + part[1]) + (part[2] + part[3]);
+    for (int i = threadIdx.x; i < cols; i += 256) yr[i] = expf(xr[i] - m) / s;
+    if (notifier) notifier->end(job_id);
+}
+
+__global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW, int size,
+                                                  float alpha, float beta, float k, uint32_t job_id, Notifier* notifier) {
+    if (notifier) notifier->start(job_id);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx < (size_t)C * HW) {
+        const int c = (int)(idx / HW);
+        const int i = (int)(idx - (size_t)c * HW);
+        const int lo = (size - 1) / 2, hi = size - 1 - lo;
+        float sq = 0.f;
+        for (int cc = max(0, c - lo); cc <= min(C - 1, c + hi); ++cc) {
+            const float v = x[(size_t)cc * HW + i];
+            sq += v * v;
+        }
+        y[idx] = x[idx] / powf(k + alpha / (float)size * sq, beta);
+    }
+    if (notifier) notifier->end(job_id);
+}
+
+inline unsigned blocks_for(size_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+inline void set_dims(paella_launch_dims* d, unsigned grid, unsigned block, unsigned lds, unsigned vgprs) {
+    d->grid = grid;
+    d->block = block;
+    d->lds_bytes = lds;
+    d->vgprs = vgprs;
+}
+
+}  // namespace
+
+extern "C" {
+
+int paella_pool_out(int in, int k, int stride, int pad, int ceil_mode) {
+    const int num = in + 2 * pad - k;
+    int out;
+    if (ceil_mode) {
+        out = (num + stride - 1) / stride + 1;
+        if ((out - 1) * stride >= in + pad) --out;  // the last window must start inside input + left padding
+    } else {
+        out = num / stride + 1;
+    }
+    return out;
+}
+
+int paella_dense_dims(int I, int O, paella_launch_dims* dims) {
+    if (I <= 0 || O <= 0 || !dims) return PAELLA_EINVAL;
+    set_dims(dims, blocks_for(O, 4), 256, 0, 32);
+    return 0;
+}
+
+int paella_dense_launch(const float* x, const float* w, const float* bias, float* y, int I, int O, int act, void* stream,
+                        uint32_t job_id, void* notifier) {
+    if (!x || !w || !y || I <= 0 || O <= 0 || act < 0 || act > PAELLA_ACT_RELU6) return PAELLA_EINVAL;
+    hipLaunchKernelGGL(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
+                       (Notifier*)notifier);
+    return (int)hipGetLastError();
+}
+
+static int pool_check(const paella_pool_desc* d, int* P, int* Q) {
+    if (!d || d->C <= 0 || d->H <= 0 || d->W <= 0 || d->R <= 0 || d->S <= 0 || d->stride_h <= 0 || d->stride_w <= 0 ||
+        d->pad_h < 0 || d->pad_w < 0 || d->pad_h * 2 > d->R || d->pad_w * 2 > d->S)
+        return PAELLA_EINVAL;
+    *P = paella_pool_out(d->H, d->R, d->stride_h, d->pad_h, d->ceil_mode);
+    *Q = paella_pool_out(d->W, d->S, d->stride_w, d->pad_w, d->ceil_mode);
+    return (*P > 0 && *Q > 0) ? 0 : PAELLA_EINVAL;
+}
+
+int paella_pool2d_dims(const paella_pool_desc* d, paella_launch_dims* dims) {
+    int P, Q;
+    if (int rc = pool_check(d, &P, &Q)) return rc;
+    if (!dims) return PAELLA_EINVAL;
+    set_dims(dims, blocks_for((size_t)d->C * P * Q, 256), 256, 0, 32);
+    return 0;
+}
+
+int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y, void* stream, uint32_t job_id, void* notifier) {
+    int P, Q;
+    if (int rc = pool_check(d, &P, &Q)) return rc;
+    if (!x || !y) return PAELLA_EINVAL;
+    PoolArgs a;
+    a.x = x; a.y = y;
+    a.C = d->C; a.H = d->H; a.W = d->W; a.P = P; a.Q = Q; a.R = d->R; a.S = d->S;
+    a.sh = d->stride_h; a.sw = d->stride_w; a.ph = d->pad_h; a.pw = d->pad_w;
+    a.is_avg = d->is_avg; a.count_include_pad = d->count_include_pad;
+    a.job_id = job_id; a.notifier = (Notifier*)notifier;
+    hipLaunchKernelGGL(pool_kernel, dim3(blocks_for((size_t)d->C * P * Q, 256)), dim3(256), 0, (hipStream_t)stream, a);
+    return (int)hipGetLastError();
+}
+
+int paella_global_avgpool_dims(int C, int HW, paella_launch_dims* dims) {
+    if (C <= 0 || HW <= 0 || !dims) return PAELLA_EINVAL;
+    set_dims(dims, blocks_for(C, 4), 256, 0, 32);
+    return 0;
+}
+
+int paella_global_avgpool_launch(const float* x, float* y, int C, int HW, void* stream, uint32_t job_id, void* notifier) {
+    if (!x || !y || C <= 0 || HW <= 0) return PAELLA_EINVAL;
+    hipLaunchKernelGGL(gap_kernel, dim3(blocks_for(C, 4)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, job_id, (Notifier*)notifier);
+    return (int)hipGetLastError();
+}
+
+int paella_eltwise_dims(int C, int HW, paella_launch_dims* dims) {
+    if (C <= 0 || HW <= 0 || !dims) return PAELLA_EINVAL;
+    const size_t n = (size_t)C * HW;
+    set_dims(dims, (HW & 3) == 0 ? blocks_for(n / 4, 256) : blocks_for(n, 256), 256, 0, 32);
+    return 0;
+}
+
+int paella_eltwise_launch(const float* a, const float* b, const float* scale, const float* shift, const float* slope, float* y,
+                          int C, int HW, int act, float lo, float hi, void* stream, uint32_t job_id, void* notifier) {
+    if (!a || !y || C <= 0 || HW <= 0 || act < 0 || act > PAELLA_ACT_CLIP) return PAELLA_EINVAL;
+    if (act == PAELLA_ACT_PRELU && !slope) return PAELLA_EINVAL;
+    EltArgs p;
+    p.a = a; p.b = b; p.scale = scale; p.shift = shift; p.slope = slope; p.y = y;
+    p.C = C; p.HW = HW; p.act = act; p.lo = lo; p.hi = hi;
+    p.job_id = job_id; p.notifier = (Notifier*)notifier;
+    const size_t n = (size_t)C * HW;
+    const bool aligned = ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) == 0);
+    if ((HW & 3) == 0 && aligned) {
+        hipLaunchKernelGGL(eltwise_kernel<true>, dim3(blocks_for(n / 4, 256)), dim3(256), 0, (hipStream_t)stream, p);
+    } else {
+        hipLaunchKernelGGL(eltwise_kernel<false>, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, p);
+    }
+    return (int)hipGetLastError();
+}
+
+int paella_copy_dims(size_t n, paella_launch_dims* dims) {
+    if (n == 0 || !dims) return PAELLA_EINVAL;
+    set_dims(dims, blocks_for((n + 3) / 4, 256), 256, 0, 16);
+    return 0;
+}
+
+int paella_copy_launch(const float* x, float* y, size_t n, void* stream, uint32_t job_id, void* notifier) {
+    if (!x || !y || n == 0) return PAELLA_EINVAL;
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream, x, y, n, job_id,
+                       (Notifier*)notifier);
+    return (int)hipGetLastError();
+}
+
+int paella_softmax_dims(int rows, int cols, paella_launch_dims* dims) {
+    if (rows <= 0 || cols <= 0 || !dims) return PAELLA_EINVAL;
+    set_dims(dims, (unsigned)rows, 256, 16, 32);
+    return 0;
+}
+
+int paella_softmax_launch(const float* x, float* y, int rows, int cols, void* stream, uint32_t job_id, void* notifier) {
+    if (!x || !y || rows <= 0 || cols <= 0) return PAELLA_EINVAL;
+    hipLaunchKernelGGL(softmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, y, cols, job_id, (Notifier*)notifier);
+    return (int)hipGetLastError();
+}
+
+int paella_lrn_dims(int C, int HW, paella_launch_dims* dims) {
+    if (C <= 0 || HW <= 0 || !dims) return PAELLA_EINVAL;
+    set_dims(dims, blocks_for((size_t)C * HW, 256), 256, 0, 32);
+    return 0;
+}
+
+int paella_lrn_launch(const float* x, float* y, int C, int HW, int size, float alpha, float beta, float k, void* stream,
+                      uint32_t job_id, void* notifier) {
+    if (!x || !y || C <= 0 || HW <= 0 || size <= 0) return PAELLA_EINVAL;
+    hipLaunchKernelGGL(lrn_kernel, dim3(blocks_for((size_t)C * HW, 256)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, size, alpha,
+                       beta, k, job_id, (Notifier*)notifier);
+    return (int)hipGetLastError();
+}
+
+int paella_kernel_vgprs(const char* family, unsigned* vgprs) {
+    if (!family || !vgprs) return PAELLA_EINVAL;
+    const void* fn = nullptr;
+    if (!std::strcmp(family, "dense")) fn = (const void*)dense_kernel;
+    else if (!std::strcmp(family, "pool")) fn = (const void*)pool_kernel;
+    else if (!std::strcmp(family, "gap")) fn = (const void*)gap_kernel;
+    else if (!std::strcmp(family, "eltwise")) fn = (const void*)eltwise_kernel<true>;
+    else if (!std::strcmp(family, "copy")) fn = (const void*)copy_kernel;
+    else if (!std::strcmp(family, "softmax")) fn = (const void*)softmax_kernel;
+    else if (!std::strcmp(family, "lrn")) fn = (const void*)lrn_kernel;
+    if (!fn) return PAELLA_EINVAL;
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, fn);
+    if (e != hipSuccess) return (int)e;
+    *vgprs = (unsigned)attr.numRegs;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,133 @@
+"""Functional front-end over the operator C-ABI for tests and benches.
+
+Tensors are torch CUDA tensors (torch is only the allocator and stream provider here); weights are packed
+on the host with paella_conv2d_pack and uploaded.  Everything runs on the calling thread's current torch
+stream unless a stream handle is given.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _abi
+from ._abi import ConvDesc, ConvPlan, LaunchDims, PoolDesc, check
+
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_PRELU, ACT_CLIP = range(5)
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+class Conv2d:
+    """One planned conv layer: packed weights resident on the device."""
+
+    def __init__(self, w, bias=None, stride=1, pad=0, dil=1, groups=1, act=ACT_NONE, lo=0.0, hi=0.0,
+                 in_hw=None, has_residual=False, slope=None, tile_hint=0, device="cuda:0"):
+        lib = _abi.ops()
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        k, cg, r, s = w.shape
+        sh, sw = _pair(stride)
+        ph, pw = _pair(pad)
+        dh, dw = _pair(dil)
+        h, wd = in_hw
+        self.desc = ConvDesc(cg * groups, h, wd, k, r, s, sh, sw, ph, pw, dh, dw, groups, act, lo, hi)
+        self.plan = ConvPlan()
+        check(lib.paella_conv2d_plan(ctypes.byref(self.desc), int(has_residual), tile_hint, ctypes.byref(self.plan)),
+              "paella_conv2d_plan")
+        blob = np.zeros(self.plan.blob_bytes, dtype=np.uint8)
+        check(lib.paella_conv2d_pack(ctypes.byref(self.plan), w.ctypes.data, blob.ctypes.data), "paella_conv2d_pack")
+        self.blob = torch.from_numpy(blob).to(device)
+        self.bias = None if bias is None else torch.tensor(np.asarray(bias, np.float32), device=device)
+        self.slope = None if slope is None else torch.tensor(np.asarray(slope, np.float32), device=device)
+        self.lib = lib
+
+    def __call__(self, x, residual=None, out=None, stream=None, job_id=0, notifier=None):
+        p = self.plan
+        assert x.shape == (1, p.d.C, p.d.H, p.d.W), (tuple(x.shape), p.d.C, p.d.H, p.d.W)
+        y = out if out is not None else torch.empty((1, p.d.K, p.P, p.Q), device=x.device, dtype=torch.float32)
+        check(self.lib.paella_conv2d_launch(ctypes.byref(p), _ptr(x), ctypes.c_void_p(self.blob.data_ptr()),
+                                            _ptr(self.bias), _ptr(residual), _ptr(self.slope), _ptr(y),
+                                            _stream(stream), job_id, notifier), "paella_conv2d_launch")
+        return y
+
+
+def dense(x, w, bias=None, act=ACT_NONE, stream=None, job_id=0, notifier=None):
+    lib = _abi.ops()
+    o, i = w.shape
+    y = torch.empty((1, o), device=x.device, dtype=torch.float32)
+    check(lib.paella_dense_launch(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), i, o, act, _stream(stream), job_id, notifier),
+          "paella_dense_launch")
+    return y
+
+
+def pool2d(x, k, stride, pad=0, ceil_mode=False, is_avg=False, count_include_pad=True, stream=None, job_id=0,
+           notifier=None):
+    lib = _abi.ops()
+    _, c, h, w = x.shape
+    r, s = _pair(k)
+    sh, sw = _pair(stride)
+    ph, pw = _pair(pad)
+    d = PoolDesc(c, h, w, r, s, sh, sw, ph, pw, int(ceil_mode), int(is_avg), int(count_include_pad))
+    p = lib.paella_pool_out(h, r, sh, ph, int(ceil_mode))
+    q = lib.paella_pool_out(w, s, sw, pw, int(ceil_mode))
+    y = torch.empty((1, c, p, q), device=x.device, dtype=torch.float32)
+    check(lib.paella_pool2d_launch(ctypes.byref(d), _ptr(x), _ptr(y), _stream(stream), job_id, notifier),
+          "paella_pool2d_launch")
+    return y
+
+
+def global_avgpool(x, stream=None, job_id=0, notifier=None):
+    lib = _abi.ops()
+    _, c, h, w = x.shape
+    y = torch.empty((1, c, 1, 1), device=x.device, dtype=torch.float32)
+    check(lib.paella_global_avgpool_launch(_ptr(x), _ptr(y), c, h * w, _stream(stream), job_id, notifier),
+          "paella_global_avgpool_launch")
+    return y
+
+
+def eltwise(a, b=None, scale=None, shift=None, slope=None, act=ACT_NONE, lo=0.0, hi=0.0, stream=None, job_id=0,
+            notifier=None):
+    lib = _abi.ops()
+    c = a.shape[1]
+    y = torch.empty_like(a)
+    check(lib.paella_eltwise_launch(_ptr(a), _ptr(b), _ptr(scale), _ptr(shift), _ptr(slope), _ptr(y), c,
+                                    a.numel() // c, act, lo, hi, _stream(stream), job_id, notifier),
+          "paella_eltwise_launch")
+    return y
+
+
+def copy(x, stream=None, job_id=0, notifier=None):
+    lib = _abi.ops()
+    y = torch.empty_like(x)
+    check(lib.paella_copy_launch(_ptr(x), _ptr(y), x.numel(), _stream(stream), job_id, notifier), "paella_copy_launch")
+    return y
+
+
+def softmax(x, stream=None, job_id=0, notifier=None):
+    lib = _abi.ops()
+    cols = x.shape[-1]
+    y = torch.empty_like(x)
+    check(lib.paella_softmax_launch(_ptr(x), _ptr(y), x.numel() // cols, cols, _stream(stream), job_id, notifier),
+          "paella_softmax_launch")
+    return y
+
+
+def lrn(x, size, alpha, beta, k, stream=None, job_id=0, notifier=None):
+    lib = _abi.ops()
+    c = x.shape[1]
+    y = torch.empty_like(x)
+    check(lib.paella_lrn_launch(_ptr(x), _ptr(y), c, x.numel() // c, size, alpha, beta, k, _stream(stream), job_id,
+                                notifier), "paella_lrn_launch")
+    return y

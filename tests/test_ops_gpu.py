@@ -1,0 +1,199 @@
+"""Parity of the hand-written gfx950 operator kernels (through the C-ABI) against the CPU oracle.
+
+Tolerance for fp32 outputs: |got - ref| <= 1e-4 + 1e-3 * |ref|  (max-abs 1e-4 / rel 1e-3).
+Pure data-movement ops (max pool, copy) are bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as orc
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+RNG = np.random.default_rng(99)
+
+
+def rnd(*shape, scale=1.0):
+    return (RNG.standard_normal(shape) * scale).astype(np.float32)
+
+
+def close(got, ref):
+    got = got.detach().cpu().numpy() if hasattr(got, "detach") else got
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    bound = ATOL + RTOL * np.abs(ref)
+    assert np.all(err <= bound), "max err %g (bound there %g), %d bad of %d" % (err.max(), bound.flat[err.argmax()], (err > bound).sum(), err.size)
+
+
+# C, H, W, K, R, S, stride, pad, dil  -- the layer shapes of the BASELINE configs plus ragged edge cases
+CONV_SHAPES = [
+    (1, 28, 28, 8, 5, 5, 1, 2, 1),          # small CNN conv1
+    (8, 14, 14, 16, 5, 5, 1, 2, 1),         # small CNN conv2
+    (3, 224, 224, 64, 7, 7, 2, 3, 1),       # ResNet stem
+    (64, 56, 56, 64, 3, 3, 1, 1, 1),        # ResNet layer1
+    (64, 56, 56, 128, 3, 3, 2, 1, 1),       # stage entry, stride 2
+    (64, 56, 56, 128, 1, 1, 2, 0, 1),       # 1x1 stride-2 downsample
+    (256, 14, 14, 256, 3, 3, 1, 1, 1),
+    (512, 7, 7, 512, 3, 3, 1, 1, 1),        # 49 pixels: ragged pixel tile
+    (3, 299, 299, 32, 3, 3, 2, 0, 1),       # Inception stem
+    (128, 17, 17, 192, 1, 7, 1, (0, 3), 1),  # factorised 1x7
+    (160, 17, 17, 160, 7, 1, 1, (3, 0), 1),  # factorised 7x1
+    (48, 35, 35, 64, 5, 5, 1, 2, 1),
+    (384, 8, 8, 384, 1, 3, 1, (0, 1), 1),
+    (384, 8, 8, 384, 3, 1, 1, (1, 0), 1),
+    (960, 7, 7, 320, 1, 1, 1, 0, 1),        # MobileNetV2 pointwise
+    (24, 56, 56, 144, 1, 1, 1, 0, 1),
+    (5, 9, 11, 7, 3, 3, 1, 1, 1),           # nothing is a multiple of anything
+    (16, 12, 12, 40, 3, 3, 1, 2, 2),        # dilation
+    (2048, 1, 1, 1000, 1, 1, 1, 0, 1),      # a dense layer expressed as 1x1 conv
+]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES)
+def test_conv2d_mfma_parity(cuda, shape):
+    from paella_amd import ops
+    c, h, w, k, r, s, stride, pad, dil = shape
+    x = rnd(1, c, h, w)
+    wt = rnd(k, c, r, s, scale=(2.0 / (c * r * s)) ** 0.5)
+    b = rnd(k, scale=0.1)
+    ref = orc.conv2d(x, wt, b, stride=stride, pad=pad, dil=dil, act=orc.ACT_RELU)
+    conv = ops.Conv2d(wt, b, stride=stride, pad=pad, dil=dil, act=ops.ACT_RELU, in_hw=(h, w))
+    got = conv(torch.tensor(x, device=cuda))
+    torch.cuda.synchronize()
+    close(got, ref)
+
+
+@pytest.mark.parametrize("mi,ni,kwlog", [(1, 1, 0), (1, 1, 1), (1, 1, 2), (1, 1, 3), (1, 2, 0), (1, 2, 2), (1, 2, 3),
+                                         (2, 1, 1), (2, 1, 2), (2, 2, 0), (2, 2, 1), (2, 2, 2), (2, 2, 3), (2, 1, 3)])
+def test_conv2d_every_tile_variant(cuda, mi, ni, kwlog):
+    from paella_amd import ops
+    c, h, w, k = 40, 19, 23, 72
+    x, wt, b = rnd(1, c, h, w), rnd(k, c, 3, 3, scale=0.05), rnd(k, scale=0.1)
+    res = rnd(1, k, h, w)
+    slope = np.abs(rnd(k, scale=0.3))
+    ref = orc.conv2d(x, wt, b, pad=1, act=orc.ACT_PRELU, residual=res, slope=slope)
+    conv = ops.Conv2d(wt, b, pad=1, act=ops.ACT_PRELU, slope=slope, in_hw=(h, w), has_residual=True,
+                      tile_hint=(mi << 8) | (ni << 4) | kwlog)
+    assert (conv.plan.mi, conv.plan.ni, conv.plan.kw) == (mi, ni, 1 << kwlog)
+    got = conv(torch.tensor(x, device=cuda), residual=torch.tensor(res, device=cuda))
+    torch.cuda.synchronize()
+    close(got, ref)
+
+
+@pytest.mark.parametrize("act", [orc.ACT_NONE, orc.ACT_RELU6, orc.ACT_CLIP])
+def test_conv2d_epilogues_and_channel_slice_output(cuda, act):
+    """Output written into channels [8, 8+24) of a 40-channel concat buffer; the rest must stay untouched."""
+    from paella_amd import ops
+    c, h, w, k = 16, 10, 10, 24
+    x, wt = rnd(1, c, h, w, scale=3.0), rnd(k, c, 3, 3, scale=0.3)
+    ref = orc.conv2d(x, wt, None, pad=1, act=act, lo=-1.0, hi=2.0)
+    conv = ops.Conv2d(wt, None, pad=1, act=act, lo=-1.0, hi=2.0, in_hw=(h, w))
+    buf = torch.full((1, 40, h, w), 7.0, device=cuda)
+    conv(torch.tensor(x, device=cuda), out=buf[:, 8:32])
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    close(out[:, 8:32], ref)
+    assert np.all(out[:, :8] == 7.0) and np.all(out[:, 32:] == 7.0)
+
+
+def test_conv2d_is_deterministic(cuda):
+    from paella_amd import ops
+    x, wt = rnd(1, 64, 28, 28), rnd(96, 64, 3, 3, scale=0.05)
+    conv = ops.Conv2d(wt, None, pad=1, in_hw=(28, 28))
+    xd = torch.tensor(x, device=cuda)
+    a = conv(xd).cpu()
+    for _ in range(3):
+        assert torch.equal(conv(xd).cpu(), a)
+
+
+def test_conv2d_rejects_what_it_does_not_implement(cuda):
+    from paella_amd import ops
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.Conv2d(rnd(8, 2, 3, 3), None, groups=4, in_hw=(8, 8))
+    with pytest.raises(RuntimeError, match="invalid"):
+        ops.Conv2d(rnd(8, 8, 3, 3), None, stride=0, in_hw=(8, 8))
+
+
+@pytest.mark.parametrize("c,h,w,r,stride,pad", [(32, 112, 112, 3, 1, 1), (96, 112, 112, 3, 2, 1), (960, 7, 7, 3, 1, 1),
+                                                 (7, 13, 9, 3, 2, 1), (16, 20, 20, 5, 1, 2)])
+def test_depthwise_conv_parity(cuda, c, h, w, r, stride, pad):
+    from paella_amd import ops
+    x, wt, b = rnd(1, c, h, w), rnd(c, 1, r, r, scale=0.3), rnd(c, scale=0.1)
+    ref = orc.conv2d(x, wt, b, stride=stride, pad=pad, groups=c, act=orc.ACT_RELU6)
+    conv = ops.Conv2d(wt, b, stride=stride, pad=pad, groups=c, act=ops.ACT_RELU6, in_hw=(h, w))
+    assert conv.plan.kind == 1
+    close(conv(torch.tensor(x, device=cuda)), ref)
+
+
+@pytest.mark.parametrize("i,o", [(256, 10), (512, 1000), (2048, 1000), (1280, 1000), (25088, 512), (37, 11)])
+def test_dense_parity(cuda, i, o):
+    from paella_amd import ops
+    x, w, b = rnd(1, i), rnd(o, i, scale=i ** -0.5), rnd(o)
+    ref = orc.dense(x, w, b)
+    got = ops.dense(torch.tensor(x, device=cuda), torch.tensor(w, device=cuda), torch.tensor(b, device=cuda))
+    close(got, ref)
+
+
+POOLS = [
+    # c, h, w, k, stride, pad, ceil, avg, count_include_pad
+    (8, 28, 28, 2, 2, 0, False, False, True),
+    (16, 14, 14, 3, 3, 0, False, False, True),
+    (64, 112, 112, 3, 2, 1, False, False, True),
+    (64, 111, 111, 3, 2, 0, True, False, True),
+    (192, 28, 28, 3, 1, 1, False, False, True),
+    (64, 147, 147, 3, 2, 0, False, False, True),
+    (128, 56, 56, 2, 2, 0, False, True, True),
+    (288, 35, 35, 3, 1, 1, False, True, False),
+    (288, 35, 35, 3, 1, 1, False, True, True),
+    (5, 13, 15, 3, 2, 1, True, True, True),
+    (5, 13, 15, 3, 2, 0, True, True, False),
+]
+
+
+@pytest.mark.parametrize("case", POOLS)
+def test_pool_parity(cuda, case):
+    from paella_amd import ops
+    c, h, w, k, stride, pad, ceil, avg, cip = case
+    x = rnd(1, c, h, w)
+    got = ops.pool2d(torch.tensor(x, device=cuda), k, stride, pad, ceil, avg, cip).cpu().numpy()
+    if avg:
+        close(got, orc.avgpool2d(x, k, stride, pad, ceil, cip))
+    else:
+        np.testing.assert_array_equal(got, orc.maxpool2d(x, k, stride, pad, ceil))
+
+
+def test_global_avgpool_eltwise_copy_softmax_lrn_parity(cuda):
+    from paella_amd import ops
+    for c, hw in [(512, 7), (2048, 8), (1000, 13), (3, 5)]:
+        x = rnd(1, c, hw, hw)
+        close(ops.global_avgpool(torch.tensor(x, device=cuda)), orc.global_avgpool(x))
+    for shape in [(1, 64, 56, 56), (1, 7, 5, 3)]:
+        a, b = rnd(*shape), rnd(*shape)
+        c = shape[1]
+        sc, sf, sl = rnd(c), rnd(c), np.abs(rnd(c))
+        ad, bd = torch.tensor(a, device=cuda), torch.tensor(b, device=cuda)
+        close(ops.eltwise(ad, bd, act=ops.ACT_RELU), orc.add(a, b, orc.ACT_RELU))
+        close(ops.eltwise(ad, scale=torch.tensor(sc, device=cuda), shift=torch.tensor(sf, device=cuda), act=ops.ACT_RELU),
+              orc.scale_shift(a, sc, sf, orc.ACT_RELU))
+        close(ops.eltwise(ad, slope=torch.tensor(sl, device=cuda), act=ops.ACT_PRELU), orc.scale_shift(a, None, None, orc.ACT_PRELU, sl))
+        close(ops.eltwise(ad, act=ops.ACT_CLIP, lo=-0.3, hi=0.6), orc.scale_shift(a, None, None, orc.ACT_CLIP, None, -0.3, 0.6))
+        assert torch.equal(ops.copy(ad), ad)
+    z = rnd(1, 1000, scale=4.0)
+    close(ops.softmax(torch.tensor(z, device=cuda)), orc.softmax(z))
+    z2 = rnd(4420, 2, scale=3.0)
+    close(ops.softmax(torch.tensor(z2, device=cuda)), orc.softmax(z2))
+    x = rnd(1, 64, 28, 28, scale=3.0)
+    close(ops.lrn(torch.tensor(x, device=cuda), 5, 1e-4, 0.75, 1.0), orc.lrn(x, 5, 1e-4, 0.75, 1.0))
+    close(ops.lrn(torch.tensor(x, device=cuda), 4, 0.3, 0.6, 2.0), orc.lrn(x, 4, 0.3, 0.6, 2.0))
+
+
+def test_conv_linearity_at_full_size(cuda):
+    """Size-independent property at a BASELINE-sized layer: conv(x, w1 + w2) == conv(x, w1) + conv(x, w2)."""
+    from paella_amd import ops
+    x = torch.tensor(rnd(1, 64, 112, 112), device=cuda)
+    w1, w2 = rnd(64, 64, 3, 3, scale=0.05), rnd(64, 64, 3, 3, scale=0.05)
+    ya = ops.Conv2d(w1 + w2, None, pad=1, in_hw=(112, 112))(x)
+    yb = ops.Conv2d(w1, None, pad=1, in_hw=(112, 112))(x) + ops.Conv2d(w2, None, pad=1, in_hw=(112, 112))(x)
+    close(ya, yb.cpu().numpy())
