@@ -116,7 +116,7 @@ template <typename T, typename U>
 LLIS_HOSTDEV inline T to_bits(const U& v) {
     static_assert(sizeof(T) == sizeof(U), "message type must be exactly one ring slot wide");
     T bits;
-    __builtin_memcpy(&bits, &v, sizeof(T));
+    __builtin_memcpy(&bits, static_cast<const void*>(&v), sizeof(T));
     return bits;
 }
 
@@ -124,7 +124,7 @@ template <typename U, typename T>
 LLIS_HOSTDEV inline U from_bits(const T& bits) {
     static_assert(sizeof(T) == sizeof(U), "message type must be exactly one ring slot wide");
     U v;
-    __builtin_memcpy(&v, &bits, sizeof(T));
+    __builtin_memcpy(static_cast<void*>(&v), &bits, sizeof(T));
     return v;
 }
 

@@ -1,0 +1,37 @@
+#pragma once
+// Process-wide state shared by the server, the job definitions it loads and the kernel library: the job
+// whose stage is being issued right now, and non-owning endpoints of the two completion channels
+// (workgroup messages from the GPU, copy-stage completions from runtime callback threads).
+// One definition lives in libllis_core.so so every loaded job sees the same copy
+// (reference include/llis/job/context.h:10-53, src/job/context.cpp:8-13).
+
+#include <llis/ipc/shm_channel.h>
+#include <llis/ipc/shm_primitive_channel.h>
+#include <llis/job/job.h>
+
+namespace llis {
+namespace job {
+
+class Context {
+  public:
+    static Job* get_current_job() { return current_job_; }
+    static void set_current_job(Job* job) { current_job_ = job; }
+
+    static void set_gpu2sched_channel(ipc::Gpu2SchedChannel* channel) { gpu2sched_channel_ = channel->fork(); }
+    static ipc::Gpu2SchedChannel* get_gpu2sched_channel() { return &gpu2sched_channel_; }
+
+    static void set_gpu2sched_block_time_channel(ipc::Gpu2SchedChannel* channel) { gpu2sched_block_time_channel_ = channel->fork(); }
+    static ipc::Gpu2SchedChannel* get_gpu2sched_block_time_channel() { return &gpu2sched_block_time_channel_; }
+
+    static void set_mem2sched_channel(ipc::ShmChannelCpuReader* channel) { mem2sched_channel_ = channel->fork(); }
+    static ipc::ShmChannelCpuWriter* get_mem2sched_channel() { return &mem2sched_channel_; }
+
+  private:
+    static Job* current_job_;
+    static ipc::Gpu2SchedChannel gpu2sched_channel_;
+    static ipc::Gpu2SchedChannel gpu2sched_block_time_channel_;
+    static ipc::ShmChannelCpuWriter mem2sched_channel_;
+};
+
+}  // namespace job
+}  // namespace llis

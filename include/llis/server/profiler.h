@@ -1,0 +1,50 @@
+#pragma once
+// Server-side recorder behind the PROFILER_CMD messages.  The wire protocol (sub-command enum, SAVE
+// carrying a path prefix) follows reference src/server/profiler.cpp:10-67 so a client's ProfilerClient
+// keeps working; recording covers kernel info and per-job event timelines, written on SAVE as
+// <prefix>_kernel_info.txt and <prefix>_job_events.txt in the reference's line formats
+// (reference src/server/profiler.cpp:76-131).  The other four files are created empty.
+
+#include <llis/ipc/defs.h>
+#include <llis/ipc/shm_channel.h>
+
+#include <chrono>
+#include <string>
+#include <tuple>
+#include <utility>
+#include <vector>
+
+namespace llis {
+namespace server {
+
+class Profiler {
+  public:
+    using TimePoint = std::chrono::steady_clock::time_point;
+
+    enum class JobEvent { JOB_SUBMITTED, KERNEL_SCHED_START, KERNEL_SCHED_ABORT, KERNEL_SUBMIT_START, KERNEL_SUBMIT_END, KERNEL_FINISHED, JOB_FINISHED };
+
+    explicit Profiler(ipc::ShmChannelCpuReader* c2s_channel) : c2s_channel_(c2s_channel) {}
+
+    // Consumes one PROFILER_CMD body from the request ring.
+    void handle_cmd();
+    void save(const std::string& path_prefix);
+
+    bool recording_kernel_info() const { return kernel_info_flag_; }
+    bool recording_job_events() const { return job_events_flag_; }
+
+    void record_kernel_info(TimePoint start, TimePoint end, unsigned num_blocks, unsigned num_threads_per_block, unsigned smem_size_per_block,
+                            unsigned num_registers_per_thread, double priority, unsigned job_ref_id);
+    void record_job_event(JobId job_id, JobEvent event);
+
+  private:
+    ipc::ShmChannelCpuReader* c2s_channel_;
+    bool kernel_info_flag_ = false;
+    bool job_events_flag_ = false;
+    bool other_flags_[4] = {false, false, false, false};
+    std::vector<std::tuple<TimePoint, TimePoint, unsigned, unsigned, unsigned, unsigned, double, unsigned>> kernel_info_;
+    std::vector<std::vector<std::pair<JobEvent, TimePoint>>> jobs_events_cur_;
+    std::vector<std::vector<std::pair<JobEvent, TimePoint>>> jobs_events_all_;
+};
+
+}  // namespace server
+}  // namespace llis

@@ -1,0 +1,71 @@
+#include <llis/server/profiler.h>
+
+#include <cstdio>
+
+namespace llis {
+namespace server {
+
+void Profiler::handle_cmd() {
+    ProfilerMsgType sub;
+    c2s_channel_->read(&sub);
+    const unsigned v = (unsigned)sub;
+    if (sub == ProfilerMsgType::SAVE) {
+        std::string prefix;
+        c2s_channel_->read(&prefix);
+        save(prefix);
+        return;
+    }
+    const bool on = (v % 2) == 0;  // SET_* are even, UNSET_* odd
+    switch (v / 2) {
+        case 0: kernel_info_flag_ = on; break;
+        case 4: job_events_flag_ = on; break;
+        case 1: other_flags_[0] = on; break;
+        case 2: other_flags_[1] = on; break;
+        case 3: other_flags_[2] = on; break;
+        case 5: other_flags_[3] = on; break;
+        default: std::fprintf(stderr, "[llis] unknown profiler command %u ignored\n", v); break;
+    }
+}
+
+void Profiler::record_kernel_info(TimePoint start, TimePoint end, unsigned num_blocks, unsigned num_threads_per_block, unsigned smem_size_per_block,
+                                  unsigned num_registers_per_thread, double priority, unsigned job_ref_id) {
+    if (kernel_info_flag_) kernel_info_.emplace_back(start, end, num_blocks, num_threads_per_block, smem_size_per_block, num_registers_per_thread, priority, job_ref_id);
+}
+
+void Profiler::record_job_event(JobId job_id, JobEvent event) {
+    if (!job_events_flag_) return;
+    if (jobs_events_cur_.size() <= job_id) jobs_events_cur_.resize(job_id + 1);
+    auto& cur = jobs_events_cur_[job_id];
+    if (event == JobEvent::JOB_SUBMITTED) cur.clear();
+    cur.emplace_back(event, std::chrono::steady_clock::now());
+    if (event == JobEvent::JOB_FINISHED) {
+        jobs_events_all_.push_back(std::move(cur));
+        cur.clear();
+    }
+}
+
+void Profiler::save(const std::string& prefix) {
+    auto ns = [](TimePoint t) { return (long long)t.time_since_epoch().count(); };
+    if (FILE* fp = std::fopen((prefix + "_kernel_info.txt").c_str(), "w")) {
+        for (const auto& k : kernel_info_)
+            std::fprintf(fp, "%lld %lld %u %u %u %u %f %u\n", ns(std::get<0>(k)), ns(std::get<1>(k)), std::get<2>(k), std::get<3>(k), std::get<4>(k),
+                         std::get<5>(k), std::get<6>(k), std::get<7>(k));
+        std::fclose(fp);
+    }
+    if (FILE* fp = std::fopen((prefix + "_job_events.txt").c_str(), "w")) {
+        for (const auto& job : jobs_events_all_) {
+            for (const auto& ev : job)
+                std::fprintf(fp, "%u %f ", (unsigned)ev.first, std::chrono::duration<double, std::micro>(ev.second.time_since_epoch()).count());
+            std::fprintf(fp, "\n");
+        }
+        std::fclose(fp);
+    }
+    for (const char* name : {"_block_exec_times.txt", "_kernel_block_mis_alloc.txt", "_run_next_times.txt", "_resource_events.txt"}) {
+        if (FILE* fp = std::fopen((prefix + name).c_str(), "w")) std::fclose(fp);
+    }
+    kernel_info_.clear();
+    jobs_events_all_.clear();
+}
+
+}  // namespace server
+}  // namespace llis
