@@ -1,0 +1,72 @@
+/*
+ * paella_models.h -- C-ABI of the model zoo and graph executor that stand where the reference has
+ * TVM-compiled model libraries.
+ *
+ * In the reference every model adapter loads "<model>-cuda_llis-pack.so" through the TVM runtime and calls
+ * its "run" function, which launches one generated kernel per scheduler stage
+ * (reference jobs/tvm_mnist/tvm_mnist.cpp:24-47; model list: jobs/tvm_<model>/, compile lines
+ * sosp23_artifact/setup/onnx2tvm_all.sh:15-23).  Here a model is a static graph of the operators in
+ * paella_ops.h with seeded fp32 weights; an executor issues it one stage at a time so the scheduler can
+ * interleave stages of different requests.
+ *
+ * Model names: mnist, resnet18, resnet34, resnet50, mobilenetv2, inception_v3, squeezenet1_1, googlenet,
+ * densenet121, ultraface320, arcfaceresnet100.
+ *
+ * Seeded weights: tensor number t of a model (creation order, listed by paella_model_describe) is filled
+ * with value_i = float(normal_i * std_t), normal_i = sqrt(-2 ln u1) cos(2 pi u2),
+ * u = ((splitmix64(seed*0x9E3779B97F4A7C15 + t*0xD1B54A32D192ED03 + 2i [+1]) >> 11) + 0.5) * 2^-53,
+ * evaluated in double; "uniform" tensors take lo + (hi-lo)*u1; "constant" tensors a fixed value.
+ *
+ * Return value: 0 ok, negative PAELLA_E* for bad arguments, positive hipError_t for runtime failures.
+ */
+#ifndef PAELLA_MODELS_H
+#define PAELLA_MODELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "paella_ops.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct paella_model paella_model;   /* graph + packed weights resident on the device; shared, immutable */
+typedef struct paella_exec paella_exec;     /* activations of one in-flight request */
+
+/* ---- no GPU needed */
+/* Comma-separated list of model names. */
+const char* paella_model_names(void);
+/* Bytes of the input / output tensor of a model. */
+int paella_model_io_bytes(const char* name, size_t* in_bytes, size_t* out_bytes);
+/* JSON description of the graph (buffers, weight tensors with stream/std/shape, nodes in stage order).
+ * Writes at most cap bytes including the terminating NUL; *needed gets the full size. */
+int paella_model_describe(const char* name, char* json, size_t cap, size_t* needed);
+/* Algorithmic totals of one forward pass. */
+int paella_model_totals(const char* name, double* macs, double* params, double* flops, double* bytes, int* stages);
+/* Fills out[i] with element i of weight tensor `tensor` of the model under `seed` (host memory). */
+int paella_model_weight_values(const char* name, uint64_t seed, int tensor, float* out, size_t count);
+
+/* ---- device */
+/* Returns the process-wide instance for (name, seed), building and uploading it on first use. */
+int paella_model_get(const char* name, uint64_t seed, paella_model** out);
+int paella_model_num_stages(const paella_model* m);
+/* Launch shape of stage i in the scheduler's units (vgprs read from the loaded code object). */
+int paella_model_stage_dims(const paella_model* m, int stage, paella_launch_dims* dims);
+/* Operator name ("conv", "dwconv", "dense", "pool", "gap", "eltwise", "softmax", "lrn") and algorithmic work of stage i. */
+int paella_model_stage_work(const paella_model* m, int stage, const char** op, double* flops, double* bytes);
+
+int paella_exec_create(const paella_model* m, paella_exec** out);
+int paella_exec_destroy(paella_exec* e);
+/* Device pointers of the request's input and output tensors. */
+void* paella_exec_input(paella_exec* e);
+void* paella_exec_output(paella_exec* e);
+/* Issues stage i on `stream`; notifier may be NULL. */
+int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier);
+/* All stages back to back on one stream, un-instrumented (plain single-stream serving). */
+int paella_exec_forward(paella_exec* e, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

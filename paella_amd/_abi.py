@@ -12,8 +12,7 @@ c_void_p, c_size_t, c_char_p = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_char_p
 c_u32, c_u64 = ctypes.c_uint32, ctypes.c_uint64
 
 
-class LaunchDims(ctypes.Structure):
-    _fields_ = [("grid", c_uint), ("block", c_uint), ("lds_bytes", c_uint), ("vgprs", c_uint)]
+from ._abi_types import LaunchDims  # noqa: E402
 
 
 class ConvDesc(ctypes.Structure):

@@ -1,0 +1,319 @@
+// Graph executor behind include/paella_models.h: builds a model once per process (seeded weights, packed
+// and uploaded), and issues it one operator per call so a scheduler can interleave requests.
+
+#include "graph.h"
+
+#include "paella_hip.h"
+#include "paella_models.h"
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <utility>
+#include <vector>
+
+using namespace paella;
+
+struct StagePlan {
+    const Node* node = nullptr;
+    paella_conv_plan conv{};
+    paella_launch_dims dims{};
+    const char* op = "";
+    double flops = 0, bytes = 0;
+    // device pointers into the weight arena
+    const void* w = nullptr;
+    const float* bias = nullptr;
+    const float* slope = nullptr;
+    const float* scale = nullptr;
+    const float* shift = nullptr;
+};
+
+struct paella_model {
+    Graph g;
+    uint64_t seed = 0;
+    char* weights_dev = nullptr;
+    std::vector<StagePlan> stages;
+};
+
+struct paella_exec {
+    const paella_model* m = nullptr;
+    float* arena = nullptr;
+    float* ptr(const View& v) const { return v.buf < 0 ? nullptr : arena + m->g.buffers[v.buf].offset + v.off; }
+};
+
+namespace {
+
+std::mutex g_mtx;
+std::map<std::pair<std::string, uint64_t>, std::unique_ptr<paella_model>> g_models;
+std::map<std::string, std::unique_ptr<Graph>> g_graphs;
+
+const Graph* graph_of(const char* name) {
+    if (!name) return nullptr;
+    std::lock_guard<std::mutex> lk(g_mtx);
+    auto it = g_graphs.find(name);
+    if (it != g_graphs.end()) return it->second.get();
+    auto g = std::make_unique<Graph>();
+    try {
+        if (!build_model(name, g.get())) return nullptr;
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "paella_models: %s: %s\n", name, e.what());
+        return nullptr;
+    }
+    return (g_graphs[name] = std::move(g)).get();
+}
+
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+unsigned vgprs_or(const char* family, unsigned fallback) {
+    unsigned v = 0;
+    return paella_kernel_vgprs(family, &v) == 0 && v > 0 ? v : fallback;
+}
+
+int build(paella_model* m) {
+    const Graph& g = m->g;
+    // Pass 1: plan every node and lay out the weight arena.
+    std::vector<size_t> tensor_off(g.weights.size(), (size_t)-1);
+    std::vector<size_t> blob_off(g.nodes.size(), (size_t)-1);
+    size_t total = 0;
+    m->stages.resize(g.nodes.size());
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        const Node& n = g.nodes[i];
+        StagePlan& st = m->stages[i];
+        st.node = &n;
+        int rc = 0;
+        switch (n.op) {
+            case Op::Conv:
+                rc = paella_conv2d_plan(&n.conv, n.x2.buf >= 0, 0, &st.conv);
+                if (rc) return rc;
+                st.dims = st.conv.dims;
+                st.op = st.conv.kind == 0 ? "conv" : "dwconv";
+                st.flops = st.conv.flops;
+                st.bytes = st.conv.bytes;
+                {
+                    unsigned v = 0;
+                    if (paella_conv_kernel_vgprs(st.conv.kind, st.conv.mi, st.conv.ni, st.conv.kw, &v) == 0 && v) st.dims.vgprs = v;
+                }
+                blob_off[i] = total;
+                total += align256(st.conv.blob_bytes);
+                break;
+            case Op::Dense:
+                rc = paella_dense_dims(n.dense_in, n.dense_out, &st.dims);
+                st.op = "dense";
+                st.flops = 2.0 * n.dense_in * n.dense_out;
+                st.bytes = 4.0 * ((double)n.dense_in * n.dense_out + n.dense_in + 2.0 * n.dense_out);
+                st.dims.vgprs = vgprs_or("dense", st.dims.vgprs);
+                break;
+            case Op::Pool:
+                rc = paella_pool2d_dims(&n.pool, &st.dims);
+                st.op = "pool";
+                st.bytes = 4.0 * (n.x.numel() + n.y.numel());
+                st.dims.vgprs = vgprs_or("pool", st.dims.vgprs);
+                break;
+            case Op::GlobalAvgPool:
+                rc = paella_global_avgpool_dims(n.x.C, n.x.H * n.x.W, &st.dims);
+                st.op = "gap";
+                st.bytes = 4.0 * (n.x.numel() + n.y.numel());
+                st.dims.vgprs = vgprs_or("gap", st.dims.vgprs);
+                break;
+            case Op::Eltwise:
+                rc = paella_eltwise_dims(n.x.C, n.x.H * n.x.W, &st.dims);
+                st.op = "eltwise";
+                st.bytes = 4.0 * (n.x.numel() * (n.x2.buf >= 0 ? 2 : 1) + n.y.numel());
+                st.dims.vgprs = vgprs_or("eltwise", st.dims.vgprs);
+                break;
+            case Op::Softmax:
+                rc = paella_softmax_dims(n.rows, n.cols, &st.dims);
+                st.op = "softmax";
+                st.bytes = 4.0 * (n.x.numel() + n.y.numel());
+                st.dims.vgprs = vgprs_or("softmax", st.dims.vgprs);
+                break;
+            case Op::Lrn:
+                rc = paella_lrn_dims(n.x.C, n.x.H * n.x.W, &st.dims);
+                st.op = "lrn";
+                st.bytes = 4.0 * (n.x.numel() + n.y.numel());
+                st.dims.vgprs = vgprs_or("lrn", st.dims.vgprs);
+                break;
+        }
+        if (rc) return rc;
+        for (int id : {n.op == Op::Conv ? -1 : n.w, n.bias, n.slope, n.scale, n.shift}) {
+            if (id >= 0 && tensor_off[id] == (size_t)-1) {
+                tensor_off[id] = total;
+                total += align256(g.weights[id].numel() * sizeof(float));
+            }
+        }
+    }
+
+    // Pass 2: generate, pack, upload.
+    std::vector<char> host(total, 0);
+    std::vector<float> tmp;
+    for (size_t t = 0; t < g.weights.size(); ++t) {
+        if (tensor_off[t] == (size_t)-1) continue;
+        fill_weight(g.weights[t], m->seed, t, reinterpret_cast<float*>(host.data() + tensor_off[t]));
+    }
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        const Node& n = g.nodes[i];
+        if (n.op != Op::Conv) continue;
+        tmp.resize(g.weights[n.w].numel());
+        fill_weight(g.weights[n.w], m->seed, (uint64_t)n.w, tmp.data());
+        int rc = paella_conv2d_pack(&m->stages[i].conv, tmp.data(), host.data() + blob_off[i]);
+        if (rc) return rc;
+    }
+    void* dev = nullptr;
+    int rc = llis_hip_device_malloc(&dev, total ? total : 256);
+    if (rc) return rc;
+    rc = llis_hip_memcpy(dev, host.data(), total, LLIS_HIP_H2D);
+    if (rc) return rc;
+    m->weights_dev = reinterpret_cast<char*>(dev);
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        const Node& n = g.nodes[i];
+        StagePlan& st = m->stages[i];
+        auto at = [&](int id) -> const float* { return id >= 0 ? reinterpret_cast<const float*>(m->weights_dev + tensor_off[id]) : nullptr; };
+        st.w = n.op == Op::Conv ? (const void*)(m->weights_dev + blob_off[i]) : (const void*)at(n.w);
+        st.bias = at(n.bias);
+        st.slope = at(n.slope);
+        st.scale = at(n.scale);
+        st.shift = at(n.shift);
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* paella_model_names(void) { return model_names(); }
+
+int paella_model_io_bytes(const char* name, size_t* in_bytes, size_t* out_bytes) {
+    const Graph* g = graph_of(name);
+    if (!g) return PAELLA_EINVAL;
+    if (in_bytes) *in_bytes = g->input.numel() * sizeof(float);
+    if (out_bytes) *out_bytes = g->output.numel() * sizeof(float);
+    return 0;
+}
+
+int paella_model_describe(const char* name, char* json, size_t cap, size_t* needed) {
+    const Graph* g = graph_of(name);
+    if (!g) return PAELLA_EINVAL;
+    const std::string s = describe_json(*g);
+    if (needed) *needed = s.size() + 1;
+    if (json && cap) {
+        const size_t n = s.size() < cap - 1 ? s.size() : cap - 1;
+        std::memcpy(json, s.data(), n);
+        json[n] = 0;
+    }
+    return 0;
+}
+
+int paella_model_totals(const char* name, double* macs, double* params, double* flops, double* bytes, int* stages) {
+    const Graph* g = graph_of(name);
+    if (!g) return PAELLA_EINVAL;
+    if (macs) *macs = g->macs();
+    if (params) *params = g->params();
+    if (flops) *flops = 2.0 * g->macs();
+    if (bytes) {
+        double b = 4.0 * (g->input.numel() + g->output.numel()) + 4.0 * g->params();
+        for (const Node& n : g->nodes) b += 4.0 * (n.x.numel() + n.y.numel() + (n.x2.buf >= 0 ? n.x2.numel() : 0));
+        *bytes = b;
+    }
+    if (stages) *stages = (int)g->nodes.size();
+    return 0;
+}
+
+int paella_model_weight_values(const char* name, uint64_t seed, int tensor, float* out, size_t count) {
+    const Graph* g = graph_of(name);
+    if (!g || tensor < 0 || (size_t)tensor >= g->weights.size() || !out || count != g->weights[tensor].numel()) return PAELLA_EINVAL;
+    fill_weight(g->weights[tensor], seed, (uint64_t)tensor, out);
+    return 0;
+}
+
+int paella_model_get(const char* name, uint64_t seed, paella_model** out) {
+    const Graph* g = graph_of(name);
+    if (!g || !out) return PAELLA_EINVAL;
+    std::lock_guard<std::mutex> lk(g_mtx);
+    auto key = std::make_pair(std::string(name), seed);
+    auto it = g_models.find(key);
+    if (it == g_models.end()) {
+        auto m = std::make_unique<paella_model>();
+        m->g = *g;
+        m->seed = seed;
+        if (int rc = build(m.get())) return rc;
+        it = g_models.emplace(key, std::move(m)).first;
+    }
+    *out = it->second.get();
+    return 0;
+}
+
+int paella_model_num_stages(const paella_model* m) { return m ? (int)m->stages.size() : PAELLA_EINVAL; }
+
+int paella_model_stage_dims(const paella_model* m, int stage, paella_launch_dims* dims) {
+    if (!m || !dims || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
+    *dims = m->stages[stage].dims;
+    return 0;
+}
+
+int paella_model_stage_work(const paella_model* m, int stage, const char** op, double* flops, double* bytes) {
+    if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
+    if (op) *op = m->stages[stage].op;
+    if (flops) *flops = m->stages[stage].flops;
+    if (bytes) *bytes = m->stages[stage].bytes;
+    return 0;
+}
+
+int paella_exec_create(const paella_model* m, paella_exec** out) {
+    if (!m || !out) return PAELLA_EINVAL;
+    void* dev = nullptr;
+    if (int rc = llis_hip_device_malloc(&dev, m->g.arena_floats * sizeof(float))) return rc;
+    paella_exec* e = new paella_exec();
+    e->m = m;
+    e->arena = reinterpret_cast<float*>(dev);
+    *out = e;
+    return 0;
+}
+
+int paella_exec_destroy(paella_exec* e) {
+    if (!e) return PAELLA_EINVAL;
+    llis_hip_device_free(e->arena);
+    delete e;
+    return 0;
+}
+
+void* paella_exec_input(paella_exec* e) { return e ? e->ptr(e->m->g.input) : nullptr; }
+void* paella_exec_output(paella_exec* e) { return e ? e->ptr(e->m->g.output) : nullptr; }
+
+int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier) {
+    if (!e || stage < 0 || (size_t)stage >= e->m->stages.size()) return PAELLA_EINVAL;
+    const StagePlan& st = e->m->stages[stage];
+    const Node& n = *st.node;
+    const float* x = e->ptr(n.x);
+    const float* x2 = e->ptr(n.x2);
+    float* y = e->ptr(n.y);
+    switch (n.op) {
+        case Op::Conv:
+            return paella_conv2d_launch(&st.conv, x, st.w, st.bias, x2, st.slope, y, stream, job_id, notifier);
+        case Op::Dense:
+            return paella_dense_launch(x, reinterpret_cast<const float*>(st.w), st.bias, y, n.dense_in, n.dense_out, n.act, stream, job_id, notifier);
+        case Op::Pool:
+            return paella_pool2d_launch(&n.pool, x, y, stream, job_id, notifier);
+        case Op::GlobalAvgPool:
+            return paella_global_avgpool_launch(x, y, n.x.C, n.x.H * n.x.W, stream, job_id, notifier);
+        case Op::Eltwise:
+            return paella_eltwise_launch(x, x2, st.scale, st.shift, st.slope, y, n.x.C, n.x.H * n.x.W, n.act, n.lo, n.hi, stream, job_id, notifier);
+        case Op::Softmax:
+            return paella_softmax_launch(x, y, n.rows, n.cols, stream, job_id, notifier);
+        case Op::Lrn:
+            return paella_lrn_launch(x, y, n.x.C, n.x.H * n.x.W, n.lrn_size, n.lrn_alpha, n.lrn_beta, n.lrn_k, stream, job_id, notifier);
+    }
+    return PAELLA_EINVAL;
+}
+
+int paella_exec_forward(paella_exec* e, void* stream) {
+    if (!e) return PAELLA_EINVAL;
+    for (size_t i = 0; i < e->m->stages.size(); ++i)
+        if (int rc = paella_exec_launch_stage(e, (int)i, stream, 0, nullptr)) return rc;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+#pragma once
+// ModelJob -- the job definition shared by the model adapters: copy the request in, run the model one
+// operator per scheduler stage, copy the result out and wake the client.  It has the shape of the
+// reference's TVM adapters (reference jobs/tvm_mnist/tvm_mnist.cpp:10-64): same sizes, same stage
+// sequence mem -> kernels -> mem(pre-notify), same extern "C" init_job entry point; the kernels come from
+// the executor in paella_models.h instead of a TVM module.
+//
+// Differences, on purpose:
+//  * the device-to-host stage copies the model OUTPUT (the reference copies its input buffer back);
+//  * request buffers in the client's shared-memory pool cannot be registered with the runtime on this
+//    platform, so both copies go through a per-instance pinned staging buffer (filled on the server
+//    thread just before the H2D copy is issued, drained in on_complete()).
+
+#include <llis/job/context.h>
+#include <llis/job/coroutine_job.h>
+
+#include "paella_hip.h"
+#include "paella_models.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+
+namespace paella {
+
+class ModelJob : public llis::job::CoroutineJob {
+  public:
+    explicit ModelJob(const char* model_name) : name_(model_name) {
+        if (paella_model_io_bytes(model_name, &in_bytes_, &out_bytes_) != 0) throw std::invalid_argument(std::string("unknown model ") + model_name);
+    }
+
+    size_t get_input_size() override { return in_bytes_; }
+    size_t get_output_size() override { return out_bytes_; }
+    size_t get_param_size() override { return 4; }
+
+    void one_time_init() override {
+        const char* seed_env = std::getenv("LLIS_MODEL_SEED");
+        const uint64_t seed = seed_env ? std::strtoull(seed_env, nullptr, 10) : 1;
+        check(paella_model_get(name_.c_str(), seed, &model_), "paella_model_get");
+        check(paella_exec_create(model_, &exec_), "paella_exec_create");
+        void* p = nullptr;
+        check(llis_hip_host_alloc_pinned(&p, in_bytes_ + out_bytes_), "pinned staging");
+        staging_ = reinterpret_cast<char*>(p);
+        num_stages_ = paella_model_num_stages(model_);
+    }
+
+    void body(void* io_ptr) override {
+        io_ptr_ = io_ptr;
+        void* stream_unused = nullptr;
+        (void)stream_unused;
+
+        set_is_mem();
+        yield();
+        std::memcpy(staging_, io_ptr, in_bytes_);
+        check(llis_hip_memcpy_async(paella_exec_input(exec_), staging_, in_bytes_, LLIS_HIP_H2D, stream()), "H2D");
+        unset_is_mem();
+
+        for (int s = 0; s < num_stages_; ++s) {
+            paella_launch_dims d;
+            paella_model_stage_dims(model_, s, &d);
+            set_num_blocks(d.grid);
+            set_num_threads_per_block(d.block);
+            set_smem_size_per_block(d.lds_bytes);
+            set_num_registers_per_thread(d.vgprs);
+            yield();
+            check(paella_exec_launch_stage(exec_, s, stream(), get_id(), get_finished_block_notifier()), "stage launch");
+        }
+
+        set_is_mem();
+        set_pre_notify();
+        yield();
+        check(llis_hip_memcpy_async(staging_ + in_bytes_, paella_exec_output(exec_), out_bytes_, LLIS_HIP_D2H, stream()), "D2H");
+    }
+
+    // The output sits right after the input bytes of the request slot (what the client library reads).
+    void on_complete() override { std::memcpy(reinterpret_cast<char*>(io_ptr_) + in_bytes_, staging_ + in_bytes_, out_bytes_); }
+
+  private:
+    void* stream() { return reinterpret_cast<void*>(get_cuda_stream()); }
+
+    static void check(int rc, const char* what) {
+        if (rc != 0) {
+            std::fprintf(stderr, "[llis] model job: %s failed: %d (%s)\n", what, rc, rc > 0 ? llis_hip_error_string(rc) : "bad argument");
+            std::abort();
+        }
+    }
+
+    std::string name_;
+    size_t in_bytes_ = 0, out_bytes_ = 0;
+    paella_model* model_ = nullptr;
+    paella_exec* exec_ = nullptr;
+    char* staging_ = nullptr;
+    void* io_ptr_ = nullptr;
+    int num_stages_ = 0;
+};
+
+}  // namespace paella
+
+#define PAELLA_DEFINE_MODEL_JOB(ClassName, model_name)                                                   \
+    class ClassName : public paella::ModelJob {                                                          \
+      public:                                                                                            \
+        ClassName() : paella::ModelJob(model_name) {}                                                    \
+    };                                                                                                   \
+    extern "C" __attribute__((visibility("default"))) llis::job::Job* init_job() { return new ClassName(); }
