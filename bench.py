@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Headline benchmark: requests/s of the serving hot path on one MI355X.
+
+A "step" is one request served end to end: client library -> shared-memory request ring -> server poll loop
+-> full3 block-level scheduler -> one HIP kernel per stage with workgroup start/end notifications -> copy out
+-> completion.  Workload at N=1: ResNet-18 (batch 1, fp32, 1x3x224x224, seeded weights, synthetic input),
+the configuration the metric is quoted on.  W warm-up requests are served untimed, then exactly K requests
+are timed from first submission to last completion with the arrival process at saturation (closed by
+--concurrency outstanding requests, the reference's `--iat 0` mode); `value` = K / elapsed.
+
+Next to it, in the same run: the comparison arms (job-by-job `fifo` on a stream pool = plain multi-stream
+serving, `fifo` on one stream, and a direct single-stream forward loop without any server), an open-loop
+Poisson sweep with p50/p99, the roofline of the dominant kernel (MFMA implicit-GEMM conv, per-launch HIP
+events on its stream), the GPU->host notification latency probes and the CPU oracle timed on the host cores.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "requests/sec at p99 latency SLO (mixed-model Poisson load, 1 GPU); notify latency µs"
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True):
+    name = "bench%d_%s_%d" % (os.getpid(), sched, int(time.time() * 1000) % 100000)
+    with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4) as srv:
+        r = serve.client_run(srv.name, jobs, iat_us, concurrency, steps, warmup_jobs=warmup, seed=seed, dist="exp", pin_threads=True)
+    return r
+
+
+def conv_roofline(models, hip, model, reps):
+    """Per-launch durations of every stage of one forward pass, measured with HIP events on the launch stream."""
+    ex = models.Exec(model, seed=1)
+    stream = ctypes.c_void_p()
+    hip.llis_hip_stream_create(ctypes.byref(stream))
+    n = ex.num_stages
+    ev = []
+    for _ in range(n + 1):
+        e = ctypes.c_void_p()
+        hip.llis_hip_event_create(ctypes.byref(e))
+        ev.append(e)
+    work = [ex.stage_work(i) for i in range(n)]
+    for _ in range(3):
+        ex.forward(stream)
+    hip.llis_hip_stream_synchronize(stream)
+    total = [0.0] * n
+    for _ in range(reps):
+        hip.llis_hip_event_record(ev[0], stream)
+        for i in range(n):
+            ex.launch_stage(i, stream)
+            hip.llis_hip_event_record(ev[i + 1], stream)
+        hip.llis_hip_stream_synchronize(stream)
+        for i in range(n):
+            ms = ctypes.c_float()
+            hip.llis_hip_event_elapsed_ms(ev[i], ev[i + 1], ctypes.byref(ms))
+            total[i] += ms.value
+    per_stage = [t / reps * 1e3 for t in total]  # us
+    # back-to-back forward without events: single-stream direct serving rate
+    t0 = time.perf_counter()
+    direct_n = 200
+    for _ in range(direct_n):
+        ex.forward(stream)
+    hip.llis_hip_stream_synchronize(stream)
+    direct_rps = direct_n / (time.perf_counter() - t0)
+    for e in ev:
+        hip.llis_hip_event_destroy(e)
+    hip.llis_hip_stream_destroy(stream)
+    ex.close()
+    conv_flops = sum(w[1] for w in work if w[0] == "conv")
+    conv_us = sum(t for t, w in zip(per_stage, work) if w[0] == "conv")
+    conv_launches = sum(1 for w in work if w[0] == "conv")
+    by_op = {}
+    for t, w in zip(per_stage, work):
+        d = by_op.setdefault(w[0], {"launches": 0, "us": 0.0, "flops": 0.0, "bytes": 0.0})
+        d["launches"] += 1
+        d["us"] += t
+        d["flops"] += w[1]
+        d["bytes"] += w[2]
+    return {"per_stage_us": per_stage, "work": work, "conv_flops": conv_flops, "conv_us": conv_us, "conv_launches": conv_launches,
+            "by_op": by_op, "direct_rps": direct_rps, "forward_us": sum(per_stage)}
+
+
+def cpu_baseline(model, budget_s):
+    from oracle import models as om
+    from oracle import ops as orc
+    from paella_amd import models
+    desc = models.describe(model)
+    x = om.make_input(desc, 1)
+    om.run(desc, x, seed=1, fast=True)  # touch everything once
+    n, t0 = 0, time.perf_counter()
+    while True:
+        om.run(desc, x, seed=1, fast=True)
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or n >= 64:
+            break
+    return {"value": n / dt, "unit": "requests/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d %s forward passes (batch 1, fp32, same graph and seeded weights) with the float-accumulate CPU oracle, %.1f s" % (n, model, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--model", default="resnet18")
+    ap.add_argument("--concurrency", type=int, default=32)
+    ap.add_argument("--num-streams", type=int, default=64)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build serves from ONE GPU (one server process per GPU, no cross-GPU exchange); run with --gpus 1")
+        sys.exit(2)
+
+    from paella_amd import _abi, models, serve
+    hip = _abi.hip()
+    _abi.ops()
+    serve.lib()
+    os.environ.setdefault("LLIS_MODEL_SEED", "1")
+    job = serve.job_path("tvm_" + {"mobilenetv2": "mobilenet"}.get(args.model, args.model))
+    jobs = [(job, 1.0, args.concurrency)]
+    tot = models.totals(args.model)
+
+    log("[bench] timed arm: full3, %d streams, concurrency %d, %d warm-up + %d timed requests" % (args.num_streams, args.concurrency, args.warmup, args.steps))
+    main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup)
+    value = main_run["throughput_rps"]
+    log("[bench]   %.1f req/s, p50 %.0f us, p99 %.0f us" % (value, main_run["all"]["p50"], main_run["all"]["p99"]))
+
+    arms, sweep = {}, []
+    if not args.no_arms:
+        n_arm = max(500, args.steps // 2)
+        for label, sched, streams in [("fifo_multi_stream", "fifo", args.concurrency), ("fifo2_kernel_by_kernel", "fifo2", args.num_streams),
+                                      ("fifo_single_stream", "fifo", 1)]:
+            r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2)
+            arms[label] = {"requests_per_s": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"], "streams": streams}
+            log("[bench]   arm %-24s %.1f req/s, p99 %.0f us" % (label, r["throughput_rps"], r["all"]["p99"]))
+        single = serve_arm(serve, "full3", args.num_streams, [(job, 1.0, 1)], 1, 300, 50)
+        arms["full3_one_outstanding"] = {"requests_per_s": single["throughput_rps"], "p50_us": single["all"]["p50"], "p99_us": single["all"]["p99"]}
+        # open-loop Poisson arrivals at fractions of the saturation rate, full3 vs multi-stream fifo
+        for frac in (0.5, 0.8, 0.95):
+            rate = frac * min(value, arms["fifo_multi_stream"]["requests_per_s"])
+            point = {"offered_rps": rate}
+            for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+                r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2, iat_us=1e6 / rate)
+                point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"]}
+            sweep.append(point)
+            log("[bench]   poisson %.0f req/s: full3 p99 %.0f us, fifo p99 %.0f us" % (rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"]))
+
+    log("[bench] per-launch timing of the forward pass (HIP events)")
+    rl = conv_roofline(models, hip, args.model, reps=50)
+    achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
+    roofline = {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+                "traffic": None, "kernel": "conv_mfma_kernel (all %d conv launches of one %s forward pass)" % (rl["conv_launches"], args.model),
+                "flops_per_launch_avg": rl["conv_flops"] / rl["conv_launches"], "us_per_launch_avg": rl["conv_us"] / rl["conv_launches"]}
+    log("[bench]   conv: %.2f TFLOP/s (%.1f%% of fp32 MFMA peak), forward %.0f us, direct loop %.0f req/s" %
+        (achieved, 100 * roofline["frac"], rl["forward_us"], rl["direct_rps"]))
+
+    ring = ctypes.c_void_p()
+    lib = _abi.ops()
+    notify = {}
+    if lib.paella_ring_create(1024000, 1, ctypes.byref(ring)) == 0:
+        us = ctypes.c_double()
+        if lib.paella_ring_bench_drain(ring, 64, 6400, 50, 500, ctypes.byref(us)) == 0:
+            notify["ring_drain_64_blocks_us_per_kernel"] = us.value
+        flag, sync = ctypes.c_double(), ctypes.c_double()
+        if lib.paella_ring_bench_pingpong(100, 2000, ctypes.byref(flag), ctypes.byref(sync), None) == 0:
+            notify["launch_plus_flag_store_us"] = flag.value
+            notify["launch_plus_stream_sync_us"] = sync.value
+        lib.paella_ring_destroy(ring)
+
+    cpu = None if args.no_cpu else cpu_baseline(args.model, args.cpu_seconds)
+
+    out = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "requests/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_run["elapsed_us"] / 1e3 / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s batch 1 fp32 1x3x224x224, seeded weights, full3 scheduler, %d streams, saturation with %d outstanding requests" %
+                               (args.model, args.num_streams, args.concurrency),
+                   "gmac_per_request": tot["macs"] / 1e9, "stages_per_request": tot["stages"] + 2},
+        "latency_us": {"p50": main_run["all"]["p50"], "p99": main_run["all"]["p99"], "mean": main_run["all"]["mean"]},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "arms": arms,
+        "poisson_sweep": sweep,
+        "direct_single_stream_rps": rl["direct_rps"],
+        "per_op_us": {k: {"launches": v["launches"], "us": v["us"], "gflop": v["flops"] / 1e9, "mbytes": v["bytes"] / 1e6} for k, v in rl["by_op"].items()},
+        "notify_us": notify,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

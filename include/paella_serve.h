@@ -1,0 +1,88 @@
+/*
+ * paella_serve.h -- C-ABI for running the llis server and the load generator INSIDE the calling process.
+ *
+ * The product binaries are paella_amd/bin/llis_server and llis_app_client (same options as the reference's
+ * llis_server and llis_app_client: reference src/server/server.cpp:203-235, app/client.cpp:246-330).  A
+ * bench or test harness that has already touched the GPU must not spawn them, so these entry points run
+ * exactly the same classes on threads of the caller:
+ *   paella_server_start   = main() of llis_server on a new thread (server poll loop)
+ *   paella_client_run     = main() of llis_app_client: register jobs, warm every instance, open-loop run
+ *   paella_client_single  = closed loop with one instance (reference tests/client/client_single_latency.cpp:16-36)
+ *                           that also carries real input bytes in and output bytes out
+ * Client and server still talk through the shared-memory rings and the datagram socket.
+ * Return value: 0 on success, -1 on error (message on stderr).
+ */
+#ifndef PAELLA_SERVE_H
+#define PAELLA_SERVE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct paella_server paella_server;
+
+typedef struct paella_server_options {
+    const char* name;          /* --name */
+    const char* sched;         /* --sched: fifo, fifo2, full3 */
+    unsigned num_streams;      /* --num_streams */
+    unsigned extra_kernels;    /* --extra_kernels */
+    float unfair;              /* --unfair */
+    unsigned sched_sleep;      /* --sched_sleep */
+    int mem_marker;            /* 1: ring-marker kernel reports copy stages, 0: runtime host callback */
+    int event_log;             /* 1: record the scheduler event log */
+    int cpu;                   /* pin the serving thread to this CPU, -1 = do not pin */
+} paella_server_options;
+
+int paella_server_start(const paella_server_options* options, paella_server** out);
+/* Stops the poll loop, joins the thread, destroys scheduler and rings. */
+int paella_server_stop(paella_server* server);
+/* Text of the event log recorded so far (call after paella_server_stop, or while the server is idle).
+ * Copies at most cap bytes including the NUL; returns the full length. */
+size_t paella_server_event_log(paella_server* server, char* buf, size_t cap);
+
+#define PAELLA_MAX_JOB_TYPES 16
+
+typedef struct paella_load_options {
+    const char* server_name;
+    int num_types;
+    const char* job_paths[PAELLA_MAX_JOB_TYPES];
+    float proportions[PAELLA_MAX_JOB_TYPES];
+    unsigned max_outstanding[PAELLA_MAX_JOB_TYPES];
+    double iat_us;             /* mean inter-arrival time; 0 = saturation */
+    int dist_exp;              /* 1 exponential (Poisson arrivals), 0 log-normal */
+    double ln_sigma;
+    int concurrency;           /* global cap on outstanding requests */
+    unsigned num_jobs;         /* measured requests */
+    unsigned warmup_jobs;      /* served before the clock starts, beyond the one run per pooled instance */
+    unsigned seed;
+    int pin_threads;           /* pin monitor/submit threads to CPUs 0 and 2 like the reference client */
+} paella_load_options;
+
+typedef struct paella_latency_stats {
+    double mean, p50, p90, p95, p99, max, sd;
+    uint64_t count;
+} paella_latency_stats;
+
+typedef struct paella_load_result {
+    double elapsed_us;         /* first submission to last completion of the measured requests */
+    double throughput_rps;
+    paella_latency_stats all;
+    paella_latency_stats per_type[PAELLA_MAX_JOB_TYPES];
+    unsigned queue_full_events, type_full_events;
+} paella_load_result;
+
+/* latencies_us (optional) receives the measured latencies in completion order; capacity num_jobs. */
+int paella_client_run(const paella_load_options* options, paella_load_result* result, double* latencies_us);
+
+/* n closed-loop requests on one instance of job_path; the same input is sent every time and the output
+ * of the last request is returned.  latencies_us (optional, capacity n) in microseconds. */
+int paella_client_single(const char* server_name, const char* job_path, const void* input, size_t in_bytes, void* output,
+                         size_t out_bytes, int n, double* latencies_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

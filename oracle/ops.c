@@ -326,3 +326,11 @@ void orc_fill_uniform(float* out, size_t n, uint64_t seed, uint64_t stream, doub
         out[i] = (float)(lo + (hi - lo) * u1);
     }
 }
+
+/* Number of threads the OpenMP loops above will use (reported as `cores` of the CPU baseline). */
+#ifdef _OPENMP
+#include <omp.h>
+int orc_num_threads(void) { return omp_get_max_threads(); }
+#else
+int orc_num_threads(void) { return 1; }
+#endif

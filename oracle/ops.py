@@ -174,3 +174,8 @@ def fill_uniform(shape, seed, stream, lo, hi):
     out = np.empty(shape, np.float32)
     _lib.orc_fill_uniform(_p(out), out.size, seed, stream, lo, hi)
     return out
+
+
+def num_threads():
+    _lib.orc_num_threads.restype = ctypes.c_int
+    return _lib.orc_num_threads()

@@ -38,192 +38,11 @@
 #include <thread>
 #include <vector>
 
+#include "serve/load_generator.h"
+
+using namespace llis::loadgen;
+
 namespace {
-
-using Clock = std::chrono::steady_clock;
-
-double us_since_epoch(Clock::time_point t) { return std::chrono::duration<double, std::micro>(t.time_since_epoch()).count(); }
-
-struct Stats {
-    double mean = 0, p50 = 0, p90 = 0, p95 = 0, p99 = 0, max = 0, sd = 0;
-};
-
-Stats summarize(std::vector<double>& v) {
-    Stats s;
-    if (v.empty()) return s;
-    std::sort(v.begin(), v.end());
-    const double n = (double)v.size();
-    double mean = 0, mean_sqr = 0;
-    for (double x : v) {
-        mean += x / n;
-        mean_sqr += x * x / n;
-    }
-    s.mean = mean;
-    s.sd = v.size() > 1 ? std::sqrt((mean_sqr - mean * mean) * (n / (n - 1))) : 0;
-    s.p50 = v[v.size() / 2];
-    s.p90 = v[(size_t)(n * 0.90)];
-    s.p95 = v[(size_t)(n * 0.95)];
-    s.p99 = v[(size_t)(n * 0.99)];
-    s.max = v.back();
-    return s;
-}
-
-struct Options {
-    std::string server_name, prefix = "llis_client", dist = "ln";
-    double iat = -1, ln_sigma = 2.0, fairness = -1;
-    int concurrency = -1;
-    unsigned num_jobs = 0, start_record_num = 0, seed = 1, sched_sleep = 0;
-    bool pin_threads = true;
-    // name-shaping switches (which parameters appear in the output file names, which one is the x column)
-    bool n_iat = false, n_lns = false, n_con = false, n_n = false, n_srn = false, n_seed = false, n_fair = false, n_scheds = false;
-    bool g_iat = false, g_lns = false, g_con = false, g_n = false, g_srn = false, g_seed = false, g_fair = false, g_scheds = false;
-};
-
-class LoadGenerator {
-  public:
-    LoadGenerator(llis::client::Client* client, const Options& opt, std::vector<float> props_cum, std::vector<unsigned> max_outstanding)
-        : client_(client), opt_(opt), props_cum_(std::move(props_cum)), max_outstanding_(std::move(max_outstanding)) {
-        const size_t types = props_cum_.size();
-        free_instances_.resize(types);
-        free_counts_ = std::vector<std::atomic<unsigned>>(types);
-        due_.resize(types);
-        outstanding_per_type_.assign(types, 0);
-        latencies_per_type_.resize(types);
-    }
-
-    void add_instance(unsigned type, llis::client::JobInstanceRef* inst) { free_instances_[type].push_back(inst); }
-
-    void publish_free_counts() {
-        for (size_t t = 0; t < free_instances_.size(); ++t) free_counts_[t].store((unsigned)free_instances_[t].size(), std::memory_order_release);
-    }
-
-    void run() {
-        std::thread monitor_thr([this] { monitor(); });
-        std::thread submit_thr([this] { submit(); });
-        if (opt_.pin_threads) {
-            pin(monitor_thr, 0);
-            pin(submit_thr, 2);
-        }
-        monitor_thr.join();
-        submit_thr.join();
-    }
-
-    double elapsed_us() const { return std::chrono::duration<double, std::micro>(end_time_ - start_time_).count(); }
-    std::vector<double>& latencies() { return latencies_; }
-    std::vector<std::vector<double>>& latencies_per_type() { return latencies_per_type_; }
-    const std::vector<unsigned>& timeline() const { return timeline_; }
-    unsigned queue_full_events() const { return num_queue_full_; }
-    unsigned type_full_events() const { return num_type_full_; }
-
-  private:
-    static void pin(std::thread& thr, int cpu) {
-        cpu_set_t set;
-        CPU_ZERO(&set);
-        CPU_SET(cpu, &set);
-        pthread_setaffinity_np(thr.native_handle(), sizeof(set), &set);  // best effort
-    }
-
-    void sample_timeline(double t) {
-        timeline_.push_back((unsigned)t);
-        for (unsigned n : outstanding_per_type_) timeline_.push_back(n);
-    }
-
-    // Caller holds mtx_.
-    void launch(unsigned type, double scheduled_arrival_us) {
-        free_counts_[type].fetch_sub(1, std::memory_order_release);
-        llis::client::JobInstanceRef* inst = free_instances_[type].back();
-        free_instances_[type].pop_back();
-        ++outstanding_per_type_[type];
-        inst->set_start_time(scheduled_arrival_us);
-        inst->launch();
-    }
-
-    void monitor() {
-        const auto very_start = Clock::now();
-        for (unsigned done = 0; done < opt_.num_jobs; ++done) {
-            llis::client::JobInstanceRef* inst = client_->wait();
-            const auto now = Clock::now();
-            const double latency = us_since_epoch(now) - inst->get_start_time();
-            const double t = std::chrono::duration<double, std::micro>(now - very_start).count();
-            const unsigned type = inst->get_job_ref_id();
-            {
-                std::lock_guard<std::mutex> lk(mtx_);
-                free_instances_[type].push_back(inst);
-                free_counts_[type].fetch_add(1, std::memory_order_release);
-                --outstanding_per_type_[type];
-                sample_timeline(t);
-                num_outstanding_.fetch_sub(1, std::memory_order_release);
-                while (!due_[type].empty() && !free_instances_[type].empty()) {
-                    launch(type, due_[type].front());
-                    due_[type].pop();
-                }
-            }
-            if (done >= opt_.start_record_num) {
-                latencies_.push_back(latency);
-                latencies_per_type_[type].push_back(latency);
-            }
-        }
-        end_time_ = Clock::now();
-    }
-
-    void submit() {
-        std::mt19937 gen(opt_.seed);
-        std::exponential_distribution<> d_exp(opt_.iat > 0 ? 1. / opt_.iat : 1.);
-        const double mu = opt_.iat > 0 ? std::log(opt_.iat) - opt_.ln_sigma * opt_.ln_sigma / 2 : 0;
-        std::lognormal_distribution<> d_ln(mu, opt_.ln_sigma);
-        std::uniform_real_distribution<float> d_type(0, 1);
-        const bool use_exp = opt_.dist == "exp";
-
-        double next_submit = 0;
-        start_time_ = Clock::now();
-        const double start_us = us_since_epoch(start_time_);
-        unsigned submitted = 0;
-
-        while (submitted < opt_.num_jobs) {
-            const double elapsed = std::chrono::duration<double, std::micro>(Clock::now() - start_time_).count();
-            if (elapsed < next_submit) continue;
-
-            if (num_outstanding_.load(std::memory_order_acquire) >= opt_.concurrency) {
-                ++num_queue_full_;
-                while (num_outstanding_.load(std::memory_order_acquire) >= opt_.concurrency) {
-                }
-            }
-            const unsigned type = (unsigned)(std::lower_bound(props_cum_.begin(), props_cum_.end(), d_type(gen)) - props_cum_.begin());
-            const unsigned t = std::min<unsigned>(type, (unsigned)props_cum_.size() - 1);
-            {
-                std::lock_guard<std::mutex> lk(mtx_);
-                if (free_counts_[t].load(std::memory_order_acquire) == 0) {
-                    ++num_type_full_;
-                    due_[t].push(start_us + next_submit);
-                } else {
-                    launch(t, start_us + next_submit);
-                    sample_timeline(elapsed);
-                }
-            }
-            num_outstanding_.fetch_add(1, std::memory_order_release);
-            ++submitted;
-            if (opt_.iat > 0) next_submit += use_exp ? d_exp(gen) : d_ln(gen);
-        }
-    }
-
-    llis::client::Client* client_;
-    const Options& opt_;
-    std::vector<float> props_cum_;
-    std::vector<unsigned> max_outstanding_;
-
-    std::mutex mtx_;
-    std::vector<std::vector<llis::client::JobInstanceRef*>> free_instances_;
-    std::vector<std::atomic<unsigned>> free_counts_;
-    std::vector<std::queue<double>> due_;
-    std::vector<unsigned> outstanding_per_type_;
-    std::atomic<int> num_outstanding_{0};
-
-    std::vector<double> latencies_;
-    std::vector<std::vector<double>> latencies_per_type_;
-    std::vector<unsigned> timeline_;
-    Clock::time_point start_time_, end_time_;
-    unsigned num_queue_full_ = 0, num_type_full_ = 0;
-};
 
 void append(std::ostringstream& os, bool named, bool grouped, bool want_grouped, const char* tag, double value) {
     if (named && grouped == want_grouped) os << tag << value;
@@ -243,7 +62,7 @@ int main(int argc, char** argv) {
                                      {"num_jobs", required_argument, nullptr, 'n'},    {"start_record_num", required_argument, nullptr, 'r'},
                                      {"seed", required_argument, nullptr, 's'},        {"prefix", required_argument, nullptr, 'p'},
                                      {"fairness", required_argument, nullptr, 'f'},    {"sched_sleep", required_argument, nullptr, 'h'},
-                                     {"dist", required_argument, nullptr, 'd'},        {"no_pin", no_argument, nullptr, 'P'}};
+                                     {"dist", required_argument, nullptr, 'd'},        {"warmup", required_argument, nullptr, 'w'},        {"no_pin", no_argument, nullptr, 'P'}};
     for (int i = 0; i < 16; ++i) long_opts.push_back(option{flag_names[i], no_argument, &flag_slot, i + 1});
     long_opts.push_back(option{nullptr, 0, nullptr, 0});
 
@@ -261,6 +80,7 @@ int main(int argc, char** argv) {
             case 'f': opt.fairness = std::atof(optarg); break;
             case 'h': opt.sched_sleep = (unsigned)std::atoi(optarg); break;
             case 'd': opt.dist = optarg; break;
+            case 'w': opt.warmup_jobs = (unsigned)std::atoi(optarg); break;
             case 'P': opt.pin_threads = false; break;
             default: return 2;
         }

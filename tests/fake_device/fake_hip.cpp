@@ -46,8 +46,9 @@ struct Stream {
     std::deque<Op> q;
 };
 
-std::mutex g_mtx;
-std::vector<Stream*> g_streams;
+// Leaked on purpose: the autorun thread may still be running while static destructors execute at exit.
+std::mutex& g_mtx = *new std::mutex();
+std::vector<Stream*>& g_streams = *new std::vector<Stream*>();
 uint64_t g_seq = 0;
 std::atomic<bool> g_autorun_started{false};
 std::atomic<unsigned long long> g_ops_executed{0};
