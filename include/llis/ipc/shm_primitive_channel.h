@@ -68,6 +68,10 @@ class ShmPrimitiveChannelBase {
     LLIS_HOSTDEV U read();
     template <typename U>
     LLIS_HOSTDEV void write(U val);
+    // Same, but the message store carries no release of its own: for producers that have already ordered
+    // their data before the message by other means.
+    template <typename U>
+    LLIS_HOSTDEV void write_relaxed(U val);
     template <typename U>
     LLIS_HOSTDEV bool can_read();
 
@@ -155,6 +159,15 @@ LLIS_HOSTDEV inline void publish(T* slot, T bits) {
 }
 
 template <typename T>
+LLIS_HOSTDEV inline void publish_relaxed(T* slot, T bits) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __hip_atomic_store(slot, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#else
+    __atomic_store_n(slot, bits, __ATOMIC_RELEASE);
+#endif
+}
+
+template <typename T>
 LLIS_HOSTDEV inline T peek(const T* slot) {
 #if defined(__HIP_DEVICE_COMPILE__)
     return __hip_atomic_load(slot, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -170,6 +183,13 @@ template <typename U>
 LLIS_HOSTDEV inline void ShmPrimitiveChannelBase<T, for_gpu>::write(U val) {
     const unsigned pos = detail::claim_slot(cursor_, count_ - 1);
     detail::publish(slots_ + pos, detail::to_bits<T>(val));
+}
+
+template <typename T, bool for_gpu>
+template <typename U>
+LLIS_HOSTDEV inline void ShmPrimitiveChannelBase<T, for_gpu>::write_relaxed(U val) {
+    const unsigned pos = detail::claim_slot(cursor_, count_ - 1);
+    detail::publish_relaxed(slots_ + pos, detail::to_bits<T>(val));
 }
 
 template <typename T, bool for_gpu>

@@ -25,7 +25,11 @@ namespace job {
 
 class FinishedBlockNotifier {
   public:
-    static constexpr unsigned noti_batch_size = 16;
+    // Workgroups per message.  The reference batches 16 on a 40-SM GPU (reference
+    // include/llis/job/finished_block_notifier.h:118); 64 keeps a comparable share of a 256-CU device per
+    // message and quarters the host's message rate.  Grids of up to 64 workgroups send exactly one start
+    // and one end message either way.
+    static constexpr unsigned noti_batch_size = 64;
 
     FinishedBlockNotifier() {}
     explicit FinishedBlockNotifier(ipc::Gpu2SchedChannel* gpu2sched_channel) {
@@ -37,15 +41,29 @@ class FinishedBlockNotifier {
 #if defined(__HIPCC__)
     __device__ __forceinline__ void start(JobId job_id) {
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
-            announce(&agg_counter_start_, 1, job_id);
+            announce<false>(&agg_counter_start_, 1, job_id);
         }
     }
 
+    // For arbitrary kernels: makes everything the workgroup wrote visible device-wide (cache write-back)
+    // before the end message can be seen.
     __device__ __forceinline__ void end(JobId job_id) {
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            announce(&agg_counter_end_, 0, job_id);
+            announce<true>(&agg_counter_end_, 0, job_id);
+        }
+    }
+
+    // For kernels that wrote ALL their results with device-scope write-through stores
+    // (__hip_atomic_store(..., __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)): every wave waits until its own
+    // stores have been acknowledged, then the barrier; no cache write-back is needed, which keeps the
+    // per-workgroup cost of the hook at one atomic.
+    __device__ __forceinline__ void end_written_through(JobId job_id) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
+            announce<false>(&agg_counter_end_, 0, job_id);
         }
     }
 #endif
@@ -56,6 +74,8 @@ class FinishedBlockNotifier {
 
   private:
 #if defined(__HIPCC__)
+    // ACQUIRE: the sender first acquires (device scope) what the other workgroups released before their bump.
+    template <bool ACQUIRE>
     __device__ __forceinline__ void announce(unsigned* counter, uint8_t is_start, JobId job_id) {
         const unsigned num_blocks = gridDim.x * gridDim.y * gridDim.z;
         const unsigned total = atomicInc(counter, num_blocks - 1) + 1;  // wraps to 0 after the last block
@@ -67,12 +87,13 @@ class FinishedBlockNotifier {
             covered = in_batch;
         }
         if (covered != 0) {
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            if (ACQUIRE) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             InstrumentInfo info;
             info.is_start = is_start;
             info.num = (uint8_t)covered;
             info.job_id = job_id;
-            gpu2sched_channel_.write(info);
+            // The counter chain already ordered every workgroup's data before this point.
+            gpu2sched_channel_.write_relaxed(info);
         }
     }
 #endif

@@ -26,6 +26,9 @@ extern "C" {
 
 typedef struct paella_ring paella_ring;
 
+/* Workgroups covered by one aggregated message (llis::job::FinishedBlockNotifier::noti_batch_size). */
+unsigned paella_ring_batch_size(void);
+
 /* A ring of `slots` 64-bit slots in coherent host memory plus `num_notifiers` device-resident notifiers. */
 int paella_ring_create(size_t slots, unsigned num_notifiers, paella_ring** out);
 int paella_ring_destroy(paella_ring* ring);

@@ -93,6 +93,7 @@ OPS_SYMBOLS = {
 }
 
 RING_SYMBOLS = {
+    "paella_ring_batch_size": (c_uint, []),
     "paella_ring_create": (c_int, [c_size_t, c_uint, ctypes.POINTER(c_void_p)]),
     "paella_ring_destroy": (c_int, [c_void_p]),
     "paella_ring_notifier": (c_void_p, [c_void_p, c_uint]),

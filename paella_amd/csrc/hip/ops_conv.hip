@@ -23,6 +23,8 @@
 #include "paella_ops.h"
 #include <llis/job/finished_block_notifier.h>
 
+#include "out_store.h"
+
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -163,7 +165,7 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
             const size_t o = (size_t)m * p.PQ + pix;
             if (p.residual) v += p.residual[o];
             const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
-            p.y[o] = apply_act(v, p.act, sl, p.lo, p.hi);
+            store_out(p.y + o, apply_act(v, p.act, sl, p.lo, p.hi));
         }
     };
 
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         }
     }
 
-    if (p.notifier) p.notifier->end(p.job_id);
+    if (p.notifier) p.notifier->end_written_through(p.job_id);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -238,9 +240,9 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
         const size_t o = (size_t)c * PQ + pix;
         if (p.residual) acc += p.residual[o];
         const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
-        p.y[o] = apply_act(acc, p.act, sl, p.lo, p.hi);
+        store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
     }
-    if (p.notifier) p.notifier->end(p.job_id);
+    if (p.notifier) p.notifier->end_written_through(p.job_id);
 }
 
 typedef void (*ConvKernel)(ConvArgs);

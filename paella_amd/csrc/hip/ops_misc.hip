@@ -10,6 +10,8 @@
 #include "paella_ops.h"
 #include <llis/job/finished_block_notifier.h>
 
+#include "out_store.h"
+
 namespace {
 
 using Notifier = llis::job::FinishedBlockNotifier;
@@ -58,9 +60,9 @@ __global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x,
             for (int i = lane; i < I; i += 64) acc += wr[i] * x[i];
         }
         acc = wave_sum(acc);
-        if (lane == 0) y[o] = act_apply(acc + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f);
+        if (lane == 0) store_out(y + o, act_apply(acc + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f));
     }
-    if (notifier) notifier->end(job_id);
+    if (notifier) notifier->end_written_through(job_id);
 }
 
 // ------------------------------------------------------------------------------------------ pooling
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
                 const int he = min(h0 + p.R, p.H + p.ph), we = min(w0 + p.S, p.W + p.pw);
                 div = (he - h0) * (we - w0);
             }
-            p.y[idx] = div ? acc / (float)div : 0.f;
+            store_out(p.y + idx, div ? acc / (float)div : 0.f);
         } else {
             float m = -FLT_MAX;
             for (int r = 0; r < p.R; ++r) {
@@ -115,10 +117,10 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
                     m = fmaxf(m, xc[(size_t)h * p.W + w]);
                 }
             }
-            p.y[idx] = m;
+            store_out(p.y + idx, m);
         }
     }
-    if (p.notifier) p.notifier->end(p.job_id);
+    if (p.notifier) p.notifier->end_written_through(p.job_id);
 }
 
 // One wave per channel.
@@ -132,9 +134,9 @@ __global__ __launch_bounds__(256) void gap_kernel(const float* __restrict__ x, f
         float acc = 0.f;
         for (int i = lane; i < HW; i += 64) acc += xc[i];
         acc = wave_sum(acc);
-        if (lane == 0) y[c] = acc / (float)HW;
+        if (lane == 0) store_out(y + c, acc / (float)HW);
     }
-    if (notifier) notifier->end(job_id);
+    if (notifier) notifier->end_written_through(job_id);
 }
 
 // ------------------------------------------------------------------------------------------ elementwise
@@ -176,13 +178,13 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs p) {
             r.y = elt_one(p, a.y, b.y, c);
             r.z = elt_one(p, a.z, b.z, c);
             r.w = elt_one(p, a.w, b.w, c);
-            reinterpret_cast<float4*>(p.y)[i4] = r;
+            store_out4(p.y + i4 * 4, r);
         }
     } else {
         const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-        if (i < n) p.y[i] = elt_one(p, p.a[i], p.b ? p.b[i] : 0.f, (int)(i / p.HW));
+        if (i < n) store_out(p.y + i, elt_one(p, p.a[i], p.b ? p.b[i] : 0.f, (int)(i / p.HW)));
     }
-    if (p.notifier) p.notifier->end(p.job_id);
+    if (p.notifier) p.notifier->end_written_through(p.job_id);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n,
@@ -190,11 +192,11 @@ __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ x, 
     if (notifier) notifier->start(job_id);
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i + 3 < n && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
-        *reinterpret_cast<float4*>(y + i) = *reinterpret_cast<const float4*>(x + i);
+        store_out4(y + i, *reinterpret_cast<const float4*>(x + i));
     } else {
-        for (size_t k = i; k < n && k < i + 4; ++k) y[k] = x[k];
+        for (size_t k = i; k < n && k < i + 4; ++k) store_out(y + k, x[k]);
     }
-    if (notifier) notifier->end(job_id);
+    if (notifier) notifier->end_written_through(job_id);
 }
 
 // ------------------------------------------------------------------------------------------ softmax / LRN
@@ -219,8 +221,8 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ 
     if (lane == 0) part[wave] = s;
     __syncthreads();
     s = (part[0] + part[1]) + (part[2] + part[3]);
-    for (int i = threadIdx.x; i < cols; i += 256) yr[i] = expf(xr[i] - m) / s;
-    if (notifier) notifier->end(job_id);
+    for (int i = threadIdx.x; i < cols; i += 256) store_out(yr + i, expf(xr[i] - m) / s);
+    if (notifier) notifier->end_written_through(job_id);
 }
 
 __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW, int size,
@@ -236,9 +238,9 @@ __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, f
             const float v = x[(size_t)cc * HW + i];
             sq += v * v;
         }
-        y[idx] = x[idx] / powf(k + alpha / (float)size * sq, beta);
+        store_out(y + idx, x[idx] / powf(k + alpha / (float)size * sq, beta));
     }
-    if (notifier) notifier->end(job_id);
+    if (notifier) notifier->end_written_through(job_id);
 }
 
 inline unsigned blocks_for(size_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }

@@ -73,6 +73,8 @@ double now_us() {
 
 extern "C" {
 
+unsigned paella_ring_batch_size(void) { return FinishedBlockNotifier::noti_batch_size; }
+
 int paella_ring_create(size_t slots, unsigned num_notifiers, paella_ring** out) {
     if (!out || slots == 0) return -1;
     try {

@@ -6,11 +6,12 @@
 // callback, copy).  An operation executes when the test says so (fake_hip_step*) or, with
 // FAKE_HIP_AUTORUN=1, on a background thread that always runs the oldest issued operation that is at the
 // head of its stream.  Executing a kernel means posting exactly the messages the aggregated workgroup hooks
-// post: ceil(n/16) start messages then ceil(n/16) end messages (full batches of 16 first, remainder last).
+// post: ceil(n/B) start messages then ceil(n/B) end messages (full batches of B = noti_batch_size first, remainder last).
 
 #include "paella_hip.h"
 
 #include <llis/job/context.h>
+#include <llis/job/finished_block_notifier.h>
 #include <llis/job/instrument_info.h>
 
 #include <unistd.h>
@@ -62,8 +63,9 @@ void post(uint8_t is_start, unsigned num, uint32_t job_id) {
 }
 
 void post_batches(uint8_t is_start, unsigned n, uint32_t job_id) {
-    for (unsigned i = 0; i < n / 16; ++i) post(is_start, 16, job_id);
-    if (n % 16) post(is_start, n % 16, job_id);
+    constexpr unsigned B = llis::job::FinishedBlockNotifier::noti_batch_size;
+    for (unsigned i = 0; i < n / B; ++i) post(is_start, B, job_id);
+    if (n % B) post(is_start, n % B, job_id);
 }
 
 // Advances the head operation of `s` by one phase (full = run it to completion).  Caller holds g_mtx,

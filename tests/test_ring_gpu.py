@@ -1,8 +1,8 @@
 """The GPU->host notification ring and the workgroup hooks on a real device.
 
 Closed forms being checked (they follow from the notifier's counter arithmetic): a grid of n workgroups
-produces exactly ceil(n/16) start and ceil(n/16) end messages for its job id, whose `num` fields are 16
-except for one remainder message n mod 16, summing to n; the un-aggregated hooks produce n + n messages of
+produces exactly ceil(n/B) start and ceil(n/B) end messages for its job id (B = the library's batch size), whose
+`num` fields are B except for one remainder message n mod B, summing to n; the un-aggregated hooks produce n + n messages of
 num 1.  Message bit layout: byte0 is_start, byte1 cu id, byte2 num, byte3 ready, bytes4-7 job id.
 """
 import ctypes
@@ -35,15 +35,21 @@ def ring(cuda):
     lib.paella_ring_destroy(handle)
 
 
+def batch():
+    from paella_amd import _abi
+    return _abi.ops().paella_ring_batch_size()
+
+
 def expected_nums(n):
-    return sorted([16] * (n // 16) + ([n % 16] if n % 16 else []))
+    b = batch()
+    return sorted([b] * (n // b) + ([n % b] if n % b else []))
 
 
 @pytest.mark.parametrize("grid", [(1, 1, 1), (5, 1, 1), (16, 1, 1), (17, 1, 1), (200, 1, 1), (7, 5, 3), (1000, 1, 1)])
 def test_aggregated_notifier_message_count_and_layout(ring, grid):
     lib, h = ring
     n = grid[0] * grid[1] * grid[2]
-    want = 2 * ((n + 15) // 16)
+    want = 2 * ((n + batch() - 1) // batch())
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     for rep in range(3):  # the counters must self-reset between kernels
         job_id = 1000 + rep
@@ -66,7 +72,7 @@ def test_aggregated_notifier_message_count_and_layout(ring, grid):
                 started += k
             else:
                 finished += k
-            assert finished <= started + 15
+            assert finished <= started + batch() - 1
 
 
 def test_raw_hooks_one_message_pair_per_workgroup(ring):
@@ -109,7 +115,7 @@ def test_ops_kernels_carry_the_hooks(ring, cuda):
     y0 = conv(x)
     y1 = conv(x, job_id=9, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, 1)))
     n = conv.plan.dims.grid
-    want = 2 * ((n + 15) // 16)
+    want = 2 * ((n + batch() - 1) // batch())
     out = np.zeros(want, np.uint64)
     assert lib.paella_ring_drain(h, out.ctypes.data, want, 20.0) == want
     m = decode(out)
