@@ -225,7 +225,10 @@ class ShmChannelWriter : public ShmChannelBase<for_gpu> {
     // producers that share THIS endpoint object's positions or re-read them (see refresh in acquire).
     LLIS_HOSTDEV void acquire_writer_lock() {
         this->lock_->acquire();
-        this->my_write_ = this->load_pos(this->write_pos_);  // another producer may have advanced it
+        // Another producer may have advanced the ring by any amount since this endpoint last wrote: both cached
+        // positions are stale (a read position more than a lap old would overstate the free space).
+        this->my_write_ = this->load_pos(this->write_pos_);
+        this->my_read_ = this->load_pos(this->read_pos_);
     }
     LLIS_HOSTDEV void release_writer_lock() { this->lock_->release(); }
 };

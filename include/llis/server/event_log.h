@@ -11,7 +11,7 @@
 //   S <job_id>                                             client woken (pre-notify)
 //   E <job_id>                                             completion posted to the client
 // The reference has no such log; it exists so that "scheduling and notification order" can be compared
-// exactly against the scheduler oracle on fake and real devices.
+// exactly against an independent replay of the policy, on scripted and on real devices.
 
 #include <cstdint>
 #include <cstdio>

@@ -1,0 +1,111 @@
+"""The C-ABI libraries load without a GPU and export every function their headers declare; the pure-host
+parts of the operator ABI (planning, weight packing, output-extent arithmetic) do what the headers say."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+HEADERS = {"paella_hip.h": "llis_hip", "paella_ops.h": "paella_ops", "paella_ring.h": "paella_ops", "paella_models.h": "paella_ops",
+           "paella_serve.h": "paella_serve"}
+
+
+def declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:llis_hip|paella)_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.mark.parametrize("header", sorted(HEADERS))
+def test_every_declared_symbol_is_exported(header):
+    from paella_amd import _abi
+    _abi.hip()
+    lib = ctypes.CDLL(os.path.join(_abi.LIB_DIR, "lib%s.so" % HEADERS[header]), mode=ctypes.RTLD_GLOBAL)
+    names = declared(header)
+    assert len(names) >= 5
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_python_tables_cover_the_headers():
+    from paella_amd import _abi, _abi_models, serve
+    tables = {"paella_hip.h": _abi.HIP_SYMBOLS, "paella_ops.h": _abi.OPS_SYMBOLS, "paella_ring.h": _abi.RING_SYMBOLS,
+              "paella_models.h": _abi_models.MODEL_SYMBOLS, "paella_serve.h": serve.SERVE_SYMBOLS}
+    for header, table in tables.items():
+        assert sorted(table) == declared(header), header
+
+
+def plan(desc_args, has_res=0, hint=0):
+    from paella_amd import _abi
+    lib = _abi.ops()
+    d = _abi.ConvDesc(*desc_args)
+    p = _abi.ConvPlan()
+    rc = lib.paella_conv2d_plan(ctypes.byref(d), has_res, hint, ctypes.byref(p))
+    return rc, p
+
+
+def test_conv_plan_arithmetic_and_rejections():
+    rc, p = plan((64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0))
+    assert rc == 0 and (p.P, p.Q) == (56, 56) and p.flops == 2.0 * 64 * 64 * 9 * 56 * 56
+    assert p.bytes == 4.0 * (64 * 56 * 56 + 64 * 64 * 9 + 64 + 64 * 56 * 56)
+    tiles = -(-64 // (32 * p.mi)) * -(-(56 * 56) // (32 * p.ni))
+    assert p.dims.grid == tiles and p.dims.block == 64 * p.kw and p.k_pad == 576 and p.m_pad % (32 * p.mi) == 0
+    assert plan((64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0), has_res=1)[1].bytes == p.bytes + 4.0 * 64 * 56 * 56
+    rc, p = plan((32, 112, 112, 32, 3, 3, 2, 2, 1, 1, 1, 1, 32, 2, 0, 0))      # depthwise
+    assert rc == 0 and p.kind == 1 and (p.P, p.Q) == (56, 56) and p.blob_bytes == 32 * 9 * 4
+    assert plan((8, 8, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 4, 0, 0, 0))[0] == -2      # grouped but not depthwise
+    assert plan((8, 8, 8, 8, 3, 3, 0, 1, 1, 1, 1, 1, 1, 0, 0, 0))[0] == -1      # stride 0
+    assert plan((8, 2, 2, 8, 5, 5, 1, 1, 0, 0, 1, 1, 1, 0, 0, 0))[0] == -1      # empty output
+    assert plan((8, 8, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1, 9, 0, 0))[0] == -1      # unknown activation
+    assert plan((8, 8, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0), hint=(3 << 8) | (1 << 4))[0] == -1  # no such tile
+
+
+def test_weight_packing_layout():
+    """Blob = table of (k_pad + 16) {byte offset, (r*dil)<<16 | s*dil} pairs, then weights as [k/4][m_pad][4]."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+    c, h, w, k, r, s = 5, 9, 7, 6, 3, 2
+    rc, p = plan((c, h, w, k, r, s, 1, 1, 1, 0, 2, 1, 1, 0, 0, 0))
+    assert rc == 0
+    wt = np.arange(k * c * r * s, dtype=np.float32).reshape(k, c, r, s)
+    blob = np.zeros(p.blob_bytes, np.uint8)
+    assert lib.paella_conv2d_pack(ctypes.byref(p), wt.ctypes.data, blob.ctypes.data) == 0
+    kdim = c * r * s
+    table = blob[:(p.k_pad + 16) * 8].view(np.int32).reshape(-1, 2)
+    for kk in range(kdim):
+        cc, rr, ss = kk // (r * s), (kk // s) % r, kk % s
+        assert table[kk, 0] == 4 * (cc * h * w + rr * 2 * w + ss) and table[kk, 1] == ((rr * 2) << 16 | ss)
+    assert np.all(table[kdim:, 1] == 0x7FFF0000)
+    packed = blob[(p.k_pad + 16) * 8:].view(np.float32).reshape(p.k_pad // 4, p.m_pad, 4)
+    flat = wt.reshape(k, kdim)
+    for m in range(k):
+        for kk in range(kdim):
+            assert packed[kk // 4, m, kk % 4] == flat[m, kk]
+    assert packed[:, k:, :].sum() == 0 and packed.reshape(-1).sum() == flat.sum()
+
+
+def test_pool_out_matches_oracle():
+    from oracle import ops as orc
+    from paella_amd import _abi
+    lib = _abi.ops()
+    for n in range(3, 40):
+        for k, s, p in [(2, 2, 0), (3, 2, 1), (3, 2, 0), (3, 1, 1), (3, 3, 0)]:
+            for ceil in (0, 1):
+                assert lib.paella_pool_out(n, k, s, p, ceil) == orc.pool_out(n, k, s, p, bool(ceil))
+
+
+def test_product_has_no_cpu_compute_path():
+    """Nothing under paella_amd/ or include/ may reference the oracle."""
+    offenders = []
+    for base in ("paella_amd", "include"):
+        for dirpath, _, files in os.walk(os.path.join(ROOT, base)):
+            if "/build" in dirpath or dirpath.endswith("/lib") or dirpath.endswith("/bin"):
+                continue
+            for f in files:
+                if f.endswith((".py", ".h", ".cpp", ".hip")):
+                    if re.search(r"\boracle\b", open(os.path.join(dirpath, f), errors="ignore").read()):
+                        offenders.append(os.path.join(dirpath, f))
+    assert not offenders, offenders

@@ -1,0 +1,97 @@
+"""The real Server + schedulers + rings (C++), driven message by message on the scripted device, against the
+scheduler oracle: every decision (job ids, dispatch order, stream and notifier handed out, wake-ups,
+completions) must be reproduced bit for bit from the inputs recorded in the same log."""
+import pytest
+
+from _fake import fake_job, run_harness
+from oracle import sched
+
+TYPES = ["fake_mem3", "fake_short", "fake_long", "fake_big"]
+
+
+def scenario(policy, streams, body, extra="", types=TYPES):
+    script = "sched %s streams %d %s\nclient\n" % (policy, streams, extra)
+    for t in types:
+        script += "job %s\n" % fake_job(t)
+    return script + body
+
+
+def check(policy, streams, body, extra="", types=TYPES, **kw):
+    replies, log = run_harness(scenario(policy, streams, body, extra, types))
+    events = sched.parse_log(log)
+    assert any(e[0] == "E" for e in events)
+    expected, actual = sched.replay(policy, [sched.FAKE_TYPES[t] for t in types], streams, events, **kw)
+    assert expected == actual, next((i, a, b) for i, (a, b) in enumerate(zip(expected + [None], actual + [None])) if a != b)
+    return replies, events
+
+
+MIXED = "launch 1 0\nlaunch 0 0\nlaunch 1 1\nstep 2\nlaunch 2 0\nlaunch 0 1\nstep 5\nlaunch 1 2\ndrain\n"
+
+
+@pytest.mark.parametrize("policy", ["fifo", "fifo2", "full3"])
+@pytest.mark.parametrize("streams", [1, 2, 8])
+def test_policy_matches_oracle_on_a_mixed_scenario(policy, streams):
+    replies, events = check(policy, streams, MIXED)
+    done = [r for r in replies if r.startswith("done")]
+    assert len(done) == 6
+    summary = [r for r in replies if r.startswith("wakeups")][0].split()
+    assert summary[1] == "6" and summary[3] == "6" and summary[5] == "0"  # every request woke the client once
+
+
+@pytest.mark.parametrize("mem", ["marker", "hostfunc"])
+def test_both_copy_completion_paths(mem):
+    check("full3", 2, "launch 0 0\nlaunch 0 1\ndrain\n", extra="mem " + mem)
+    check("fifo", 2, "launch 0 0\nlaunch 0 1\ndrain\n", extra="mem " + mem)
+
+
+def test_request_bytes_travel_through_the_pool_slots():
+    """fake_mem3 returns input + 1: checks the (chunk, offset) addressing of the shared-memory pool."""
+    replies, _ = run_harness(scenario("full3", 4, "put 0 0 7\nput 0 3 41\nlaunch 0 0\nlaunch 0 3\ndrain\nget 0 0\nget 0 3\n"))
+    outs = [r for r in replies if r.startswith("out")]
+    assert outs == ["out 8 8 8 8 8 8 8 8", "out 42 42 42 42 42 42 42 42"]
+    assert sorted(r for r in replies if r.startswith("done")) == ["done 1000", "done 1003"]
+
+
+def test_oversubscription_credit_path():
+    """fake_big (3000 x 256 x 64 regs) never fits a small budget: it is admitted as an 'unfit' kernel while
+    credits last, the credit returns when its start messages are complete (or at its end), and the
+    head-of-queue job blocks everything behind it once credits are gone."""
+    budget = (2_000_000, 1 << 20, 100_000, 400)
+    body = "launch 3 0\nlaunch 3 1\nlaunch 1 0\nlaunch 3 2\nstart 7\nstart 6\nfinish 7\ndrain\n"
+    replies, events = check("full3", 8, body, extra="extra 1 budget %d %d %d %d" % budget, budget=budget, extra_kernels=1)
+    dispatches = [e for e in events if e[0] == "D"]
+    assert dispatches[0][6] == 1, "first big kernel must go out as unfit"
+    # with one credit the second big job cannot start until the first is fully resident
+    first_start_done = next(i for i, e in enumerate(events) if e[0] == "B" and e[2] == 1)
+    assert all(e[1] == 0 for e in events[:first_start_done] if e[0] == "D")
+
+
+def test_fairness_threshold_changes_the_order():
+    body = "".join("launch 1 %d\n" % i for i in range(4)) + "launch 2 0\n" + "drain\n"
+    _, fair = check("full3", 1, body, extra="unfair 1", unfair=1.0)
+    _, unfair = check("full3", 1, body, extra="unfair 1000000", unfair=1e6)
+    order = lambda evs: [e[1:3] for e in evs if e[0] == "D"]
+    assert order(fair) != order(unfair)
+
+
+def test_job_ids_are_reused_most_recent_first():
+    _, events = check("fifo2", 4, "launch 1 0\nlaunch 1 1\nlaunch 1 2\ndrain\nlaunch 1 0\nlaunch 1 1\ndrain\n")
+    js = [e for e in events if e[0] == "J"]
+    assert [j[1] for j in js[:3]] == [0, 1, 2]
+    ends = [e[1] for e in events if e[0] == "E"][:3]
+    assert [j[1] for j in js[3:]] == [ends[-1], ends[-2]]  # LIFO free list
+    assert [j[3] for j in js] == list(range(5))            # unique ids count arrivals
+
+
+def test_dummy_shape_closed_form_through_the_real_server():
+    """One fake_short alone under full3: per stage exactly D, B start 5, B end 5; wake-up at the last dispatch."""
+    _, events = check("full3", 3, "launch 1 0\ndrain\n")
+    core = [e for e in events if e[0] != "L"]
+    expect = [("J", 0, 1, 0, 0)]
+    for s in range(10):
+        expect.append(("D", 0, s, 2, 2, 0, 0))
+        if s == 9:
+            expect.append(("S", 0))
+        expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
+    expect.append(("E", 0))
+    assert core == expect

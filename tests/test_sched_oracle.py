@@ -1,0 +1,188 @@
+"""Pins the scheduler oracle (oracle/sched.py) with hand-derived logs, closed forms and brute force, so that
+replaying a product log through it means something."""
+import itertools
+import random
+
+from oracle import sched
+from oracle.sched import Stage
+
+
+def kernel(blocks, pre=False, threads=256, regs=32, smem=0):
+    return Stage(False, blocks, threads, smem, regs, pre)
+
+
+def test_dummy_job_closed_form_full3():
+    """dummy_short alone: 10 stages, each dispatched on the same (LIFO) stream and notifier, one start and one
+    end message of num=5 per stage, client woken at the dispatch of the last stage, then the completion."""
+    s = sched.Full3([sched.dummy_stages(10)], num_streams=4)
+    s.new_job(0)
+    expect = [("J", 0, 0, 0, 0)]
+    for stage in range(10):
+        expect.append(("D", 0, stage, 3, 3, 0, 0))
+        if stage == 9:
+            expect.append(("S", 0))
+        s.block(0, True, 5)
+        s.block(0, False, 5, lambda: 100.0)
+    expect.append(("E", 0))
+    assert s.out == expect
+    # the id returns to the pool and is reused first
+    s.new_job(0)
+    assert s.out[-1] == ("D", 0, 0, 3, 3, 0, 0) and s.out[-2] == ("J", 0, 0, 1, 0)
+
+
+def test_fifo_hand_derived_two_jobs_one_stream():
+    """Job-by-job on one stream: A (mem, kernel 3 blocks, mem+pre-notify) is issued whole; B waits for the
+    stream.  A's wake-up fires when everything up to and including its pre-notify stage finished = its end."""
+    a = [Stage(True), kernel(3), Stage(True, pre_notify=True)]
+    b = [kernel(2, pre=True)]
+    s = sched.Fifo([a, b], num_streams=1)
+    s.new_job(0)
+    s.new_job(1)
+    assert s.out == [("J", 0, 0, 0, 1), ("D", 0, 0, 0, 0, 1, 0), ("D", 0, 1, 0, 0, 0, 0), ("D", 0, 2, 0, 0, 1, 0), ("J", 1, 1, 1, 0)]
+    s.mem(0)
+    s.block(0, True, 3)
+    s.block(0, False, 3)
+    assert s.out[5:] == []
+    s.mem(0)
+    assert s.out[5:] == [("S", 0), ("E", 0), ("D", 1, 0, 0, 0, 0, 0)]
+    s.block(1, False, 2)
+    assert s.out[8:] == [("S", 1), ("E", 1)]
+
+
+def test_fifo2_arrival_order_and_lifo_pools():
+    """Kernel-by-kernel FIFO: with two streams, two 2-stage jobs alternate; a finished stage's stream goes back
+    on top of the pool and is handed to whichever job arrived first among those waiting."""
+    t = [kernel(1), kernel(1, pre=True)]
+    s = sched.Fifo2([t], num_streams=2)
+    s.new_job(0)
+    s.new_job(0)
+    s.new_job(0)  # no stream left: queued
+    assert [e for e in s.out if e[0] == "D"] == [("D", 0, 0, 1, 1, 0, 0), ("D", 1, 0, 0, 0, 0, 0)]
+    s.block(1, False, 1)  # job 1's stage ends first; job 2 (unique 2) waits, job 1 (unique 1) re-queues: 1 goes first
+    assert s.out[-2:] == [("D", 1, 1, 0, 0, 0, 0), ("S", 1)]
+    s.block(0, False, 1)
+    assert s.out[-2:] == [("D", 0, 1, 1, 1, 0, 0), ("S", 0)]
+    s.block(0, False, 1)
+    assert s.out[-2:] == [("E", 0), ("D", 2, 0, 1, 1, 0, 0)]
+
+
+def test_sm_resources_closed_form():
+    r = sched.SmResources(1000, 100, 64, 4)
+    st = kernel(2, threads=8, regs=10, smem=20)
+    assert r.fits(st)
+    r.acquire(st, 2)
+    assert r.free == [1000 - 160, 60, 48, 2]
+    assert not r.fits(kernel(3, threads=8, regs=10))      # workgroup slots
+    assert not r.fits(kernel(1, threads=8, regs=10, smem=61))
+    r.release(st, 1)
+    assert r.free == [920, 80, 56, 3]
+
+
+def test_stage_length_estimator_recurrence():
+    t = sched.TypeStats()
+    for v in (8.0, 4.0, 10.0):
+        t.update_length(0, v)
+    assert t.lengths == [((8.0 + 4.0) / 2 + 10.0) / 2]
+    t.update_length(1, 3.0)
+    t.set_resource(0, 1.0)
+    t.set_resource(1, 1.0)
+    t.set_resource(1, 5.0)  # resources never change once set
+    assert t.remaining_rl(0) == 8.0 + 3.0 and t.remaining_rl(1) == 3.0 and t.remaining_rl(2) == 0.0
+
+
+def test_srpt_prefers_the_job_with_less_remaining_work():
+    """Two types with learned stage lengths; with one stream the queued job with less remaining work goes first."""
+    short = [kernel(1), kernel(1, pre=True)]
+    long_ = [kernel(1)] * 5 + [kernel(1, pre=True)]
+    s = sched.Full3([short, long_], num_streams=1)
+    # teach the estimator: run one job of each type alone
+    for type_id, n in ((0, 2), (1, 6)):
+        s.new_job(type_id)
+        for _ in range(n):
+            s.block(0, True, 1)
+            s.block(0, False, 1, lambda: 10.0)
+    s.out.clear()
+    s.new_job(1)   # long: takes the stream
+    s.new_job(1)   # another long queued, remaining 60
+    s.new_job(0)   # short queued, remaining 20 -> higher priority (-20 > -60)
+    s.block(0, True, 1)
+    s.block(0, False, 1, lambda: 10.0)
+    # candidates now: job 0 (long, 50 left), job 1 (long, 60), job 2 (short, 20)
+    d = [e for e in s.out if e[0] == "D"]
+    assert d[0][1] == 0 and d[1][1] == 2
+
+
+class NaiveQueue:
+    """Independent model of the fairness rule, written from the policy's description: every pop credits each
+    active type 1/n and charges the served type 1; a type joins (or re-joins after running dry) at the baseline."""
+
+    def __init__(self, threshold):
+        self.credit = 0.0          # total credit handed out per type so far
+        self.th0 = threshold
+        self.items = []            # (priority, order, type)
+        self.join = {}             # type -> (credit at join, charges since, order)
+        self.order = 0
+
+    def push(self, pri, typ):
+        if typ not in self.join:
+            self.join[typ] = [self.credit, 0, self.order]
+            self.order += 1
+        self.items.append((pri, self.order, typ))
+        self.order += 1
+
+    def pop(self):
+        # deficit of a type = credits since it joined - charges; fairness when the largest reaches the threshold
+        def deficit(t):
+            return (self.credit - self.join[t][0]) - self.join[t][1]
+        best_t = min(self.join, key=lambda t: (-deficit(t), self.join[t][2]))
+        pool = [i for i in self.items if i[2] == best_t] if deficit(best_t) >= self.th0 else self.items
+        item = min(pool, key=lambda i: (-i[0], i[1]))
+        self.items.remove(item)
+        self.credit += 1.0 / len(self.join)
+        t = item[2]
+        if any(i[2] == t for i in self.items):
+            self.join[t][1] += 1
+            self.join[t][2] = self.order
+            self.order += 1
+        else:
+            del self.join[t]
+        return item
+
+
+def test_jobqueue_against_naive_model_on_small_cases():
+    """Random short push/pop programs with 2 types, so that every fair share (1 or 1/2), priority and threshold
+    is exact in binary and the two formulations cannot differ by rounding."""
+    rng = random.Random(5)
+    for trial in range(2000):
+        th = rng.choice([0.5, 1.0, 2.0, 1e6])
+        q, naive = sched.JobQueue(th), NaiveQueue(th)
+        live = 0
+        for step in range(14):
+            if live == 0 or (live < 6 and rng.random() < 0.6):
+                pri, typ = -float(rng.randrange(0, 4)), rng.randrange(0, 2)
+                job = sched.Job(typ, [])
+                job.priority = pri
+                job.tag = (pri, typ)
+                q.push(job)
+                naive.push(pri, typ)
+                live += 1
+            else:
+                got = q.pop()
+                want = naive.pop()
+                assert got.tag == (want[0], want[2]), (trial, step, th)
+                live -= 1
+
+
+def test_jobqueue_fairness_triggers_and_is_fifo_among_equals():
+    q = sched.JobQueue(1.0)
+    jobs = []
+    for i, (pri, typ) in enumerate([(-1.0, 0), (-1.0, 0), (-1.0, 0), (-5.0, 1)]):
+        j = sched.Job(typ, [])
+        j.priority = pri
+        j.tag = i
+        q.push(j)
+        jobs.append(j)
+    # first pops follow priority with FIFO ties; type 1's deficit grows by 1/2 per pop: 0 -> .5 -> 1.0 >= threshold(1 - .5 - .5 = 0)...
+    order = [q.pop().tag for _ in range(4)]
+    assert order[0] == 0
+    assert 3 in order[:3], "the starved type must be served before type 0 is exhausted"

@@ -1,0 +1,103 @@
+"""The shipped binaries (llis_server, llis_app_client, llis_app_single_latency) and the in-process serve ABI,
+end to end over the real shared-memory rings and sockets, with the scripted device standing in for the GPU."""
+import ctypes
+import json
+import os
+import subprocess
+import time
+
+import pytest
+
+from _fake import BIN, FAKE_LIB, ensure_built, fake_env, fake_job
+
+
+@pytest.fixture(scope="module", autouse=True)
+def built():
+    ensure_built()
+
+
+def start_server(name, sched, streams=64, **env):
+    p = subprocess.Popen([os.path.join(BIN, "llis_server"), "--name", name, "--sched", sched, "--num_streams", str(streams)],
+                         env=fake_env(**env), stderr=subprocess.PIPE, text=True)
+    for _ in range(200):
+        if os.path.exists("/dev/shm/llis:channel:c2s:" + name):
+            return p
+        time.sleep(0.01)
+    p.kill()
+    raise AssertionError("server did not come up: " + p.stderr.read())
+
+
+@pytest.mark.parametrize("sched", ["fifo", "fifo2", "full3"])
+def test_load_generator_against_server_process(tmp_path, sched):
+    name = "pt%d%s" % (os.getpid(), sched)
+    srv = start_server(name, sched, FAKE_HIP_OP_US="20")
+    prefix = str(tmp_path / "run")
+    out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "300", "--dist", "exp", "--concurrency", "48",
+                          "--num_jobs", "600", "--start_record_num", "100", "--seed", "1", "--prefix", prefix, "--no_pin",
+                          fake_job("fake_short"), "0.7", "30", fake_job("fake_mem3"), "0.3", "30"],
+                         env=fake_env(), capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    stats = json.loads(out.stdout.strip().splitlines()[-1])
+    assert stats["num_jobs"] == 600 and stats["throughput_rps"] > 100
+    assert sum(stats["per_type_count"]) == 500  # 100 unrecorded
+    assert srv.wait(timeout=30) == 0           # EXIT_CMD ends the server cleanly
+    # stats row: x,num_jobs,elapsed then 7 numbers overall and per type (reference app/client.cpp:479-495)
+    row = open(prefix + ".txt").read().strip().split(",")
+    assert row[0] == "300" and row[1] == "600" and len(row) == 3 + 7 * 3
+    assert len(open(prefix + "_raw.txt").read().split()) == 500
+    assert not [f for f in os.listdir("/dev/shm") if name in f and "channel" in f]
+
+
+def test_arrival_process_is_reproducible_for_a_seed():
+    """Same seed, same job mix => same sequence of job types (draw order: type first, then inter-arrival)."""
+    counts = []
+    for rep in range(2):
+        name = "ptseed%d_%d" % (os.getpid(), rep)
+        srv = start_server(name, "fifo2")
+        out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "100", "--dist", "ln", "--ln_sigma", "1.5",
+                              "--concurrency", "32", "--num_jobs", "400", "--seed", "7", "--prefix", "/tmp/ptseed", "--no_pin",
+                              fake_job("fake_short"), "0.25", "16", fake_job("fake_mem3"), "0.75", "16"],
+                             env=fake_env(), capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        counts.append(json.loads(out.stdout.strip().splitlines()[-1])["per_type_count"])
+        srv.wait(timeout=30)
+    assert counts[0] == counts[1] and abs(counts[0][0] - 100) < 40
+
+
+def test_unknown_scheduler_is_an_error_not_a_crash():
+    out = subprocess.run([os.path.join(BIN, "llis_server"), "--name", "x", "--sched", "nope"], env=fake_env(), capture_output=True, text=True, timeout=30)
+    assert out.returncode == 4 and "unknown scheduler" in out.stderr and "full3" in out.stderr
+
+
+def test_single_latency_client(tmp_path):
+    name = "ptsl%d" % os.getpid()
+    srv = start_server(name, "full3", 4)
+    out = subprocess.run([os.path.join(BIN, "llis_app_single_latency"), name, fake_job("fake_mem3"), "50", "--quiet"], env=fake_env(),
+                         capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    assert json.loads(out.stdout.strip().splitlines()[-1])["num_jobs"] == 50
+    assert srv.wait(timeout=30) == 0
+
+
+def test_in_process_serve_abi_on_the_scripted_device():
+    """paella_server_start / paella_client_run / paella_client_single in a child interpreter that loads the
+    scripted device first (same soname as the HIP layer)."""
+    code = r'''
+import ctypes, os, sys, json
+sys.path.insert(0, %r)
+os.environ["FAKE_HIP_AUTORUN"] = "1"
+ctypes.CDLL(%r, mode=ctypes.RTLD_GLOBAL)
+from paella_amd import serve, _abi
+_abi._cache["llis_hip"] = True
+import numpy as np
+with serve.Server("inproc%%d" %% os.getpid(), "full3", num_streams=8, event_log=True) as s:
+    r = serve.client_run(s.name, [(%r, 1.0, 6)], 0.0, 6, 200, warmup_jobs=30)
+    x = np.full(100, 5, np.uint8)
+    out, lat = serve.client_single(s.name, %r, x, 25, n=3)
+log = s.event_log()
+print(json.dumps({"rps": r["throughput_rps"], "count": r["all"]["count"], "out": out.view(np.uint8)[:4].tolist(), "log_lines": len(log.splitlines())}))
+''' % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.join(FAKE_LIB, "libllis_hip.so"), fake_job("fake_short"), fake_job("fake_mem3"))
+    out = subprocess.run(["python3", "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    res = json.loads(out.stdout.strip().splitlines()[-1])
+    assert res["count"] == 200 and res["out"] == [6, 6, 6, 6] and res["log_lines"] > 1000
