@@ -433,7 +433,11 @@ def replay(policy, types, num_streams, events, **kw):
     """Feeds the log's inputs (J/B/M with the L lengths) to the oracle and returns (expected, actual) decision
     lists including the ids chosen for J, for comparison with ==."""
     sched = POLICIES[policy](types, num_streams, **kw)
-    it = iter(range(len(events)))
+    # unique ids count arrivals per PROCESS (a function-local static in Job::set_id), so a server that is not the
+    # first in its process starts from a non-zero base: take it from the first admission in the log
+    first = next((e for e in events if e[0] == "J"), None)
+    if first is not None:
+        sched.next_unique = first[3]
     pos = {"i": 0}
 
     def next_length(job_id, stage):

@@ -4,11 +4,19 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "paella_hip.h"
 
 namespace {
+
+// HIP multiplexes streams onto a small number of hardware queues (4 by default) and kernels that share a
+// queue run one after another, which caps how many requests can overlap on the GPU.  The block-level
+// scheduler relies on real concurrency between streams, so unless the user chose a value the library asks
+// for 16 queues before the runtime initialises (measured: 4 -> 16 queues raises served requests/s by ~30 %;
+// 32 is slower again).
+__attribute__((constructor)) void request_hardware_queues() { setenv("GPU_MAX_HW_QUEUES", "16", /*overwrite=*/0); }
 
 __global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, size_t count) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

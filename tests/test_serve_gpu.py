@@ -1,0 +1,168 @@
+"""End to end on the GPU, through the real path: client library -> shared-memory rings -> server thread ->
+scheduler -> instrumented HIP kernels -> notification ring -> completion.  Everything runs inside this
+process (threads), because a process that has touched the GPU must not spawn the server binaries."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from oracle import models as om
+from oracle import sched
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+_counter = [0]
+
+
+def server_name(tag):
+    _counter[0] += 1
+    return "gt%d_%s_%d" % (os.getpid(), tag, _counter[0])
+
+
+def device_budget():
+    from paella_amd import _abi
+    caps = _abi.DeviceCaps()
+    _abi.check(_abi.hip().llis_hip_get_device_caps(ctypes.byref(caps)))
+    n = caps.num_cus
+    return (n * caps.vgprs_per_cu, n * caps.lds_bytes_per_cu, n * caps.max_threads_per_cu, n * caps.max_blocks_per_cu)
+
+
+def close(got, ref):
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    assert np.all(err <= ATOL + RTOL * np.abs(ref)), err.max()
+
+
+@pytest.mark.parametrize("sched_name", ["fifo", "fifo2", "full3"])
+@pytest.mark.parametrize("model,job", [("mnist", "tvm_mnist"), ("resnet18", "tvm_resnet18")])
+def test_request_output_through_the_server_matches_oracle(cuda, sched_name, model, job):
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    desc = models.describe(model)
+    x = om.make_input(desc, 21, "uniform" if model == "mnist" else "normal")
+    ref = om.run(desc, x, seed=1)
+    print("case", sched_name, model, flush=True)
+    with serve.Server(server_name(sched_name), sched_name, num_streams=8) as srv:
+        out, lat = serve.client_single(srv.name, serve.job_path(job), x, ref.size, n=5)
+    close(out, ref)
+
+
+@pytest.mark.parametrize("mem_marker", [True, False])
+def test_both_copy_completion_paths_on_the_gpu(cuda, mem_marker):
+    from paella_amd import serve
+    x = np.arange(32000, dtype=np.float32)
+    with serve.Server(server_name("mem"), "full3", num_streams=4, mem_marker=mem_marker) as srv:
+        out, lat = serve.client_single(srv.name, serve.job_path("vec_add_coroutine"), x, 32000, n=4)
+    np.testing.assert_array_equal(out, 10 * x)
+
+
+def test_plain_job_with_raw_hooks(cuda):
+    from paella_amd import serve
+    with serve.Server(server_name("hello"), "full3", num_streams=4, event_log=True) as srv:
+        serve.client_single(srv.name, serve.job_path("helloworld"), np.zeros(5, np.uint8), 0, n=3)
+    ev = sched.parse_log(srv.event_log())
+    # stage i launches i workgroups, each sending its own start and end message
+    starts = sum(e[3] for e in ev if e[0] == "B" and e[2] == 1)
+    ends = sum(e[3] for e in ev if e[0] == "B" and e[2] == 0)
+    assert starts == ends == 3 * (1 + 2 + 3 + 4 + 5)
+
+
+@pytest.mark.parametrize("sched_name", ["fifo", "fifo2", "full3"])
+def test_dummy_job_event_log_is_bit_exact_closed_form(cuda, sched_name):
+    """dummy_short alone, three requests back to back: per stage exactly one dispatch, one start message and
+    one end message with num=5; stream, notifier and job id come from LIFO pools; the wake-up is sent when the
+    last stage is dispatched (fifo: when the work up to the pre-notify stage has finished)."""
+    from paella_amd import serve
+    streams = 6
+    with serve.Server(server_name("dummy"), sched_name, num_streams=streams, event_log=True) as srv:
+        serve.client_single(srv.name, serve.job_path("dummy_short"), np.zeros(5, np.uint8), 0, n=3)
+    ev = [e for e in sched.parse_log(srv.event_log()) if e[0] != "L"]
+    top = streams - 1
+    expect = []
+    base = ev[0][3]  # arrival counter of this process when the server started
+    for req in range(3):
+        expect.append(("J", 0, 0, base + req, 0))
+        if sched_name == "fifo":
+            expect += [("D", 0, s, top, top, 0, 0) for s in range(10)]
+            for s in range(10):
+                expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
+            expect += [("S", 0), ("E", 0)]
+        else:
+            for s in range(10):
+                expect.append(("D", 0, s, top, top, 0, 0))
+                if s == 9:
+                    expect.append(("S", 0))
+                expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
+            expect.append(("E", 0))
+    assert ev == expect
+
+
+@pytest.mark.parametrize("sched_name", ["fifo", "fifo2", "full3"])
+def test_concurrent_dummy_jobs_replay_exactly(cuda, sched_name):
+    """Several dummy jobs of two types in flight: the order in which the GPU posts messages is not determined,
+    but given the observed inputs every decision of the server must equal the oracle's."""
+    from paella_amd import serve
+    streams = 8
+    with serve.Server(server_name("mix"), sched_name, num_streams=streams, event_log=True) as srv:
+        r = serve.client_run(srv.name, [(serve.job_path("dummy_10"), 0.6, 3), (serve.job_path("dummy_21"), 0.4, 2)], 3000.0, 5, 24, seed=3)
+    assert r["all"]["count"] == 24
+    events = sched.parse_log(srv.event_log())
+    types = [sched.dummy_stages(10), sched.dummy_stages(21)]
+    expected, actual = sched.replay(sched_name, types, streams, events, budget=device_budget())
+    assert expected == actual
+    assert sum(1 for e in actual if e[0] == "E") == 24 + 5  # plus one warm-up run per pooled instance
+
+
+def test_mixed_model_load_then_outputs_still_correct(cuda):
+    """Small CNN : ResNet-18 = 9 : 1 Poisson load under full3, then a checked request of each model on the same
+    server (the instances and their buffers were recycled by the load)."""
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    with serve.Server(server_name("mixed"), "full3", num_streams=32) as srv:
+        r = serve.client_run(srv.name, [(serve.job_path("tvm_mnist"), 0.9, 16), (serve.job_path("tvm_resnet18"), 0.1, 8)], 200.0, 24, 1500,
+                             warmup_jobs=100, seed=1)
+        assert r["all"]["count"] == 1500 and r["per_type"][0]["count"] > r["per_type"][1]["count"] > 50
+        for model, job in [("mnist", "tvm_mnist"), ("resnet18", "tvm_resnet18")]:
+            desc = models.describe(model)
+            x = om.make_input(desc, 33, "uniform" if model == "mnist" else "normal")
+            out, _ = serve.client_single(srv.name, serve.job_path(job), x, models.io_bytes(model)[1] // 4, n=2)
+            close(out, om.run(desc, x, seed=1))
+
+
+def test_stream_order_independence_of_results(cuda):
+    """Stages of one request issued on different streams, each only after the previous stage's end message was
+    read from the ring, give the same bits as the single-stream forward: the end hook's ordering is sufficient."""
+    from paella_amd import _abi, models
+    lib, hip = _abi.ops(), _abi.hip()
+    name = "resnet18"
+    desc = models.describe(name)
+    x = om.make_input(desc, 5)
+    ex = models.Exec(name, seed=1)
+    ring = ctypes.c_void_p()
+    _abi.check(lib.paella_ring_create(65536, 4, ctypes.byref(ring)))
+    streams = []
+    for _ in range(4):
+        s = ctypes.c_void_p()
+        _abi.check(hip.llis_hip_stream_create(ctypes.byref(s)))
+        streams.append(s)
+    try:
+        ex.set_input(x)
+        ex.forward()
+        ref = ex.get_output()
+        b = lib.paella_ring_batch_size()
+        for rep in range(20):
+            ex.set_input(x)
+            for i in range(ex.num_stages):
+                grid = ex.stage_dims(i).grid
+                ex.launch_stage(i, streams[(i + rep) % 4], job_id=i, notifier=ctypes.c_void_p(lib.paella_ring_notifier(ring, (i + rep) % 4)))
+                want = 2 * ((grid + b - 1) // b)
+                assert lib.paella_ring_drain(ring, None, want, 20.0) == want
+            # the last end message has been read: the output must be complete without any stream synchronisation
+            np.testing.assert_array_equal(ex.get_output(), ref)
+    finally:
+        for s in streams:
+            hip.llis_hip_stream_synchronize(s)
+            hip.llis_hip_stream_destroy(s)
+        lib.paella_ring_destroy(ring)
+        ex.close()
