@@ -33,9 +33,9 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True):
+def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2):
     name = "bench%d_%s_%d" % (os.getpid(), sched, int(time.time() * 1000) % 100000)
-    with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4) as srv:
+    with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4, extra_kernels=extra_kernels) as srv:
         r = serve.client_run(srv.name, jobs, iat_us, concurrency, steps, warmup_jobs=warmup, seed=seed, dist="exp", pin_threads=True)
     return r
 
@@ -119,6 +119,7 @@ def main():
     ap.add_argument("--concurrency", type=int, default=32)
     ap.add_argument("--num-streams", type=int, default=64)
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--extra-kernels", type=int, default=16, help="full3: kernels admitted beyond the occupancy budget")
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -136,7 +137,7 @@ def main():
     tot = models.totals(args.model)
 
     log("[bench] timed arm: full3, %d streams, concurrency %d, %d warm-up + %d timed requests" % (args.num_streams, args.concurrency, args.warmup, args.steps))
-    main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup)
+    main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup, extra_kernels=args.extra_kernels)
     value = main_run["throughput_rps"]
     log("[bench]   %.1f req/s, p50 %.0f us, p99 %.0f us" % (value, main_run["all"]["p50"], main_run["all"]["p99"]))
 
@@ -148,14 +149,14 @@ def main():
             r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2)
             arms[label] = {"requests_per_s": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"], "streams": streams}
             log("[bench]   arm %-24s %.1f req/s, p99 %.0f us" % (label, r["throughput_rps"], r["all"]["p99"]))
-        single = serve_arm(serve, "full3", args.num_streams, [(job, 1.0, 1)], 1, 300, 50)
+        single = serve_arm(serve, "full3", args.num_streams, [(job, 1.0, 1)], 1, 300, 50, extra_kernels=args.extra_kernels)
         arms["full3_one_outstanding"] = {"requests_per_s": single["throughput_rps"], "p50_us": single["all"]["p50"], "p99_us": single["all"]["p99"]}
         # open-loop Poisson arrivals at fractions of the saturation rate, full3 vs multi-stream fifo
         for frac in (0.5, 0.8, 0.95):
             rate = frac * min(value, arms["fifo_multi_stream"]["requests_per_s"])
             point = {"offered_rps": rate}
             for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
-                r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2, iat_us=1e6 / rate)
+                r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2, iat_us=1e6 / rate, extra_kernels=args.extra_kernels)
                 point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"]}
             sweep.append(point)
             log("[bench]   poisson %.0f req/s: full3 p99 %.0f us, fifo p99 %.0f us" % (rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"]))

@@ -27,6 +27,11 @@
 extern "C" {
 #endif
 
+/* OR-ed into the job_id argument of a launch: the kernel reports only workgroup ENDS, not starts.  A scheduler
+ * needs start messages only for kernels it admitted beyond the occupancy budget (to learn when they have
+ * become fully resident); for every other kernel they are pure overhead.  Messages carry the id without the bit. */
+#define PAELLA_JOB_ID_NO_START 0x80000000u
+
 #define PAELLA_EINVAL (-1)   /* malformed descriptor */
 #define PAELLA_ENOSUP (-2)   /* shape class not implemented (e.g. grouped conv that is not depthwise) */
 
@@ -57,23 +62,27 @@ typedef struct paella_conv_plan {
     int P, Q;                    /* output extent */
     int kind;                    /* 0 = MFMA implicit GEMM, 1 = depthwise */
     int mi, ni, kw;              /* per-wave tile = (32*mi) x (32*ni) outputs, kw waves split the reduction */
+    int splits;                  /* workgroups per output tile that split the reduction further (grid z) */
     int m_pad, k_pad;            /* padded GEMM dims of the packed weight blob */
     size_t blob_bytes;           /* size of the packed weight blob (table + weights) */
+    size_t workspace_bytes;      /* per-request scratch for splits > 1 (0 otherwise); must start out zeroed */
     paella_launch_dims dims;
     double flops;                /* algorithmic: 2*K*(C/g)*R*S*P*Q */
     double bytes;                /* algorithmic: 4*(C*H*W + K*(C/g)*R*S + K + K*P*Q [+K*P*Q residual]) */
 } paella_conv_plan;
 
 /* Pure host arithmetic: picks the kernel variant and launch shape.  tile_hint = 0 lets the library
- * choose; otherwise mi<<8 | ni<<4 | log2(kw) forces a tile (used by the tuning sweeps and tests). */
+ * choose; otherwise log2(splits)<<12 | mi<<8 | ni<<4 | log2(kw) forces a shape (tuning sweeps and tests). */
 int paella_conv2d_plan(const paella_conv_desc* desc, int has_residual, int tile_hint, paella_conv_plan* plan);
 
 /* Re-lays out OIHW weights [K][C/g][R][S] into the blob the kernel reads (host memory to host memory). */
 int paella_conv2d_pack(const paella_conv_plan* plan, const float* w_oihw, void* blob_host);
 
-/* y = act(conv(x, w) + bias + residual); bias, residual, slope may be NULL (slope: PReLU, per channel). */
+/* y = act(conv(x, w) + bias + residual); bias, residual, slope may be NULL (slope: PReLU, per channel).
+ * workspace: device buffer of plan->workspace_bytes, private to the request (launches that share it must not
+ * overlap), zero-filled once before its first use; NULL when workspace_bytes == 0. */
 int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
-                         const float* residual, const float* slope, float* y,
+                         const float* residual, const float* slope, float* y, void* workspace,
                          void* stream, uint32_t job_id, void* notifier);
 
 /* ---------------------------------------------------------------- dense (O3) */

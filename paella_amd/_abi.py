@@ -22,7 +22,7 @@ class ConvDesc(ctypes.Structure):
 
 class ConvPlan(ctypes.Structure):
     _fields_ = [("d", ConvDesc), ("P", c_int), ("Q", c_int), ("kind", c_int), ("mi", c_int), ("ni", c_int),
-                ("kw", c_int), ("m_pad", c_int), ("k_pad", c_int), ("blob_bytes", c_size_t), ("dims", LaunchDims),
+                ("kw", c_int), ("splits", c_int), ("m_pad", c_int), ("k_pad", c_int), ("blob_bytes", c_size_t), ("workspace_bytes", c_size_t), ("dims", LaunchDims),
                 ("flops", c_double), ("bytes", c_double)]
 
 
@@ -72,7 +72,7 @@ _TAIL = [c_void_p, c_u32, c_void_p]  # stream, job_id, notifier
 OPS_SYMBOLS = {
     "paella_conv2d_plan": (c_int, [ctypes.POINTER(ConvDesc), c_int, c_int, ctypes.POINTER(ConvPlan)]),
     "paella_conv2d_pack": (c_int, [ctypes.POINTER(ConvPlan), c_void_p, c_void_p]),
-    "paella_conv2d_launch": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 6 + _TAIL),
+    "paella_conv2d_launch": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 7 + _TAIL),
     "paella_dense_dims": (c_int, [c_int, c_int, ctypes.POINTER(LaunchDims)]),
     "paella_dense_launch": (c_int, [c_void_p] * 4 + [c_int] * 3 + _TAIL),
     "paella_pool_out": (c_int, [c_int] * 5),

@@ -40,6 +40,9 @@ struct ConvArgs {
     int H, W, Q, PQ;
     int sh, sw, ph, pw;
     int K, m_pad, nchunks;
+    int splits, chunks_per_split;   // grid-level split of the reduction (gridDim.z == splits)
+    float* ws_partials;             // [tile][split][NACC][64] partial tiles (request-private workspace)
+    unsigned* ws_counters;          // [tile] arrival counters, zero between launches
     unsigned x_bytes;
     int act;
     float lo, hi;
@@ -65,9 +68,12 @@ struct Frag {
 
 template <int MI, int NI, int KW>
 __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
-    if (p.notifier) p.notifier->start(p.job_id);
+    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
 
-    extern __shared__ float red[];
+    // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
+    extern __shared__ __align__(16) char smem[];
+    int2* ltab = reinterpret_cast<int2*>(smem);
+    float* red = reinterpret_cast<float*>(smem);
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -89,9 +95,12 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         base[ni] = (hb[ni] * p.W + wb[ni]) * 4;
     }
 
-    const int cpw = (p.nchunks + KW - 1) / KW;
-    const int c_begin = wave * cpw;
-    const int c_end = min(p.nchunks, c_begin + cpw);
+    // Reduction range of this workgroup (grid-level split), then of this wave inside it.
+    const int g_begin = blockIdx.z * p.chunks_per_split;
+    const int g_end = min(p.nchunks, g_begin + p.chunks_per_split);
+    const int cpw = (g_end - g_begin + KW - 1) / KW;
+    const int c_begin = g_begin + wave * cpw;
+    const int c_end = min(g_end, c_begin + cpw);
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -101,12 +110,9 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
-    auto load_tab = [&](int c, int4& t0, int4& t1) {
-        const int4* t = reinterpret_cast<const int4*>(p.table + c * 8 + kk * 4);
-        t0 = t[0];
-        t1 = t[1];
-    };
-    auto load_frag = [&](int c, const int4& t0, const int4& t1, Frag<MI, NI>& f) {
+    auto load_frag = [&](int c, Frag<MI, NI>& f) {
+        const int4* t = reinterpret_cast<const int4*>(ltab + (c - g_begin) * 8 + kk * 4);
+        const int4 t0 = t[0], t1 = t[1];
         const float4* wrow = p.wpk + (size_t)(c * 2 + kk) * p.m_pad + m0 + j;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) f.a[mi] = wrow[mi * 32];
@@ -125,31 +131,69 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         }
     };
 
+    // Stage the table in LDS: its entries are then a short-latency LDS read away and the operand loads form
+    // two independent streams (packed weights, gathered activations) that can be kept in flight.
+    {
+        const int2* src = p.table + g_begin * 8;
+        const int n_entries = (g_end - g_begin) * 8;
+        constexpr int T = 64 * KW;
+        for (int i0 = threadIdx.x; i0 < n_entries; i0 += 4 * T) {  // four loads in flight per thread
+            int2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = (i0 + u * T < n_entries) ? src[i0 + u * T] : make_int2(0, 0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i0 + u * T < n_entries) ltab[i0 + u * T] = v[u];
+        }
+    }
+    __syncthreads();
+    // Drain every earlier vector-memory operation (the start hook's store among them) once, here: with a
+    // store still pending the compiler must assume out-of-order completion and would make every wait in
+    // the pipelined loop below a full vmcnt(0).
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+
+    // Software pipeline of depth D: D chunks of operands are in flight per wave; each slot is refilled with
+    // the chunk D ahead right after it has been consumed.  Chunk indices past the wave's range are clamped:
+    // those loads are wasted, never out of bounds.
+    constexpr int D = 4;
     if (c_begin < c_end) {
-        int4 tc0, tc1, tn0, tn1;
-        Frag<MI, NI> cur, nxt;
-        load_tab(c_begin, tc0, tc1);
-        load_tab(c_begin + 1, tn0, tn1);  // the table carries two chunks of slack past k_pad
-        load_frag(c_begin, tc0, tc1, cur);
-        for (int c = c_begin; c < c_end; ++c) {
-            int4 tf0, tf1;
-            load_tab(c + 2, tf0, tf1);
-            if (c + 1 < c_end) load_frag(c + 1, tn0, tn1, nxt);
+        const int c_last = g_end - 1;
+        Frag<MI, NI> frag[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            load_frag(min(c_begin + d, c_last), frag[d]);
+            __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
+        }
+        auto compute = [&](const Frag<MI, NI>& f) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
                 for (int mi = 0; mi < MI; ++mi) {
-                    const float av = t == 0 ? cur.a[mi].x : t == 1 ? cur.a[mi].y : t == 2 ? cur.a[mi].z : cur.a[mi].w;
+                    const float av = t == 0 ? f.a[mi].x : t == 1 ? f.a[mi].y : t == 2 ? f.a[mi].z : f.a[mi].w;
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, cur.b[ni][t], acc[mi][ni], 0, 0, 0);
-                    }
+                    for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
                 }
             }
-            cur = nxt;
-            tn0 = tf0;
-            tn1 = tf1;
+        };
+        const int n = c_end - c_begin;
+        const int c_main_end = c_begin + (n / D) * D;
+        // Branch-free steady state: whole groups of D chunks.
+        for (int c = c_begin; c < c_main_end; c += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(frag[d]);
+                // keep the refill of this slot right here: hoisting all loads to one place would make every
+                // iteration wait for the whole memory latency
+                __builtin_amdgcn_sched_barrier(0);
+                load_frag(min(c + D + d, c_last), frag[d]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
+        // Up to D-1 leftover chunks are already sitting in the first slots.
+        const int rest = n - (n / D) * D;
+#pragma unroll
+        for (int d = 0; d < D - 1; ++d)
+            if (d < rest) compute(frag[d]);
     }
 
     constexpr int NACC = MI * NI * 16;
@@ -169,14 +213,18 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         }
     };
 
+    // Each wave ends up owning RPW of the tile's NACC accumulator registers (summed over the KW waves).
+    constexpr int RPW = NACC / KW;
+    float mine[RPW];
     if (KW == 1) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) epilogue((mi * NI + ni) * 16 + e, acc[mi][ni][e]);
+                for (int e = 0; e < 16; ++e) mine[(mi * NI + ni) * 16 + e] = acc[mi][ni][e];
     } else {
+        __syncthreads();  // every wave is done with the table before the partial tiles overwrite it
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -185,18 +233,45 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
                 for (int e = 0; e < 16; ++e)
                     red[((wave * NACC) + (mi * NI + ni) * 16 + e) * 64 + lane] = acc[mi][ni][e];
         __syncthreads();
-        constexpr int RPW = NACC / KW;
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            const int r = wave * RPW + rr;
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < KW; ++w) v += red[((w * NACC) + r) * 64 + lane];
-            epilogue(r, v);
+            for (int w = 0; w < KW; ++w) v += red[((w * NACC) + wave * RPW + rr) * 64 + lane];
+            mine[rr] = v;
         }
     }
 
-    if (p.notifier) p.notifier->end_written_through(p.job_id);
+    if (p.splits == 1) {
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) epilogue(wave * RPW + rr, mine[rr]);
+    } else {
+        // Deterministic split-k: every workgroup parks its partial tile in the workspace (write-through),
+        // bumps the tile's counter, and the workgroup that arrives last adds the partials in split order and
+        // runs the epilogue.  The counter is left at zero for the next launch.
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        float* part = p.ws_partials + ((size_t)tile * p.splits + blockIdx.z) * (NACC * 64);
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) store_out(part + (wave * RPW + rr) * 64 + lane, mine[rr]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        __shared__ unsigned arrived;
+        if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(p.ws_counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (arrived == (unsigned)p.splits - 1) {
+            const float* all = p.ws_partials + (size_t)tile * p.splits * (NACC * 64);
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) {
+                float v = 0.f;
+                for (int z = 0; z < p.splits; ++z)
+                    v += __hip_atomic_load(all + (size_t)z * (NACC * 64) + (wave * RPW + rr) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                epilogue(wave * RPW + rr, v);
+            }
+            if (threadIdx.x == 0) __hip_atomic_store(p.ws_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+
+    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -218,7 +293,7 @@ struct DwArgs {
 };
 
 __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
-    if (p.notifier) p.notifier->start(p.job_id);
+    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
     const int c = blockIdx.y;
     const int pix = blockIdx.x * 256 + threadIdx.x;
     const int PQ = p.P * p.Q;
@@ -242,7 +317,7 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
         const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
         store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
     }
-    if (p.notifier) p.notifier->end_written_through(p.job_id);
+    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
 }
 
 typedef void (*ConvKernel)(ConvArgs);
@@ -265,6 +340,8 @@ ConvKernel pick_kernel(int mi, int ni, int kw) {
     if (mi == 2 && ni == 2) return pick_kw<2, 2>(kw);
     return nullptr;
 }
+
+constexpr size_t kMaxSplitTiles = 16384;  // counters at the head of a split-k workspace
 
 int conv_out(int in, int k, int stride, int pad, int dil) { return (in + 2 * pad - dil * (k - 1) - 1) / stride + 1; }
 
@@ -300,6 +377,7 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         const int k_pad = round_up(kdim, 8);
         const int nchunks = k_pad / 8;
         int mi, ni, kw;
+        auto tiles = [&](int a, int b) { return ((d->K + 32 * a - 1) / (32 * a)) * ((PQ + 32 * b - 1) / (32 * b)); };
         if (tile_hint > 0) {
             mi = (tile_hint >> 8) & 0xF;
             ni = (tile_hint >> 4) & 0xF;
@@ -308,25 +386,44 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         } else {
             // Largest tile that still yields at least one workgroup per CU; otherwise the smallest.
             const int target = 256;
-            auto tiles = [&](int a, int b) { return ((d->K + 32 * a - 1) / (32 * a)) * ((PQ + 32 * b - 1) / (32 * b)); };
             if (d->K > 32 && tiles(2, 2) >= target) { mi = 2; ni = 2; }
             else if (tiles(1, 2) >= target) { mi = 1; ni = 2; }
             else if (d->K > 32 && tiles(2, 1) >= target && PQ <= 32) { mi = 2; ni = 1; }
             else { mi = 1; ni = 1; }
-            kw = 4;
+            kw = 8;
             while (kw > 1 && nchunks / kw < 4) kw >>= 1;
-            if (tiles(mi, ni) * kw < 512 && nchunks / 8 >= 8) kw = 8;
         }
+        // Grid-level split of the reduction: layers with few output tiles (small feature maps) would otherwise
+        // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU, keep >= 4 chunks per wave.
+        const int n_tiles = tiles(mi, ni);
+        int splits = 1;
+        if (tile_hint > 0) {
+            splits = 1 << ((tile_hint >> 12) & 0xF);
+        } else {
+            while (splits < 16 && n_tiles * splits * 2 <= 288 && nchunks / (splits * 2 * kw) >= 4) splits *= 2;
+        }
+        int chunks_per_split = (nchunks + splits - 1) / splits;
+        splits = (nchunks + chunks_per_split - 1) / chunks_per_split;  // no empty split
         plan->mi = mi;
         plan->ni = ni;
         plan->kw = kw;
+        plan->splits = splits;
         plan->m_pad = round_up(d->K, 32 * mi);
         plan->k_pad = k_pad;
         const size_t table_bytes = (size_t)(k_pad + 16) * sizeof(int2);
         plan->blob_bytes = table_bytes + (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
-        plan->dims.grid = (unsigned)(((PQ + 32 * ni - 1) / (32 * ni)) * (plan->m_pad / (32 * mi)));
+        // Workspace = fixed-size counter area (so that stages of one request, which share the workspace, never
+        // see each other's partial sums where they expect zeroed counters) followed by the partial tiles.
+        if (splits > 1 && n_tiles > kMaxSplitTiles) return PAELLA_ENOSUP;
+        plan->workspace_bytes = splits > 1 ? kMaxSplitTiles * sizeof(unsigned) + (size_t)n_tiles * splits * (mi * ni * 16 * 64) * sizeof(float) : 0;
+        plan->dims.grid = (unsigned)(n_tiles * splits);
         plan->dims.block = 64u * kw;
-        plan->dims.lds_bytes = kw > 1 ? (unsigned)(kw * mi * ni * 16 * 64 * sizeof(float)) : 0u;
+        {
+            const unsigned red_bytes = kw > 1 ? (unsigned)(kw * mi * ni * 16 * 64 * sizeof(float)) : 0u;
+            const unsigned tab_bytes = (unsigned)(chunks_per_split * 8 * sizeof(int2));
+            plan->dims.lds_bytes = red_bytes > tab_bytes ? red_bytes : tab_bytes;
+            if (plan->dims.lds_bytes > 160 * 1024) return PAELLA_ENOSUP;  // table does not fit the CU's LDS
+        }
         plan->dims.vgprs = 128;
         return 0;
     }
@@ -371,8 +468,8 @@ extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, 
 }
 
 extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
-                                    const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
-                                    void* notifier) {
+                                    const float* residual, const float* slope, float* y, void* workspace, void* stream,
+                                    uint32_t job_id, void* notifier) {
     if (!plan || !x || !blob_dev || !y) return PAELLA_EINVAL;
     const paella_conv_desc& d = plan->d;
     if (d.act == PAELLA_ACT_PRELU && !slope) return PAELLA_EINVAL;
@@ -393,11 +490,23 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
         a.H = d.H; a.W = d.W; a.Q = plan->Q; a.PQ = PQ;
         a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
         a.K = d.K; a.m_pad = plan->m_pad; a.nchunks = plan->k_pad / 8;
+        a.splits = plan->splits;
+        a.chunks_per_split = (a.nchunks + plan->splits - 1) / plan->splits;
+        a.ws_partials = nullptr;
+        a.ws_counters = nullptr;
+        if (plan->splits > 1) {
+            if (!workspace) return PAELLA_EINVAL;
+            const size_t n_tiles = (size_t)((PQ + 32 * plan->ni - 1) / (32 * plan->ni)) * (plan->m_pad / (32 * plan->mi));
+            // counters first (they must be zero before the first launch; the kernel leaves them at zero)
+            a.ws_counters = reinterpret_cast<unsigned*>(workspace);
+            a.ws_partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kMaxSplitTiles * sizeof(unsigned));
+            (void)n_tiles;
+        }
         a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
         a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
         a.job_id = job_id;
         a.notifier = nf;
-        dim3 grid((PQ + 32 * plan->ni - 1) / (32 * plan->ni), plan->m_pad / (32 * plan->mi));
+        dim3 grid((PQ + 32 * plan->ni - 1) / (32 * plan->ni), plan->m_pad / (32 * plan->mi), plan->splits);
         if (plan->dims.lds_bytes > 65536) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->dims.lds_bytes);
             if (e != hipSuccess) return (int)e;

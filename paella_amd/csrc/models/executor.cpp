@@ -33,6 +33,7 @@ struct StagePlan {
 
 struct paella_model {
     Graph g;
+    size_t workspace_bytes = 0;  // largest conv workspace of any stage (stages of one request never overlap)
     uint64_t seed = 0;
     char* weights_dev = nullptr;
     std::vector<StagePlan> stages;
@@ -41,6 +42,7 @@ struct paella_model {
 struct paella_exec {
     const paella_model* m = nullptr;
     float* arena = nullptr;
+    void* workspace = nullptr;
     float* ptr(const View& v) const { return v.buf < 0 ? nullptr : arena + m->g.buffers[v.buf].offset + v.off; }
 };
 
@@ -98,6 +100,7 @@ int build(paella_model* m) {
                 }
                 blob_off[i] = total;
                 total += align256(st.conv.blob_bytes);
+                if (st.conv.workspace_bytes > m->workspace_bytes) m->workspace_bytes = st.conv.workspace_bytes;
                 break;
             case Op::Dense:
                 rc = paella_dense_dims(n.dense_in, n.dense_out, &st.dims);
@@ -269,6 +272,11 @@ int paella_exec_create(const paella_model* m, paella_exec** out) {
     paella_exec* e = new paella_exec();
     e->m = m;
     e->arena = reinterpret_cast<float*>(dev);
+    if (m->workspace_bytes) {
+        if (int rc = llis_hip_device_malloc(&e->workspace, m->workspace_bytes)) return rc;
+        if (int rc = llis_hip_fill_u32_async(e->workspace, 0, m->workspace_bytes / 4, nullptr)) return rc;
+        if (int rc = llis_hip_stream_synchronize(nullptr)) return rc;
+    }
     *out = e;
     return 0;
 }
@@ -276,6 +284,7 @@ int paella_exec_create(const paella_model* m, paella_exec** out) {
 int paella_exec_destroy(paella_exec* e) {
     if (!e) return PAELLA_EINVAL;
     llis_hip_device_free(e->arena);
+    if (e->workspace) llis_hip_device_free(e->workspace);
     delete e;
     return 0;
 }
@@ -292,7 +301,7 @@ int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t j
     float* y = e->ptr(n.y);
     switch (n.op) {
         case Op::Conv:
-            return paella_conv2d_launch(&st.conv, x, st.w, st.bias, x2, st.slope, y, stream, job_id, notifier);
+            return paella_conv2d_launch(&st.conv, x, st.w, st.bias, x2, st.slope, y, e->workspace, stream, job_id, notifier);
         case Op::Dense:
             return paella_dense_launch(x, reinterpret_cast<const float*>(st.w), st.bias, y, n.dense_in, n.dense_out, n.act, stream, job_id, notifier);
         case Op::Pool:

@@ -65,7 +65,9 @@ class ModelJob : public llis::job::CoroutineJob {
             set_smem_size_per_block(d.lds_bytes);
             set_num_registers_per_thread(d.vgprs);
             yield();
-            check(paella_exec_launch_stage(exec_, s, stream(), get_id(), get_finished_block_notifier()), "stage launch");
+            // Only a kernel admitted beyond the occupancy budget ("unfit") needs its workgroup starts reported.
+            const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START);
+            check(paella_exec_launch_stage(exec_, s, stream(), id, get_finished_block_notifier()), "stage launch");
         }
 
         set_is_mem();

@@ -51,6 +51,7 @@ class Conv2d:
         self.blob = torch.from_numpy(blob).to(device)
         self.bias = None if bias is None else torch.tensor(np.asarray(bias, np.float32), device=device)
         self.slope = None if slope is None else torch.tensor(np.asarray(slope, np.float32), device=device)
+        self.workspace = torch.zeros(max(self.plan.workspace_bytes, 4) // 4, dtype=torch.int32, device=device) if self.plan.workspace_bytes else None
         self.lib = lib
 
     def __call__(self, x, residual=None, out=None, stream=None, job_id=0, notifier=None):
@@ -59,6 +60,7 @@ class Conv2d:
         y = out if out is not None else torch.empty((1, p.d.K, p.P, p.Q), device=x.device, dtype=torch.float32)
         check(self.lib.paella_conv2d_launch(ctypes.byref(p), _ptr(x), ctypes.c_void_p(self.blob.data_ptr()),
                                             _ptr(self.bias), _ptr(residual), _ptr(self.slope), _ptr(y),
+                                            ctypes.c_void_p(self.workspace.data_ptr()) if self.workspace is not None else None,
                                             _stream(stream), job_id, notifier), "paella_conv2d_launch")
         return y
 
