@@ -46,8 +46,9 @@ def conv_roofline(models, hip, model, reps):
     stream = ctypes.c_void_p()
     hip.llis_hip_stream_create(ctypes.byref(stream))
     n = ex.num_stages
+    ops = models._abi.ops()
     ev = []
-    for _ in range(n + 1):
+    for _ in range(2):
         e = ctypes.c_void_p()
         hip.llis_hip_event_create(ctypes.byref(e))
         ev.append(e)
@@ -55,17 +56,18 @@ def conv_roofline(models, hip, model, reps):
     for _ in range(3):
         ex.forward(stream)
     hip.llis_hip_stream_synchronize(stream)
+    # Each launch stamps the event pair with the kernel's own begin/end time on the device (what a kernel trace
+    # reports); one launch at a time on an otherwise idle GPU, in forward-pass order so caches see the real sequence.
     total = [0.0] * n
+    ops.paella_ops_time_launches(ev[0], ev[1])
     for _ in range(reps):
-        hip.llis_hip_event_record(ev[0], stream)
         for i in range(n):
             ex.launch_stage(i, stream)
-            hip.llis_hip_event_record(ev[i + 1], stream)
-        hip.llis_hip_stream_synchronize(stream)
-        for i in range(n):
+            hip.llis_hip_stream_synchronize(stream)
             ms = ctypes.c_float()
-            hip.llis_hip_event_elapsed_ms(ev[i], ev[i + 1], ctypes.byref(ms))
+            hip.llis_hip_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms))
             total[i] += ms.value
+    ops.paella_ops_time_launches(None, None)
     per_stage = [t / reps * 1e3 for t in total]  # us
     # back-to-back forward without events: single-stream direct serving rate
     t0 = time.perf_counter()
@@ -122,6 +124,8 @@ def main():
     ap.add_argument("--extra-kernels", type=int, default=16, help="full3: kernels admitted beyond the occupancy budget")
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the isolated per-launch timing of one forward pass (the leg roofline.achieved comes from); value is null")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build serves from ONE GPU (one server process per GPU, no cross-GPU exchange); run with --gpus 1")
@@ -137,9 +141,13 @@ def main():
     tot = models.totals(args.model)
 
     log("[bench] timed arm: full3, %d streams, concurrency %d, %d warm-up + %d timed requests" % (args.num_streams, args.concurrency, args.warmup, args.steps))
-    main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup, extra_kernels=args.extra_kernels)
-    value = main_run["throughput_rps"]
-    log("[bench]   %.1f req/s, p50 %.0f us, p99 %.0f us" % (value, main_run["all"]["p50"], main_run["all"]["p99"]))
+    if args.roofline_only:
+        args.no_arms = args.no_cpu = True
+        main_run, value = None, None
+    else:
+        main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup, extra_kernels=args.extra_kernels)
+        value = main_run["throughput_rps"]
+        log("[bench]   %.1f req/s" % value)
 
     arms, sweep = {}, []
     if not args.no_arms:
@@ -161,7 +169,7 @@ def main():
             sweep.append(point)
             log("[bench]   poisson %.0f req/s: full3 p99 %.0f us, fifo p99 %.0f us" % (rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"]))
 
-    log("[bench] per-launch timing of the forward pass (HIP events)")
+    log("[bench] per-launch timing of the forward pass (kernel begin/end timestamps through HIP events)")
     rl = conv_roofline(models, hip, args.model, reps=50)
     achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
@@ -173,7 +181,7 @@ def main():
     ring = ctypes.c_void_p()
     lib = _abi.ops()
     notify = {}
-    if lib.paella_ring_create(1024000, 1, ctypes.byref(ring)) == 0:
+    if not args.roofline_only and lib.paella_ring_create(1024000, 1, ctypes.byref(ring)) == 0:
         us = ctypes.c_double()
         if lib.paella_ring_bench_drain(ring, 64, 6400, 50, 500, ctypes.byref(us)) == 0:
             notify["ring_drain_64_blocks_us_per_kernel"] = us.value
@@ -192,7 +200,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": main_run["elapsed_us"] / 1e3 / args.steps,
+        "ms_per_step": main_run["elapsed_us"] / 1e3 / args.steps if main_run else None,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -201,7 +209,10 @@ def main():
         "config": {"workload": "%s batch 1 fp32 1x3x224x224, seeded weights, full3 scheduler, %d streams, saturation with %d outstanding requests" %
                                (args.model, args.num_streams, args.concurrency),
                    "gmac_per_request": tot["macs"] / 1e9, "stages_per_request": tot["stages"] + 2},
-        "latency_us": {"p50": main_run["all"]["p50"], "p99": main_run["all"]["p99"], "mean": main_run["all"]["mean"]},
+        # open-loop latency at 80 % of the saturation rate; at saturation every request is submitted at t = 0 and
+        # its latency is its position in the queue, so no latency is quoted for the timed arm itself
+        "latency_us": ({"offered_rps": sweep[1]["offered_rps"], "p50": sweep[1]["full3"]["p50_us"], "p99": sweep[1]["full3"]["p99_us"]}
+                       if len(sweep) > 1 else None),
         "roofline": roofline,
         "cpu_baseline": cpu,
         "arms": arms,

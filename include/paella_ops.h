@@ -141,6 +141,14 @@ int paella_kernel_vgprs(const char* family, unsigned* vgprs);
 /* Same for a conv variant: kind 0 = MFMA implicit GEMM with tile (mi, ni, kw), kind 1 = depthwise. */
 int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs);
 
+/*
+ * Measurement aid.  While a pair of events (llis_hip_event_create) is armed on the calling thread, every
+ * operator launch made by that thread stamps them with the kernel's own begin and end time on the device, so
+ * llis_hip_event_elapsed_ms(start, stop) after a stream synchronize is that launch's execution time, the same
+ * quantity a kernel trace reports.  Pass NULL, NULL to disarm.  Not for concurrent use of one event pair.
+ */
+int paella_ops_time_launches(void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

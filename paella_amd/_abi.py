@@ -90,6 +90,7 @@ OPS_SYMBOLS = {
     "paella_lrn_launch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_float] + _TAIL),
     "paella_kernel_vgprs": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv_kernel_vgprs": (c_int, [c_int] * 4 + [ctypes.POINTER(c_uint)]),
+    "paella_ops_time_launches": (c_int, [c_void_p, c_void_p]),
 }
 
 RING_SYMBOLS = {

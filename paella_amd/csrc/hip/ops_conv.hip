@@ -23,6 +23,7 @@
 #include "paella_ops.h"
 #include <llis/job/finished_block_notifier.h>
 
+#include "launch.h"
 #include "out_store.h"
 
 namespace {
@@ -511,7 +512,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->dims.lds_bytes);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(kern, grid, dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
+        paella::launch(kern, grid, dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
         return (int)hipGetLastError();
     }
     DwArgs a;
@@ -522,7 +523,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.job_id = job_id;
     a.notifier = nf;
     dim3 grid((PQ + 255) / 256, d.C);
-    hipLaunchKernelGGL(dwconv_kernel, grid, dim3(256), 0, st, a);
+    paella::launch(dwconv_kernel, grid, dim3(256), 0, st, a);
     return (int)hipGetLastError();
 }
 

@@ -10,6 +10,7 @@
 #include "paella_ops.h"
 #include <llis/job/finished_block_notifier.h>
 
+#include "launch.h"
 #include "out_store.h"
 
 namespace {
@@ -254,6 +255,11 @@ inline void set_dims(paella_launch_dims* d, unsigned grid, unsigned block, unsig
 
 }  // namespace
 
+paella::TimingEvents& paella::timing_events() {
+    static thread_local paella::TimingEvents events;
+    return events;
+}
+
 extern "C" {
 
 int paella_pool_out(int in, int k, int stride, int pad, int ceil_mode) {
@@ -277,7 +283,7 @@ int paella_dense_dims(int I, int O, paella_launch_dims* dims) {
 int paella_dense_launch(const float* x, const float* w, const float* bias, float* y, int I, int O, int act, void* stream,
                         uint32_t job_id, void* notifier) {
     if (!x || !w || !y || I <= 0 || O <= 0 || act < 0 || act > PAELLA_ACT_RELU6) return PAELLA_EINVAL;
-    hipLaunchKernelGGL(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
+    paella::launch(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
                        (Notifier*)notifier);
     return (int)hipGetLastError();
 }
@@ -309,7 +315,7 @@ int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y, vo
     a.sh = d->stride_h; a.sw = d->stride_w; a.ph = d->pad_h; a.pw = d->pad_w;
     a.is_avg = d->is_avg; a.count_include_pad = d->count_include_pad;
     a.job_id = job_id; a.notifier = (Notifier*)notifier;
-    hipLaunchKernelGGL(pool_kernel, dim3(blocks_for((size_t)d->C * P * Q, 256)), dim3(256), 0, (hipStream_t)stream, a);
+    paella::launch(pool_kernel, dim3(blocks_for((size_t)d->C * P * Q, 256)), dim3(256), 0, (hipStream_t)stream, a);
     return (int)hipGetLastError();
 }
 
@@ -321,7 +327,7 @@ int paella_global_avgpool_dims(int C, int HW, paella_launch_dims* dims) {
 
 int paella_global_avgpool_launch(const float* x, float* y, int C, int HW, void* stream, uint32_t job_id, void* notifier) {
     if (!x || !y || C <= 0 || HW <= 0) return PAELLA_EINVAL;
-    hipLaunchKernelGGL(gap_kernel, dim3(blocks_for(C, 4)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, job_id, (Notifier*)notifier);
+    paella::launch(gap_kernel, dim3(blocks_for(C, 4)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, job_id, (Notifier*)notifier);
     return (int)hipGetLastError();
 }
 
@@ -343,9 +349,9 @@ int paella_eltwise_launch(const float* a, const float* b, const float* scale, co
     const size_t n = (size_t)C * HW;
     const bool aligned = ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) == 0);
     if ((HW & 3) == 0 && aligned) {
-        hipLaunchKernelGGL(eltwise_kernel<true>, dim3(blocks_for(n / 4, 256)), dim3(256), 0, (hipStream_t)stream, p);
+        paella::launch(eltwise_kernel<true>, dim3(blocks_for(n / 4, 256)), dim3(256), 0, (hipStream_t)stream, p);
     } else {
-        hipLaunchKernelGGL(eltwise_kernel<false>, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, p);
+        paella::launch(eltwise_kernel<false>, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, p);
     }
     return (int)hipGetLastError();
 }
@@ -358,7 +364,7 @@ int paella_copy_dims(size_t n, paella_launch_dims* dims) {
 
 int paella_copy_launch(const float* x, float* y, size_t n, void* stream, uint32_t job_id, void* notifier) {
     if (!x || !y || n == 0) return PAELLA_EINVAL;
-    hipLaunchKernelGGL(copy_kernel, dim3(blocks_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream, x, y, n, job_id,
+    paella::launch(copy_kernel, dim3(blocks_for((n + 3) / 4, 256)), dim3(256), 0, (hipStream_t)stream, x, y, n, job_id,
                        (Notifier*)notifier);
     return (int)hipGetLastError();
 }
@@ -371,7 +377,7 @@ int paella_softmax_dims(int rows, int cols, paella_launch_dims* dims) {
 
 int paella_softmax_launch(const float* x, float* y, int rows, int cols, void* stream, uint32_t job_id, void* notifier) {
     if (!x || !y || rows <= 0 || cols <= 0) return PAELLA_EINVAL;
-    hipLaunchKernelGGL(softmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, y, cols, job_id, (Notifier*)notifier);
+    paella::launch(softmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, y, cols, job_id, (Notifier*)notifier);
     return (int)hipGetLastError();
 }
 
@@ -384,9 +390,17 @@ int paella_lrn_dims(int C, int HW, paella_launch_dims* dims) {
 int paella_lrn_launch(const float* x, float* y, int C, int HW, int size, float alpha, float beta, float k, void* stream,
                       uint32_t job_id, void* notifier) {
     if (!x || !y || C <= 0 || HW <= 0 || size <= 0) return PAELLA_EINVAL;
-    hipLaunchKernelGGL(lrn_kernel, dim3(blocks_for((size_t)C * HW, 256)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, size, alpha,
+    paella::launch(lrn_kernel, dim3(blocks_for((size_t)C * HW, 256)), dim3(256), 0, (hipStream_t)stream, x, y, C, HW, size, alpha,
                        beta, k, job_id, (Notifier*)notifier);
     return (int)hipGetLastError();
+}
+
+int paella_ops_time_launches(void* start_event, void* stop_event) {
+    if ((start_event == nullptr) != (stop_event == nullptr)) return PAELLA_EINVAL;
+    paella::TimingEvents& t = paella::timing_events();
+    t.start = (hipEvent_t)start_event;
+    t.stop = (hipEvent_t)stop_event;
+    return 0;
 }
 
 int paella_kernel_vgprs(const char* family, unsigned* vgprs) {
