@@ -26,7 +26,15 @@ class Context {
     static void set_mem2sched_channel(ipc::ShmChannelCpuReader* channel) { mem2sched_channel_ = channel->fork(); }
     static ipc::ShmChannelCpuWriter* get_mem2sched_channel() { return &mem2sched_channel_; }
 
+    // True when the active scheduler issues a job's next stage only after the previous one has been reported
+    // finished (fifo2, full3); false when it issues all stages at once and relies on stream order (fifo).
+    // A job may submit its kernels outside its stream only in the first case.  Not in the reference, whose
+    // jobs always launch on the stream.
+    static void set_stage_by_stage(bool v) { stage_by_stage_ = v; }
+    static bool is_stage_by_stage() { return stage_by_stage_; }
+
   private:
+    static bool stage_by_stage_;
     static Job* current_job_;
     static ipc::Gpu2SchedChannel gpu2sched_channel_;
     static ipc::Gpu2SchedChannel gpu2sched_block_time_channel_;

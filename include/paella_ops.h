@@ -33,7 +33,8 @@ extern "C" {
 #define PAELLA_JOB_ID_NO_START 0x80000000u
 
 #define PAELLA_EINVAL (-1)   /* malformed descriptor */
-#define PAELLA_ENOSUP (-2)   /* shape class not implemented (e.g. grouped conv that is not depthwise) */
+#define PAELLA_ENOSUP (-2)   /* shape class not implemented (e.g. grouped conv that is not depthwise), or facility unavailable */
+#define PAELLA_ETIMEDOUT (-3) /* a bounded wait expired */
 
 enum paella_act { PAELLA_ACT_NONE = 0, PAELLA_ACT_RELU = 1, PAELLA_ACT_RELU6 = 2, PAELLA_ACT_PRELU = 3, PAELLA_ACT_CLIP = 4 };
 
@@ -64,7 +65,7 @@ typedef struct paella_conv_plan {
     int mi, ni, kw;              /* per-wave tile = (32*mi) x (32*ni) outputs, kw waves split the reduction */
     int splits;                  /* workgroups per output tile that split the reduction further (grid z) */
     int m_pad, k_pad;            /* padded GEMM dims of the packed weight blob */
-    size_t blob_bytes;           /* size of the packed weight blob (table + weights) */
+    size_t blob_bytes;           /* size of the packed weight blob */
     size_t workspace_bytes;      /* per-request scratch for splits > 1 (0 otherwise); must start out zeroed */
     paella_launch_dims dims;
     double flops;                /* algorithmic: 2*K*(C/g)*R*S*P*Q */
@@ -140,6 +141,26 @@ int paella_lrn_launch(const float* x, float* y, int C, int HW, int size, float a
 int paella_kernel_vgprs(const char* family, unsigned* vgprs);
 /* Same for a conv variant: kind 0 = MFMA implicit GEMM with tile (mi, ni, kw), kind 1 = depthwise. */
 int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs);
+
+/*
+ * Direct dispatch.  A queue created here is a user-mode hardware queue owned by this library; its handle can
+ * be passed wherever a launch function of this header (or paella_exec_launch_stage / paella_exec_forward)
+ * takes `void* stream`, and the kernel is then submitted as one AQL packet written by the calling thread
+ * instead of going through the HIP launch path (a few hundred nanoseconds instead of 2.3 to 3.9 us of host
+ * time).  Kernels submitted to one queue are NOT ordered with respect to each other or to HIP streams: the
+ * caller orders dependent work itself, as the serving path does with the notification ring (or with
+ * paella_direct_queue_wait).  One producer thread per queue.  Returns PAELLA_ENOSUP when the runtime cannot
+ * provide such queues.  No counterpart in the reference: CUDA launches are cheap enough there.
+ */
+int paella_direct_queue_create(void** queue);
+/* ordered != 0: every later kernel waits for all earlier ones of this queue (stream semantics). Default 0. */
+int paella_direct_queue_set_ordered(void* queue, int ordered);
+/* Blocks until every kernel submitted to the queue so far has finished (at most 10 s: PAELLA_ETIMEDOUT). */
+int paella_direct_queue_wait(void* queue);
+/* Next of a process-wide set of unordered queues (PAELLA_DIRECT_QUEUES of them, default 4), round-robin.  All
+ * callers must be the same thread.  The set lives until the process ends. */
+int paella_direct_queue_shared(void** queue);
+int paella_direct_queue_destroy(void* queue);
 
 /*
  * Measurement aid.  While a pair of events (llis_hip_event_create) is armed on the calling thread, every

@@ -91,6 +91,11 @@ OPS_SYMBOLS = {
     "paella_kernel_vgprs": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv_kernel_vgprs": (c_int, [c_int] * 4 + [ctypes.POINTER(c_uint)]),
     "paella_ops_time_launches": (c_int, [c_void_p, c_void_p]),
+    "paella_direct_queue_create": (c_int, [ctypes.POINTER(c_void_p)]),
+    "paella_direct_queue_set_ordered": (c_int, [c_void_p, c_int]),
+    "paella_direct_queue_wait": (c_int, [c_void_p]),
+    "paella_direct_queue_shared": (c_int, [ctypes.POINTER(c_void_p)]),
+    "paella_direct_queue_destroy": (c_int, [c_void_p]),
 }
 
 RING_SYMBOLS = {

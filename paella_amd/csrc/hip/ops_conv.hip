@@ -12,8 +12,9 @@
 //   * weights are pre-packed on the host as float4 groups [k/4][m][4], so lane (i, kk) fetches the four
 //     k values {8c + 4kk + t} of row i with one 16-byte load and a half wave reads 512 contiguous bytes;
 //   * the im2col operand is gathered straight from the activation tensor with raw buffer loads whose
-//     out-of-range offsets return 0: padding taps, the k tail and the pixel tail need no branches.  A
-//     per-layer table maps k -> {byte offset c*H*W + r*dil*W + s*dil, (r*dil) << 16 | (s*dil)}.
+//     out-of-range offsets return 0: padding taps, the k tail and the pixel tail need no branches.  Each
+//     workgroup first builds, in LDS, the table k -> {byte offset c*H*W + r*dil*W + s*dil, (r*dil) << 16 | (s*dil)}
+//     for its slice of the reduction.
 
 #include <hip/hip_runtime.h>
 
@@ -26,13 +27,27 @@
 #include "launch.h"
 #include "out_store.h"
 
+// Build-time diagnostic (never defined in the shipped library): thread 0 of every workgroup records the
+// 100 MHz wall clock at a few points of the kernel.
+#ifdef PAELLA_CONV_TIMELINE
+__device__ unsigned long long g_conv_timeline[8192 * 12];
+#define CONV_TL(i)                                                                                        \
+    do {                                                                                                  \
+        if (threadIdx.x == 0) {                                                                           \
+            const unsigned b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;           \
+            if (b_ < 8192) g_conv_timeline[b_ * 12 + (i)] = wall_clock64();                               \
+        }                                                                                                 \
+    } while (0)
+#else
+#define CONV_TL(i)
+#endif
+
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct ConvArgs {
     const float* x;
-    const int2* table;
     const float4* wpk;
     const float* bias;
     const float* residual;
@@ -41,6 +56,8 @@ struct ConvArgs {
     int H, W, Q, PQ;
     int sh, sw, ph, pw;
     int K, m_pad, nchunks;
+    int kdim, RS, S, dh, dw;        // reduction length C*R*S, filter plane R*S, filter width, dilations
+    unsigned w_bytes;               // size of the packed weights
     int splits, chunks_per_split;   // grid-level split of the reduction (gridDim.z == splits)
     float* ws_partials;             // [tile][split][NACC][64] partial tiles (request-private workspace)
     unsigned* ws_counters;          // [tile] arrival counters, zero between launches
@@ -67,8 +84,22 @@ struct Frag {
     float b[NI][4];
 };
 
+// Build-time diagnostic: -DPAELLA_CONV_ABLATE=<bits> removes parts of the kernel to see what bounds it
+// (1 = no MFMA, 2 = no operand loads, 4 = no cross-wave reduction, 8 = no table build, 16 = empty kernel, 32 = no epilogue).  Results are wrong.
+#ifndef PAELLA_CONV_ABLATE
+#define PAELLA_CONV_ABLATE 0
+#endif
+#ifndef PAELLA_CONV_DEPTH
+#define PAELLA_CONV_DEPTH 8
+#endif
+#ifndef PAELLA_CONV_MINB
+#define PAELLA_CONV_MINB 1
+#endif
+
 template <int MI, int NI, int KW>
-__global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
+__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
+    CONV_TL(0);
+    if (PAELLA_CONV_ABLATE & 16) return;
     if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
 
     // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
@@ -111,12 +142,19 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
-    auto load_frag = [&](int c, Frag<MI, NI>& f) {
-        const int4* t = reinterpret_cast<const int4*>(ltab + (c - g_begin) * 8 + kk * 4);
+    // Chunks outside [c_begin, c_end) are requested at an out-of-range offset: the loads keep their place in
+    // the (static) issue order, return zeros and touch no memory.
+    __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, p.w_bytes, 0x00027000);
+    auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
+        if (PAELLA_CONV_ABLATE & 2) valid = false;
+        const int4* t = reinterpret_cast<const int4*>(ltab + ((valid ? c : g_begin) - g_begin) * 8 + kk * 4);
         const int4 t0 = t[0], t1 = t[1];
-        const float4* wrow = p.wpk + (size_t)(c * 2 + kk) * p.m_pad + m0 + j;
+        const int woff = valid ? (int)((((unsigned)(c * 2 + kk) * (unsigned)p.m_pad) + (unsigned)(m0 + j)) * 16u) : -1;
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) f.a[mi] = wrow[mi * 32];
+        for (int mi = 0; mi < MI; ++mi) {
+            const auto v = __builtin_amdgcn_raw_buffer_load_b128(wres, woff, mi * 32 * 16, 0);
+            f.a[mi] = __builtin_bit_cast(float4, v);
+        }
         const int off[4] = {t0.x, t0.z, t1.x, t1.z};
         const int rs[4] = {t0.y, t0.w, t1.y, t1.w};
 #pragma unroll
@@ -125,26 +163,28 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
             for (int t = 0; t < 4; ++t) {
                 const int h = hb[ni] + (rs[t] >> 16);
                 const int w = wb[ni] + (rs[t] & 0xFFFF);
-                const bool ok = ((unsigned)h < (unsigned)p.H) & ((unsigned)w < (unsigned)p.W);
+                const bool ok = valid & ((unsigned)h < (unsigned)p.H) & ((unsigned)w < (unsigned)p.W);
                 const int voff = ok ? base[ni] + off[t] : -1;
                 f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, voff, 0, 0));
             }
         }
     };
 
-    // Stage the table in LDS: its entries are then a short-latency LDS read away and the operand loads form
-    // two independent streams (packed weights, gathered activations) that can be kept in flight.
+    // Build this workgroup's slice of the k -> offset table in LDS (a few entries per thread, arithmetic only).
     {
-        const int2* src = p.table + g_begin * 8;
         const int n_entries = (g_end - g_begin) * 8;
-        constexpr int T = 64 * KW;
-        for (int i0 = threadIdx.x; i0 < n_entries; i0 += 4 * T) {  // four loads in flight per thread
-            int2 v[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = (i0 + u * T < n_entries) ? src[i0 + u * T] : make_int2(0, 0);
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-                if (i0 + u * T < n_entries) ltab[i0 + u * T] = v[u];
+        const int HW4 = p.H * p.W * 4;
+        for (int i = threadIdx.x; i < ((PAELLA_CONV_ABLATE & 8) ? 0 : n_entries); i += 64 * KW) {
+            const int k = g_begin * 8 + i;
+            const int c = k / p.RS;
+            const int rem = k - c * p.RS;
+            const int r = rem / p.S;
+            const int sx = rem - r * p.S;
+            int2 e;
+            e.x = c * HW4 + (r * p.dh * p.W + sx * p.dw) * 4;
+            e.y = ((r * p.dh) << 16) | (sx * p.dw);
+            if (k >= p.kdim) e = make_int2(0, 0x7FFF0000);  // row far outside the image: the tap reads as zero
+            ltab[i] = e;
         }
     }
     __syncthreads();
@@ -152,17 +192,43 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
     // store still pending the compiler must assume out-of-order completion and would make every wait in
     // the pipelined loop below a full vmcnt(0).
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+    CONV_TL(1);
+
+    // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
+    // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
+    constexpr int NACC = MI * NI * 16;
+    constexpr int RPW = NACC / KW;
+    constexpr bool kPrefetchEpilogue = RPW <= 16;
+    float bias_v[RPW], res_v[RPW];
+    auto out_coords = [&](int r, int& m, int& pix) {
+        const int tile = r >> 4;
+        const int e = r & 15;
+        const int mi = tile / NI;
+        const int ni = tile - mi * NI;
+        m = m0 + mi * 32 + (e >> 2) * 8 + kk * 4 + (e & 3);
+        pix = n0 + ni * 32 + j;
+    };
+    if (kPrefetchEpilogue) {
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {
+            int m, pix;
+            out_coords(wave * RPW + rr, m, pix);
+            const bool ok = m < p.K && pix < p.PQ;
+            bias_v[rr] = (ok && p.bias) ? p.bias[m] : 0.f;
+            res_v[rr] = (ok && p.residual) ? p.residual[(size_t)m * p.PQ + pix] : 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     // Software pipeline of depth D: D chunks of operands are in flight per wave; each slot is refilled with
-    // the chunk D ahead right after it has been consumed.  Chunk indices past the wave's range are clamped:
-    // those loads are wasted, never out of bounds.
-    constexpr int D = 4;
+    // the chunk D ahead right after it has been consumed.  With the small tile a wave's whole slice of a
+    // typical layer (8 to 10 chunks) is requested up front.
+    constexpr int D = (MI * NI == 1) ? PAELLA_CONV_DEPTH : 4;
     if (c_begin < c_end) {
-        const int c_last = g_end - 1;
         Frag<MI, NI> frag[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            load_frag(min(c_begin + d, c_last), frag[d]);
+            load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
         }
         auto compute = [&](const Frag<MI, NI>& f) {
@@ -172,10 +238,14 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
                 for (int mi = 0; mi < MI; ++mi) {
                     const float av = t == 0 ? f.a[mi].x : t == 1 ? f.a[mi].y : t == 2 ? f.a[mi].z : f.a[mi].w;
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
+                    for (int ni = 0; ni < NI; ++ni) {
+                        if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * f.b[ni][t];
+                        else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
+                    }
                 }
             }
         };
+        CONV_TL(2);
         const int n = c_end - c_begin;
         const int c_main_end = c_begin + (n / D) * D;
         // Branch-free steady state: whole groups of D chunks.
@@ -186,7 +256,7 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
                 // keep the refill of this slot right here: hoisting all loads to one place would make every
                 // iteration wait for the whole memory latency
                 __builtin_amdgcn_sched_barrier(0);
-                load_frag(min(c + D + d, c_last), frag[d]);
+                load_frag(c + D + d, c + D + d < c_end, frag[d]);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -197,33 +267,33 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
             if (d < rest) compute(frag[d]);
     }
 
-    constexpr int NACC = MI * NI * 16;
-    auto epilogue = [&](int r, float v) {
-        const int tile = r >> 4;
-        const int e = r & 15;
-        const int mi = tile / NI;
-        const int ni = tile - mi * NI;
-        const int m = m0 + mi * 32 + (e >> 2) * 8 + kk * 4 + (e & 3);
-        const int pix = n0 + ni * 32 + j;
+    CONV_TL(3);
+    auto epilogue = [&](int rr, float v) {
+        int m, pix;
+        out_coords(wave * RPW + rr, m, pix);
         if (m < p.K && pix < p.PQ) {
-            if (p.bias) v += p.bias[m];
             const size_t o = (size_t)m * p.PQ + pix;
-            if (p.residual) v += p.residual[o];
+            if (kPrefetchEpilogue) {
+                v += bias_v[rr];
+                v += res_v[rr];
+            } else {
+                if (p.bias) v += p.bias[m];
+                if (p.residual) v += p.residual[o];
+            }
             const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
             store_out(p.y + o, apply_act(v, p.act, sl, p.lo, p.hi));
         }
     };
 
-    // Each wave ends up owning RPW of the tile's NACC accumulator registers (summed over the KW waves).
-    constexpr int RPW = NACC / KW;
     float mine[RPW];
-    if (KW == 1) {
+    if (KW == 1 || (PAELLA_CONV_ABLATE & 4)) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) mine[(mi * NI + ni) * 16 + e] = acc[mi][ni][e];
+                for (int e = 0; e < 16; ++e)
+                    if ((mi * NI + ni) * 16 + e < RPW) mine[(mi * NI + ni) * 16 + e] = acc[mi][ni][e];
     } else {
         __syncthreads();  // every wave is done with the table before the partial tiles overwrite it
 #pragma unroll
@@ -243,9 +313,14 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         }
     }
 
+    CONV_TL(4);
+    if (PAELLA_CONV_ABLATE & 32) {
+        if (mine[0] == 12345.f) p.y[0] = 0.f;
+        return;
+    }
     if (p.splits == 1) {
 #pragma unroll
-        for (int rr = 0; rr < RPW; ++rr) epilogue(wave * RPW + rr, mine[rr]);
+        for (int rr = 0; rr < RPW; ++rr) epilogue(rr, mine[rr]);
     } else {
         // Deterministic split-k: every workgroup parks its partial tile in the workspace (write-through),
         // bumps the tile's counter, and the workgroup that arrives last adds the partials in split order and
@@ -256,23 +331,43 @@ __global__ __launch_bounds__(64 * KW) void conv_mfma_kernel(ConvArgs p) {
         for (int rr = 0; rr < RPW; ++rr) store_out(part + (wave * RPW + rr) * 64 + lane, mine[rr]);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        CONV_TL(5);
         __shared__ unsigned arrived;
         if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(p.ws_counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
+        CONV_TL(6);
         if (arrived == (unsigned)p.splits - 1) {
-            const float* all = p.ws_partials + (size_t)tile * p.splits * (NACC * 64);
+            const float* all = p.ws_partials + (size_t)tile * p.splits * (NACC * 64) + (size_t)(wave * RPW) * 64 + lane;
+            float v[RPW];
 #pragma unroll
-            for (int rr = 0; rr < RPW; ++rr) {
-                float v = 0.f;
-                for (int z = 0; z < p.splits; ++z)
-                    v += __hip_atomic_load(all + (size_t)z * (NACC * 64) + (wave * RPW + rr) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                epilogue(wave * RPW + rr, v);
+            for (int rr = 0; rr < RPW; ++rr) v[rr] = 0.f;
+            constexpr int ZB = RPW <= 4 ? 8 : (RPW <= 16 ? 4 : 1);  // partial tiles requested together
+            for (int z0 = 0; z0 < p.splits; z0 += ZB) {
+                float t[ZB][RPW];
+#pragma unroll
+                for (int u = 0; u < ZB; ++u)
+#pragma unroll
+                    for (int rr = 0; rr < RPW; ++rr)
+                        t[u][rr] = (z0 + u < p.splits)
+                                       ? __hip_atomic_load(all + (size_t)(z0 + u) * (NACC * 64) + rr * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0.f;
+#pragma unroll
+                for (int u = 0; u < ZB; ++u)  // split order: the sum does not depend on which workgroup came last
+#pragma unroll
+                    for (int rr = 0; rr < RPW; ++rr) v[rr] += t[u][rr];
             }
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) epilogue(rr, v[rr]);
             if (threadIdx.x == 0) __hip_atomic_store(p.ws_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 
+    CONV_TL(7);
     if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
+#ifdef PAELLA_CONV_TIMELINE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    CONV_TL(8);
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -411,8 +506,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->splits = splits;
         plan->m_pad = round_up(d->K, 32 * mi);
         plan->k_pad = k_pad;
-        const size_t table_bytes = (size_t)(k_pad + 16) * sizeof(int2);
-        plan->blob_bytes = table_bytes + (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
+        plan->blob_bytes = (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
+        if (plan->blob_bytes >= ((size_t)1 << 31)) return PAELLA_ENOSUP;  // weights are addressed with 32-bit byte offsets
         // Workspace = fixed-size counter area (so that stages of one request, which share the workspace, never
         // see each other's partial sums where they expect zeroed counters) followed by the partial tiles.
         if (splits > 1 && n_tiles > kMaxSplitTiles) return PAELLA_ENOSUP;
@@ -448,20 +543,7 @@ extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, 
         return 0;
     }
     const int kdim = d.C * d.R * d.S;
-    int2* table = reinterpret_cast<int2*>(blob_host);
-    for (int k = 0; k < plan->k_pad + 16; ++k) {
-        if (k < kdim) {
-            const int c = k / (d.R * d.S);
-            const int r = (k / d.S) % d.R;
-            const int s = k % d.S;
-            table[k].x = (c * d.H * d.W + r * d.dil_h * d.W + s * d.dil_w) * 4;
-            table[k].y = ((r * d.dil_h) << 16) | (s * d.dil_w);
-        } else {
-            table[k].x = 0;
-            table[k].y = 0x7FFF0000;  // row far outside the image: the tap always reads as zero
-        }
-    }
-    float* wp = reinterpret_cast<float*>(reinterpret_cast<char*>(blob_host) + (size_t)(plan->k_pad + 16) * sizeof(int2));
+    float* wp = reinterpret_cast<float*>(blob_host);
     std::memset(wp, 0, (size_t)(plan->k_pad / 4) * plan->m_pad * sizeof(float4));
     for (int m = 0; m < d.K; ++m)
         for (int k = 0; k < kdim; ++k) wp[((size_t)(k / 4) * plan->m_pad + m) * 4 + (k % 4)] = w[(size_t)m * kdim + k];
@@ -482,8 +564,9 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
         if (!kern) return PAELLA_EINVAL;
         ConvArgs a;
         a.x = x;
-        a.table = reinterpret_cast<const int2*>(blob_dev);
-        a.wpk = reinterpret_cast<const float4*>(reinterpret_cast<const char*>(blob_dev) + (size_t)(plan->k_pad + 16) * sizeof(int2));
+        a.wpk = reinterpret_cast<const float4*>(blob_dev);
+        a.w_bytes = (unsigned)plan->blob_bytes;
+        a.kdim = d.C * d.R * d.S; a.RS = d.R * d.S; a.S = d.S; a.dh = d.dil_h; a.dw = d.dil_w;
         a.bias = bias;
         a.residual = residual;
         a.slope = slope;

@@ -44,13 +44,22 @@ class ModelJob : public llis::job::CoroutineJob {
         check(llis_hip_host_alloc_pinned(&p, in_bytes_ + out_bytes_), "pinned staging");
         staging_ = reinterpret_cast<char*>(p);
         num_stages_ = paella_model_num_stages(model_);
+        // Kernels go out as AQL packets on the operator library's own queues unless PAELLA_DISPATCH=hip; the
+        // copies stay on the pooled HIP stream.  Only under a scheduler that orders a job's stages through the
+        // notification ring (fifo2, full3): the queues have no ordering of their own, and fifo relies on the stream.
+        const char* dispatch = std::getenv("PAELLA_DISPATCH");
+        direct_ = !(dispatch && std::strcmp(dispatch, "hip") == 0) && llis::job::Context::is_stage_by_stage();
+        if (direct_) {
+            void* probe = nullptr;
+            if (paella_direct_queue_shared(&probe) != 0) {
+                std::fprintf(stderr, "[llis] model job: direct dispatch unavailable, using HIP launches\n");
+                direct_ = false;
+            }
+        }
     }
 
     void body(void* io_ptr) override {
         io_ptr_ = io_ptr;
-        void* stream_unused = nullptr;
-        (void)stream_unused;
-
         set_is_mem();
         yield();
         std::memcpy(staging_, io_ptr, in_bytes_);
@@ -67,7 +76,9 @@ class ModelJob : public llis::job::CoroutineJob {
             yield();
             // Only a kernel admitted beyond the occupancy budget ("unfit") needs its workgroup starts reported.
             const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START);
-            check(paella_exec_launch_stage(exec_, s, stream(), id, get_finished_block_notifier()), "stage launch");
+            void* target = stream();
+            if (direct_) check(paella_direct_queue_shared(&target), "direct queue");
+            check(paella_exec_launch_stage(exec_, s, target, id, get_finished_block_notifier()), "stage launch");
         }
 
         set_is_mem();
@@ -96,6 +107,7 @@ class ModelJob : public llis::job::CoroutineJob {
     char* staging_ = nullptr;
     void* io_ptr_ = nullptr;
     int num_stages_ = 0;
+    bool direct_ = true;
 };
 
 }  // namespace paella

@@ -1,4 +1,5 @@
 #include <llis/job/context.h>
+#include <llis/server/phase_clock.h>
 #include <llis/server/scheduler.h>
 #include <llis/utils/error.h>
 
@@ -59,6 +60,7 @@ StreamPoolScheduler::~StreamPoolScheduler() {
 
 void StreamPoolScheduler::try_handle_block_start_finish() {
     if (gpu2sched_channel_.can_read<job::InstrumentInfo>()) {
+        LLIS_PHASE(kRing);
         const job::InstrumentInfo info = gpu2sched_channel_.read<job::InstrumentInfo>();
         job::Job* job = job_of(info.job_id);
         if (info.is_start == 1) {
@@ -72,7 +74,11 @@ void StreamPoolScheduler::try_handle_block_start_finish() {
             handle_mem_finish(job);
         }
     }
+    else {
+        LLIS_PHASE(kIdle);
+    }
     if (mem2sched_channel_.can_read()) {
+        LLIS_PHASE(kRing);
         job::Job* job;
         mem2sched_channel_.read(&job);
         log_->add('M', job->get_id());

@@ -4,7 +4,7 @@
 namespace llis {
 namespace server {
 
-SchedulerFifo::SchedulerFifo(const SchedulerOptions& options) : StreamPoolScheduler(options, 10240) {}
+SchedulerFifo::SchedulerFifo(const SchedulerOptions& options) : StreamPoolScheduler(options, 10240) { job::Context::set_stage_by_stage(false); }
 
 void SchedulerFifo::handle_new_job(std::unique_ptr<job::Job> owned) {
     if (!owned->has_next()) {  // a job without stages has nothing to run

@@ -4,7 +4,7 @@
 namespace llis {
 namespace server {
 
-SchedulerFifo2::SchedulerFifo2(const SchedulerOptions& options) : StreamPoolScheduler(options, 10240) {}
+SchedulerFifo2::SchedulerFifo2(const SchedulerOptions& options) : StreamPoolScheduler(options, 10240) { job::Context::set_stage_by_stage(true); }
 
 void SchedulerFifo2::handle_new_job(std::unique_ptr<job::Job> owned) {
     if (!owned->has_next()) {

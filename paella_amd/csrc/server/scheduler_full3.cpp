@@ -1,4 +1,5 @@
 #include <llis/job/context.h>
+#include <llis/server/phase_clock.h>
 #include <llis/server/scheduler_full3.h>
 
 #include <chrono>
@@ -68,10 +69,14 @@ job::Job* JobQueue::pop() {
 
 // ------------------------------------------------------------------------------------------ SchedulerFull3
 
-SchedulerFull3::SchedulerFull3(const SchedulerOptions& options) : StreamPoolScheduler(options, 409600), job_queue_(options.unfair) {}
+SchedulerFull3::SchedulerFull3(const SchedulerOptions& options) : StreamPoolScheduler(options, 409600), job_queue_(options.unfair) {
+    job::Context::set_stage_by_stage(true);
+}
 
 SchedulerFull3::SchedulerFull3(const SchedulerOptions& options, const SmResources& budget)
-    : StreamPoolScheduler(options, 409600), job_queue_(options.unfair), gpu_resources_(budget) {}
+    : StreamPoolScheduler(options, 409600), job_queue_(options.unfair), gpu_resources_(budget) {
+    job::Context::set_stage_by_stage(true);
+}
 
 void SchedulerFull3::set_server(Server* server) {
     Scheduler::set_server(server);
@@ -198,8 +203,11 @@ void SchedulerFull3::schedule_job() {
 
         job::Context::set_current_job(job);
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_START);
-        job->run_next();
-        if (is_mem) post_mem_completion(job);
+        {
+            LLIS_PHASE(kLaunch);
+            job->run_next();
+            if (is_mem) post_mem_completion(job);
+        }
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);
     }
 }

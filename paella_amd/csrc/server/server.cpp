@@ -1,6 +1,7 @@
 #include <llis/ipc/name_format.h>
 #include <llis/server/scheduler.h>
 #include <llis/server/server.h>
+#include <llis/server/phase_clock.h>
 #include <llis/utils/error.h>
 
 #include "paella_hip.h"
@@ -24,6 +25,7 @@ Server::Server(std::string server_name, Scheduler* scheduler)
 }
 
 Server::~Server() {
+    LLIS_PHASE_REPORT();
     if (const char* path = std::getenv("LLIS_EVENT_LOG")) {
         if (*path && event_log_.enabled()) event_log_.save(path);
     }
@@ -34,7 +36,10 @@ void Server::serve() {
 }
 
 void Server::poll_once() {
-    if (c2s_channel_.can_read()) handle_c2s();
+    if (c2s_channel_.can_read()) {
+        LLIS_PHASE(kRequests);
+        handle_c2s();
+    }
     scheduler_->try_handle_block_start_finish();
     if (total_owed_wakeups_ != 0 && ++polls_since_retry_ >= 64) retry_owed_wakeups();
 }
@@ -106,6 +111,7 @@ void Server::handle_launch_job() {
     JobRefId id;
     c2s_channel_.read(&id);
     if (id >= registered_jobs_.size()) throw std::runtime_error("LAUNCH_JOB for an unknown job type");
+    LLIS_PHASE_WARMUP_TICK();
     scheduler_->handle_new_job(registered_jobs_[id]->create_instance());
 }
 

@@ -133,3 +133,29 @@ def lrn(x, size, alpha, beta, k, stream=None, job_id=0, notifier=None):
     check(lib.paella_lrn_launch(_ptr(x), _ptr(y), c, x.numel() // c, size, alpha, beta, k, _stream(stream), job_id,
                                 notifier), "paella_lrn_launch")
     return y
+
+
+class DirectQueue:
+    """A user-mode hardware queue of the operator library; pass `.handle` as `stream=` to any launch."""
+
+    def __init__(self, ordered=False):
+        self.lib = _abi.ops()
+        h = ctypes.c_void_p()
+        check(self.lib.paella_direct_queue_create(ctypes.byref(h)), "paella_direct_queue_create")
+        self.handle = h.value
+        if ordered:
+            check(self.lib.paella_direct_queue_set_ordered(h, 1), "paella_direct_queue_set_ordered")
+
+    def wait(self):
+        check(self.lib.paella_direct_queue_wait(ctypes.c_void_p(self.handle)), "paella_direct_queue_wait")
+
+    def close(self):
+        if self.handle:
+            check(self.lib.paella_direct_queue_destroy(ctypes.c_void_p(self.handle)), "paella_direct_queue_destroy")
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

@@ -64,7 +64,7 @@ def test_conv_plan_arithmetic_and_rejections():
 
 
 def test_weight_packing_layout():
-    """Blob = table of (k_pad + 16) {byte offset, (r*dil)<<16 | s*dil} pairs, then weights as [k/4][m_pad][4]."""
+    """Blob = weights as [k/4][m_pad][4] with k = (c, r, s) flattened, zero padded."""
     from paella_amd import _abi
     lib = _abi.ops()
     c, h, w, k, r, s = 5, 9, 7, 6, 3, 2
@@ -74,12 +74,8 @@ def test_weight_packing_layout():
     blob = np.zeros(p.blob_bytes, np.uint8)
     assert lib.paella_conv2d_pack(ctypes.byref(p), wt.ctypes.data, blob.ctypes.data) == 0
     kdim = c * r * s
-    table = blob[:(p.k_pad + 16) * 8].view(np.int32).reshape(-1, 2)
-    for kk in range(kdim):
-        cc, rr, ss = kk // (r * s), (kk // s) % r, kk % s
-        assert table[kk, 0] == 4 * (cc * h * w + rr * 2 * w + ss) and table[kk, 1] == ((rr * 2) << 16 | ss)
-    assert np.all(table[kdim:, 1] == 0x7FFF0000)
-    packed = blob[(p.k_pad + 16) * 8:].view(np.float32).reshape(p.k_pad // 4, p.m_pad, 4)
+    assert p.blob_bytes == p.k_pad * p.m_pad * 4
+    packed = blob.view(np.float32).reshape(p.k_pad // 4, p.m_pad, 4)
     flat = wt.reshape(k, kdim)
     for m in range(k):
         for kk in range(kdim):
