@@ -90,7 +90,7 @@ struct Frag {
 #define PAELLA_CONV_ABLATE 0
 #endif
 #ifndef PAELLA_CONV_DEPTH
-#define PAELLA_CONV_DEPTH 8
+#define PAELLA_CONV_DEPTH 4
 #endif
 #ifndef PAELLA_CONV_MINB
 #define PAELLA_CONV_MINB 1
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     }
 
     // Software pipeline of depth D: D chunks of operands are in flight per wave; each slot is refilled with
-    // the chunk D ahead right after it has been consumed.  With the small tile a wave's whole slice of a
-    // typical layer (8 to 10 chunks) is requested up front.
+    // the chunk D ahead right after it has been consumed.  (Depth 8 was measured too: no faster alone, slower
+    // with several kernels in flight because of the registers it takes.)
     constexpr int D = (MI * NI == 1) ? PAELLA_CONV_DEPTH : 4;
     if (c_begin < c_end) {
         Frag<MI, NI> frag[D];
@@ -491,6 +491,9 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         }
         // Grid-level split of the reduction: layers with few output tiles (small feature maps) would otherwise
         // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU, keep >= 4 chunks per wave.
+        // (Measured alternative: about 18 chunks per wave and half as many workgroups runs 15 to 20 % faster
+        // when many kernels are in flight, but 13 to 27 % slower alone; served throughput was the same within
+        // 2 %, so the choice that is faster alone stays.)
         const int n_tiles = tiles(mi, ni);
         int splits = 1;
         if (tile_hint > 0) {
