@@ -33,6 +33,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+# HBM-side bytes per conv launch (mean over the conv launches of one forward pass), from the FETCH_SIZE / WRITE_SIZE
+# counter passes of `bench.py --roofline-only` scaled by the copy-kernel calibration (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0);
+# counters cannot be collected from inside this process, so the figure is carried here and is null for other models.
+CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 5.53e6}
+
+
 def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2):
     name = "bench%d_%s_%d" % (os.getpid(), sched, int(time.time() * 1000) % 100000)
     with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4, extra_kernels=extra_kernels) as srv:
@@ -124,6 +130,8 @@ def main():
     ap.add_argument("--extra-kernels", type=int, default=16, help="full3: kernels admitted beyond the occupancy budget")
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the plain copy kernel over a 64 MiB buffer five times (reference point for memory-traffic counters)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the isolated per-launch timing of one forward pass (the leg roofline.achieved comes from); value is null")
     args = ap.parse_args()
@@ -135,6 +143,17 @@ def main():
     hip = _abi.hip()
     _abi.ops()
     serve.lib()
+    if args.copy_calibration:
+        import torch
+        n = 16 << 20  # floats: 64 MiB read + 64 MiB written per launch
+        x = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        y = torch.empty_like(x)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            _abi.check(_abi.ops().paella_copy_launch(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(y.data_ptr()), n, None, 0, None), "copy")
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"launches": 5, "kib_read_per_launch": n * 4 / 1024, "kib_written_per_launch": n * 4 / 1024}}), flush=True)
+        return
     os.environ.setdefault("LLIS_MODEL_SEED", "1")
     job = serve.job_path("tvm_" + {"mobilenetv2": "mobilenet"}.get(args.model, args.model))
     jobs = [(job, 1.0, args.concurrency)]
@@ -182,7 +201,7 @@ def main():
     rl = conv_roofline(models, hip, args.model, reps=50)
     achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-                "traffic": None, "kernel": "conv_mfma_kernel (all %d conv launches of one %s forward pass)" % (rl["conv_launches"], args.model),
+                "traffic": CONV_TRAFFIC_BYTES_PER_LAUNCH.get(args.model), "kernel": "conv_mfma_kernel (all %d conv launches of one %s forward pass)" % (rl["conv_launches"], args.model),
                 "flops_per_launch_avg": rl["conv_flops"] / rl["conv_launches"], "us_per_launch_avg": rl["conv_us"] / rl["conv_launches"]}
     log("[bench]   conv: %.2f TFLOP/s (%.1f%% of fp32 MFMA peak), forward %.0f us, direct loop %.0f req/s" %
         (achieved, 100 * roofline["frac"], rl["forward_us"], rl["direct_rps"]))

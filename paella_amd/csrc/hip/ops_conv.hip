@@ -19,6 +19,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "paella_ops.h"
@@ -34,7 +35,7 @@ __device__ unsigned long long g_conv_timeline[8192 * 12];
 #define CONV_TL(i)                                                                                        \
     do {                                                                                                  \
         if (threadIdx.x == 0) {                                                                           \
-            const unsigned b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;           \
+            const unsigned b_ = blockIdx.x;                                                               \
             if (b_ < 8192) g_conv_timeline[b_ * 12 + (i)] = wall_clock64();                               \
         }                                                                                                 \
     } while (0)
@@ -58,7 +59,9 @@ struct ConvArgs {
     int K, m_pad, nchunks;
     int kdim, RS, S, dh, dw;        // reduction length C*R*S, filter plane R*S, filter width, dilations
     unsigned w_bytes;               // size of the packed weights
-    int splits, chunks_per_split;   // grid-level split of the reduction (gridDim.z == splits)
+    int splits, chunks_per_split;   // grid-level split of the reduction
+    int n_tiles_n, n_tiles_m;       // output tiles along pixels and along channels; the grid is 1-D over n*m*splits
+    int slab_major;                 // which workgroups share an XCD: 1 = same weights, 0 = neighbouring pixels
     float* ws_partials;             // [tile][split][NACC][64] partial tiles (request-private workspace)
     unsigned* ws_counters;          // [tile] arrival counters, zero between launches
     unsigned x_bytes;
@@ -111,8 +114,31 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     const int wave = threadIdx.x >> 6;
     const int j = lane & 31;
     const int kk = lane >> 5;
-    const int m0 = blockIdx.y * (32 * MI);
-    const int n0 = blockIdx.x * (32 * NI);
+    // Workgroup -> (pixel tile, channel tile, reduction split).  Workgroup ids go round-robin over the eight
+    // XCDs, each with its own L2; the ids that land on one XCD are given a contiguous run of the work list, and
+    // the list is ordered so that a run shares what the layer reads most of: the same slab of weights (layers
+    // with small feature maps) or neighbouring pixel tiles, whose 3x3 halos overlap (layers with large ones).
+    int tile_n, tile_m, split;
+    {
+        const unsigned total = (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits);
+        const unsigned xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+        const unsigned q = total >> 3, r = total & 7u;
+        const unsigned w = p.slab_major == 2 ? blockIdx.x : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
+        if (p.slab_major) {
+            const unsigned slab = w / (unsigned)p.n_tiles_n;
+            tile_n = (int)(w - slab * (unsigned)p.n_tiles_n);
+            split = (int)(slab / (unsigned)p.n_tiles_m);
+            tile_m = (int)(slab - (unsigned)split * (unsigned)p.n_tiles_m);
+        } else {
+            const unsigned per_n = (unsigned)(p.n_tiles_m * p.splits);
+            tile_n = (int)(w / per_n);
+            const unsigned rest = w - (unsigned)tile_n * per_n;
+            split = (int)(rest / (unsigned)p.n_tiles_m);
+            tile_m = (int)(rest - (unsigned)split * (unsigned)p.n_tiles_m);
+        }
+    }
+    const int m0 = tile_m * (32 * MI);
+    const int n0 = tile_n * (32 * NI);
 
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, p.x_bytes, 0x00027000);
 
@@ -128,7 +154,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     }
 
     // Reduction range of this workgroup (grid-level split), then of this wave inside it.
-    const int g_begin = blockIdx.z * p.chunks_per_split;
+    const int g_begin = split * p.chunks_per_split;
     const int g_end = min(p.nchunks, g_begin + p.chunks_per_split);
     const int cpw = (g_end - g_begin + KW - 1) / KW;
     const int c_begin = g_begin + wave * cpw;
@@ -325,8 +351,8 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
         // Deterministic split-k: every workgroup parks its partial tile in the workspace (write-through),
         // bumps the tile's counter, and the workgroup that arrives last adds the partials in split order and
         // runs the epilogue.  The counter is left at zero for the next launch.
-        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-        float* part = p.ws_partials + ((size_t)tile * p.splits + blockIdx.z) * (NACC * 64);
+        const int tile = tile_m * p.n_tiles_n + tile_n;
+        float* part = p.ws_partials + ((size_t)tile * p.splits + split) * (NACC * 64);
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) store_out(part + (wave * RPW + rr) * 64 + lane, mine[rr]);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -593,7 +619,12 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
         a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
         a.job_id = job_id;
         a.notifier = nf;
-        dim3 grid((PQ + 32 * plan->ni - 1) / (32 * plan->ni), plan->m_pad / (32 * plan->mi), plan->splits);
+        a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
+        a.n_tiles_m = plan->m_pad / (32 * plan->mi);
+        // Weights outweigh the input: keep the workgroups that read one slab of weights on one XCD.
+        a.slab_major = (double)d.K * d.C * d.R * d.S > (double)d.C * d.H * d.W ? 1 : 0;
+        if (const char* force = std::getenv("PAELLA_CONV_ORDER")) a.slab_major = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : a.slab_major));
+        dim3 grid((unsigned)(a.n_tiles_n * a.n_tiles_m * plan->splits), 1, 1);
         if (plan->dims.lds_bytes > 65536) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->dims.lds_bytes);
             if (e != hipSuccess) return (int)e;
