@@ -130,6 +130,7 @@ def main():
     ap.add_argument("--extra-kernels", type=int, default=16, help="full3: kernels admitted beyond the occupancy budget")
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-mix", action="store_true", help="skip the small-CNN + Inception-v3 two-tenant arm")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel over a 64 MiB buffer five times (reference point for memory-traffic counters)")
     ap.add_argument("--roofline-only", action="store_true",
@@ -197,6 +198,30 @@ def main():
             sweep.append(point)
             log("[bench]   poisson %.0f req/s: full3 p99 %.0f us, fifo p99 %.0f us" % (rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"]))
 
+    # The two-tenant mix of the target statement: small CNN : Inception-v3 (299x299) = 9 : 1, full3 against plain
+    # multi-stream serving (fifo), first at saturation, then open-loop Poisson at fractions of the lower of the two.
+    mix = None
+    if not args.no_arms and not args.no_mix:
+        mix_jobs = [(serve.job_path("tvm_mnist"), 0.9, args.concurrency), (serve.job_path("tvm_inception_v3"), 0.1, args.concurrency)]
+        n_mix = 3000
+        sat = {}
+        for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+            r = serve_arm(serve, sched, streams, mix_jobs, args.concurrency, n_mix, 300, extra_kernels=args.extra_kernels)
+            sat[label] = r["throughput_rps"]
+        mix = {"workload": "small CNN : Inception-v3 = 9 : 1, inputs resident", "saturation_rps": sat, "poisson": []}
+        log("[bench]   mix saturation: full3 %.0f req/s, fifo %.0f req/s" % (sat["full3"], sat["fifo_multi_stream"]))
+        for frac in (0.5, 0.8):
+            rate = frac * min(sat.values())
+            point = {"offered_rps": rate}
+            for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+                r = serve_arm(serve, sched, streams, mix_jobs, args.concurrency, n_mix, 300, iat_us=1e6 / rate, extra_kernels=args.extra_kernels)
+                point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"],
+                                "small_cnn_p99_us": r["per_type"][0]["p99"], "inception_v3_p99_us": r["per_type"][1]["p99"]}
+            mix["poisson"].append(point)
+            log("[bench]   mix poisson %.0f req/s: p99 small CNN / Inception: full3 %.0f / %.0f us, fifo %.0f / %.0f us" %
+                (rate, point["full3"]["small_cnn_p99_us"], point["full3"]["inception_v3_p99_us"],
+                 point["fifo_multi_stream"]["small_cnn_p99_us"], point["fifo_multi_stream"]["inception_v3_p99_us"]))
+
     log("[bench] per-launch timing of the forward pass (kernel begin/end timestamps through HIP events)")
     rl = conv_roofline(models, hip, args.model, reps=50)
     achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
@@ -246,6 +271,7 @@ def main():
         "cpu_baseline": cpu,
         "arms": arms,
         "poisson_sweep": sweep,
+        "two_tenant_mix": mix,
         "direct_single_stream_rps": rl["direct_rps"],
         "per_op_us": {k: {"launches": v["launches"], "us": v["us"], "gflop": v["flops"] / 1e9, "mbytes": v["bytes"] / 1e6} for k, v in rl["by_op"].items()},
         "notify_us": notify,
