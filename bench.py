@@ -230,6 +230,9 @@ def main():
                 "flops_per_launch_avg": rl["conv_flops"] / rl["conv_launches"], "us_per_launch_avg": rl["conv_us"] / rl["conv_launches"]}
     log("[bench]   conv: %.2f TFLOP/s (%.1f%% of fp32 MFMA peak), forward %.0f us, direct loop %.0f req/s" %
         (achieved, 100 * roofline["frac"], rl["forward_us"], rl["direct_rps"]))
+    for op, v in rl["by_op"].items():
+        log("[bench]     %-8s %3d launches %8.1f us  %7.3f GFLOP %8.2f MB  -> %6.2f TFLOP/s %7.1f GB/s" %
+            (op, v["launches"], v["us"], v["flops"] / 1e9, v["bytes"] / 1e6, v["flops"] / (v["us"] * 1e-6) / 1e12, v["bytes"] / (v["us"] * 1e-6) / 1e9))
 
     ring = ctypes.c_void_p()
     lib = _abi.ops()
@@ -273,7 +276,10 @@ def main():
         "poisson_sweep": sweep,
         "two_tenant_mix": mix,
         "direct_single_stream_rps": rl["direct_rps"],
-        "per_op_us": {k: {"launches": v["launches"], "us": v["us"], "gflop": v["flops"] / 1e9, "mbytes": v["bytes"] / 1e6} for k, v in rl["by_op"].items()},
+        # per operator family, one forward pass, isolated launches: time, algorithmic work, and the rates they imply
+        "per_op_us": {k: {"launches": v["launches"], "us": v["us"], "gflop": v["flops"] / 1e9, "mbytes": v["bytes"] / 1e6,
+                          "tflops": v["flops"] / (v["us"] * 1e-6) / 1e12 if v["us"] else None,
+                          "gbytes_per_s": v["bytes"] / (v["us"] * 1e-6) / 1e9 if v["us"] else None} for k, v in rl["by_op"].items()},
         "notify_us": notify,
     }
     print(json.dumps(out), flush=True)

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs p) {
             r.y = elt_one(p, a.y, b.y, c);
             r.z = elt_one(p, a.z, b.z, c);
             r.w = elt_one(p, a.w, b.w, c);
-            store_out4(p.y + i4 * 4, r);
+            store_out4(p.y, i4 * 4, r);
         }
     } else {
         const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -192,8 +192,8 @@ __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ x, 
                                                    uint32_t job_id, Notifier* notifier) {
     if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i + 3 < n && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
-        store_out4(y + i, *reinterpret_cast<const float4*>(x + i));
+    if (i + 3 < n && n < ((size_t)1 << 30) && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
+        store_out4(y, i, *reinterpret_cast<const float4*>(x + i));
     } else {
         for (size_t k = i; k < n && k < i + 4; ++k) store_out(y + k, x[k]);
     }
@@ -348,7 +348,7 @@ int paella_eltwise_launch(const float* a, const float* b, const float* scale, co
     p.job_id = job_id; p.notifier = (Notifier*)notifier;
     const size_t n = (size_t)C * HW;
     const bool aligned = ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) == 0);
-    if ((HW & 3) == 0 && aligned) {
+    if ((HW & 3) == 0 && aligned && n < ((size_t)1 << 30)) {
         paella::launch(eltwise_kernel<true>, dim3(blocks_for(n / 4, 256)), dim3(256), 0, (hipStream_t)stream, p);
     } else {
         paella::launch(eltwise_kernel<false>, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, p);

@@ -10,9 +10,13 @@
 
 __device__ __forceinline__ void store_out(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-__device__ __forceinline__ void store_out4(float* p, const float4& v) {
-    store_out(p + 0, v.x);
-    store_out(p + 1, v.y);
-    store_out(p + 2, v.z);
-    store_out(p + 3, v.w);
+// Four consecutive floats at base[index .. index+3] (16-byte aligned) as ONE 16-byte write-through store.  Four
+// separate dword stores per lane would be 16 bytes apart across lanes: sixteen partial-line writes per
+// instruction instead of full lines.  `base` must be uniform over the wave; index * 4 must fit 32 bits.
+__device__ __forceinline__ void store_out4(float* base, size_t index, const float4& v) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xFFFFFFFFu, 0x00027000);
+    const u32x4 bits = {__builtin_bit_cast(unsigned, v.x), __builtin_bit_cast(unsigned, v.y), __builtin_bit_cast(unsigned, v.z),
+                        __builtin_bit_cast(unsigned, v.w)};
+    __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc, (int)(unsigned)(index * 4), 0, 16 /* sc1: write through */);
 }
