@@ -159,6 +159,8 @@ def main():
     job = serve.job_path("tvm_" + {"mobilenetv2": "mobilenet"}.get(args.model, args.model))
     jobs = [(job, 1.0, args.concurrency)]
     tot = models.totals(args.model)
+    in_bytes = models.io_bytes(args.model)[0]
+    in_shape = {602112: "1x3x224x224", 3136: "1x1x28x28", 1072812: "1x3x299x299", 921600: "1x3x240x320", 150528: "1x3x112x112"}.get(in_bytes, "%d input bytes" % in_bytes)
 
     log("[bench] timed arm: full3, %d streams, concurrency %d, %d warm-up + %d timed requests" % (args.num_streams, args.concurrency, args.warmup, args.steps))
     # The timed arm and its comparison arms serve requests whose input already sits in device memory (the job
@@ -262,8 +264,8 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "%s batch 1 fp32 1x3x224x224, seeded weights, inputs resident in device memory, full3 scheduler, %d streams, "
-                               "saturation with %d outstanding requests" % (args.model, args.num_streams, args.concurrency),
+        "config": {"workload": "%s batch 1 fp32 %s, seeded weights, inputs resident in device memory, full3 scheduler, %d streams, "
+                               "saturation with %d outstanding requests" % (args.model, in_shape, args.num_streams, args.concurrency),
                    "gmac_per_request": tot["macs"] / 1e9, "stages_per_request": tot["stages"] + 1},
         "pcie_inclusive_requests_per_s": pcie_inclusive,
         # open-loop latency at 80 % of the saturation rate; at saturation every request is submitted at t = 0 and

@@ -65,6 +65,7 @@ typedef struct paella_conv_plan {
     int mi, ni, kw;              /* per-wave tile = (32*mi) x (32*ni) outputs, kw waves split the reduction */
     int splits;                  /* workgroups per output tile that split the reduction further (grid z) */
     int m_pad, k_pad;            /* padded GEMM dims of the packed weight blob */
+    int k_order;                 /* reduction order of the blob: 0 = (c, r, s), 1 = (r, s, c) (chosen when C % 8 == 0) */
     size_t blob_bytes;           /* size of the packed weight blob */
     size_t workspace_bytes;      /* per-request scratch for splits > 1 (0 otherwise); must start out zeroed */
     paella_launch_dims dims;

@@ -14,7 +14,11 @@
 //   * the im2col operand is gathered straight from the activation tensor with raw buffer loads whose
 //     out-of-range offsets return 0: padding taps, the k tail and the pixel tail need no branches.  Each
 //     workgroup first builds, in LDS, the table k -> {byte offset c*H*W + r*dil*W + s*dil, (r*dil) << 16 | (s*dil)}
-//     for its slice of the reduction.
+//     for its slice of the reduction;
+//   * when C is a multiple of 8 the reduction index is ordered k = (r, s, c) instead ("tap-major"): the 8 values
+//     of a chunk then share one filter tap and differ only in the channel, so the address is a few additions on
+//     wave-uniform running counters, the bounds test is done once per chunk instead of once per value, and
+//     neither table nor LDS staging nor the barrier after it is needed: the first loads leave right away.
 
 #include <hip/hip_runtime.h>
 
@@ -58,6 +62,7 @@ struct ConvArgs {
     int sh, sw, ph, pw;
     int K, m_pad, nchunks;
     int kdim, RS, S, dh, dw;        // reduction length C*R*S, filter plane R*S, filter width, dilations
+    int CB;                         // tap-major order only: chunks per filter tap (C / 8)
     unsigned w_bytes;               // size of the packed weights
     int splits, chunks_per_split;   // grid-level split of the reduction
     int n_tiles_n, n_tiles_m;       // output tiles along pixels and along channels; the grid is 1-D over n*m*splits
@@ -99,7 +104,7 @@ struct Frag {
 #define PAELLA_CONV_MINB 1
 #endif
 
-template <int MI, int NI, int KW>
+template <int MI, int NI, int KW, bool TAP_MAJOR>
 __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
     CONV_TL(0);
     if (PAELLA_CONV_ABLATE & 16) return;
@@ -111,7 +116,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     float* red = reinterpret_cast<float*>(smem);
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and the compiler may know it
     const int j = lane & 31;
     const int kk = lane >> 5;
     // Workgroup -> (pixel tile, channel tile, reduction split).  Workgroup ids go round-robin over the eight
@@ -171,16 +176,50 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     // Chunks outside [c_begin, c_end) are requested at an out-of-range offset: the loads keep their place in
     // the (static) issue order, return zeros and touch no memory.
     __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, p.w_bytes, 0x00027000);
+    // Tap-major order: running, wave-uniform position of the next chunk to request (load_frag is always called
+    // with consecutive chunk indices): channel block within the tap, filter row, filter column.
+    const int HW4 = p.H * p.W * 4;
+    const int kk4hw = kk * 4 * HW4;
+    int st_cb = 0, st_r = 0, st_s = 0;
+    if (TAP_MAJOR) {
+        const int tap = c_begin / p.CB;
+        st_cb = c_begin - tap * p.CB;
+        st_r = tap / p.S;
+        st_s = tap - st_r * p.S;
+    }
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
         if (PAELLA_CONV_ABLATE & 2) valid = false;
-        const int4* t = reinterpret_cast<const int4*>(ltab + ((valid ? c : g_begin) - g_begin) * 8 + kk * 4);
-        const int4 t0 = t[0], t1 = t[1];
         const int woff = valid ? (int)((((unsigned)(c * 2 + kk) * (unsigned)p.m_pad) + (unsigned)(m0 + j)) * 16u) : -1;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
             const auto v = __builtin_amdgcn_raw_buffer_load_b128(wres, woff, mi * 32 * 16, 0);
             f.a[mi] = __builtin_bit_cast(float4, v);
         }
+        if (TAP_MAJOR) {
+            const int dy = st_r * p.dh, dx = st_s * p.dw;
+            const int chunk_off = (dy * p.W + dx) * 4 + st_cb * 8 * HW4;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int h = hb[ni] + dy;
+                const int w = wb[ni] + dx;
+                const bool ok = valid & ((unsigned)h < (unsigned)p.H) & ((unsigned)w < (unsigned)p.W);
+                const int voff = ok ? base[ni] + chunk_off + kk4hw : -1;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)  // the channel step rides in the scalar offset, which is not range-checked:
+                                             // an out-of-range voff stays out of range, a valid one stays valid
+                    f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, voff, t * HW4, 0));
+            }
+            if (++st_cb == p.CB) {
+                st_cb = 0;
+                if (++st_s == p.S) {
+                    st_s = 0;
+                    ++st_r;
+                }
+            }
+            return;
+        }
+        const int4* t = reinterpret_cast<const int4*>(ltab + ((valid ? c : g_begin) - g_begin) * 8 + kk * 4);
+        const int4 t0 = t[0], t1 = t[1];
         const int off[4] = {t0.x, t0.z, t1.x, t1.z};
         const int rs[4] = {t0.y, t0.w, t1.y, t1.w};
 #pragma unroll
@@ -197,9 +236,8 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     };
 
     // Build this workgroup's slice of the k -> offset table in LDS (a few entries per thread, arithmetic only).
-    {
+    if (!TAP_MAJOR) {
         const int n_entries = (g_end - g_begin) * 8;
-        const int HW4 = p.H * p.W * 4;
         for (int i = threadIdx.x; i < ((PAELLA_CONV_ABLATE & 8) ? 0 : n_entries); i += 64 * KW) {
             const int k = g_begin * 8 + i;
             const int c = k / p.RS;
@@ -212,8 +250,8 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
             if (k >= p.kdim) e = make_int2(0, 0x7FFF0000);  // row far outside the image: the tap reads as zero
             ltab[i] = e;
         }
+        __syncthreads();
     }
-    __syncthreads();
     // Drain every earlier vector-memory operation (the start hook's store among them) once, here: with a
     // store still pending the compiler must assume out-of-order completion and would make every wait in
     // the pipelined loop below a full vmcnt(0).
@@ -321,7 +359,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
                 for (int e = 0; e < 16; ++e)
                     if ((mi * NI + ni) * 16 + e < RPW) mine[(mi * NI + ni) * 16 + e] = acc[mi][ni][e];
     } else {
-        __syncthreads();  // every wave is done with the table before the partial tiles overwrite it
+        if (!TAP_MAJOR) __syncthreads();  // every wave is done with the table before the partial tiles overwrite it
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -444,24 +482,27 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
 
 typedef void (*ConvKernel)(ConvArgs);
 
-template <int MI, int NI>
+template <int MI, int NI, bool TM>
 ConvKernel pick_kw(int kw) {
     switch (kw) {
-        case 1: return conv_mfma_kernel<MI, NI, 1>;
-        case 2: return conv_mfma_kernel<MI, NI, 2>;
-        case 4: return conv_mfma_kernel<MI, NI, 4>;
-        case 8: return conv_mfma_kernel<MI, NI, 8>;
+        case 1: return conv_mfma_kernel<MI, NI, 1, TM>;
+        case 2: return conv_mfma_kernel<MI, NI, 2, TM>;
+        case 4: return conv_mfma_kernel<MI, NI, 4, TM>;
+        case 8: return conv_mfma_kernel<MI, NI, 8, TM>;
         default: return nullptr;
     }
 }
 
-ConvKernel pick_kernel(int mi, int ni, int kw) {
-    if (mi == 1 && ni == 1) return pick_kw<1, 1>(kw);
-    if (mi == 1 && ni == 2) return pick_kw<1, 2>(kw);
-    if (mi == 2 && ni == 1) return pick_kw<2, 1>(kw);
-    if (mi == 2 && ni == 2) return pick_kw<2, 2>(kw);
+template <bool TM>
+ConvKernel pick_tile(int mi, int ni, int kw) {
+    if (mi == 1 && ni == 1) return pick_kw<1, 1, TM>(kw);
+    if (mi == 1 && ni == 2) return pick_kw<1, 2, TM>(kw);
+    if (mi == 2 && ni == 1) return pick_kw<2, 1, TM>(kw);
+    if (mi == 2 && ni == 2) return pick_kw<2, 2, TM>(kw);
     return nullptr;
 }
+
+ConvKernel pick_kernel(int mi, int ni, int kw, int k_order = 0) { return k_order ? pick_tile<true>(mi, ni, kw) : pick_tile<false>(mi, ni, kw); }
 
 constexpr size_t kMaxSplitTiles = 16384;  // counters at the head of a split-k workspace
 
@@ -535,6 +576,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->splits = splits;
         plan->m_pad = round_up(d->K, 32 * mi);
         plan->k_pad = k_pad;
+        // Reduction order: (r, s, c) when whole chunks of 8 share a filter tap, else (c, r, s) with the offset table.
+        plan->k_order = (d->C % 8 == 0 && !std::getenv("PAELLA_CONV_NO_TAP_MAJOR")) ? 1 : 0;
         plan->blob_bytes = (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
         if (plan->blob_bytes >= ((size_t)1 << 31)) return PAELLA_ENOSUP;  // weights are addressed with 32-bit byte offsets
         // Workspace = fixed-size counter area (so that stages of one request, which share the workspace, never
@@ -545,7 +588,7 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->dims.block = 64u * kw;
         {
             const unsigned red_bytes = kw > 1 ? (unsigned)(kw * mi * ni * 16 * 64 * sizeof(float)) : 0u;
-            const unsigned tab_bytes = (unsigned)(chunks_per_split * 8 * sizeof(int2));
+            const unsigned tab_bytes = plan->k_order ? 0u : (unsigned)(chunks_per_split * 8 * sizeof(int2));
             plan->dims.lds_bytes = red_bytes > tab_bytes ? red_bytes : tab_bytes;
             if (plan->dims.lds_bytes > 160 * 1024) return PAELLA_ENOSUP;  // table does not fit the CU's LDS
         }
@@ -574,8 +617,12 @@ extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, 
     const int kdim = d.C * d.R * d.S;
     float* wp = reinterpret_cast<float*>(blob_host);
     std::memset(wp, 0, (size_t)(plan->k_pad / 4) * plan->m_pad * sizeof(float4));
+    const int RS = d.R * d.S;
     for (int m = 0; m < d.K; ++m)
-        for (int k = 0; k < kdim; ++k) wp[((size_t)(k / 4) * plan->m_pad + m) * 4 + (k % 4)] = w[(size_t)m * kdim + k];
+        for (int k = 0; k < kdim; ++k) {  // k indexes the source in (c, r, s) order
+            const int kp = plan->k_order ? (k % RS) * d.C + k / RS : k;  // position in the kernel's reduction order
+            wp[((size_t)(kp / 4) * plan->m_pad + m) * 4 + (kp % 4)] = w[(size_t)m * kdim + k];
+        }
     return 0;
 }
 
@@ -589,13 +636,14 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
     const int PQ = plan->P * plan->Q;
     if (plan->kind == 0) {
-        ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw);
+        ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order);
         if (!kern) return PAELLA_EINVAL;
         ConvArgs a;
         a.x = x;
         a.wpk = reinterpret_cast<const float4*>(blob_dev);
         a.w_bytes = (unsigned)plan->blob_bytes;
         a.kdim = d.C * d.R * d.S; a.RS = d.R * d.S; a.S = d.S; a.dh = d.dil_h; a.dw = d.dil_w;
+        a.CB = d.C / 8;
         a.bias = bias;
         a.residual = residual;
         a.slope = slope;
@@ -645,6 +693,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
 }
 
 extern "C" int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs) {
+    // the tap-major twin of a variant uses no more registers than the table variant reported here
     const void* fn = kind == 1 ? reinterpret_cast<const void*>(dwconv_kernel) : reinterpret_cast<const void*>(pick_kernel(mi, ni, kw));
     if (!fn || !vgprs) return PAELLA_EINVAL;
     hipFuncAttributes attr;

@@ -69,7 +69,7 @@ def test_weight_packing_layout():
     lib = _abi.ops()
     c, h, w, k, r, s = 5, 9, 7, 6, 3, 2
     rc, p = plan((c, h, w, k, r, s, 1, 1, 1, 0, 2, 1, 1, 0, 0, 0))
-    assert rc == 0
+    assert rc == 0 and p.k_order == 0
     wt = np.arange(k * c * r * s, dtype=np.float32).reshape(k, c, r, s)
     blob = np.zeros(p.blob_bytes, np.uint8)
     assert lib.paella_conv2d_pack(ctypes.byref(p), wt.ctypes.data, blob.ctypes.data) == 0
@@ -81,6 +81,25 @@ def test_weight_packing_layout():
         for kk in range(kdim):
             assert packed[kk // 4, m, kk % 4] == flat[m, kk]
     assert packed[:, k:, :].sum() == 0 and packed.reshape(-1).sum() == flat.sum()
+
+
+def test_weight_packing_layout_tap_major():
+    """C % 8 == 0: the blob's reduction index runs (r, s, c), so a chunk of 8 shares one filter tap."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+    c, h, w, k, r, s = 16, 9, 7, 6, 3, 2
+    rc, p = plan((c, h, w, k, r, s, 1, 1, 1, 0, 1, 1, 1, 0, 0, 0))
+    assert rc == 0 and p.k_order == 1 and p.k_pad == c * r * s
+    wt = np.random.default_rng(1).standard_normal((k, c, r, s)).astype(np.float32)
+    blob = np.zeros(p.blob_bytes, np.uint8)
+    assert lib.paella_conv2d_pack(ctypes.byref(p), wt.ctypes.data, blob.ctypes.data) == 0
+    packed = blob.view(np.float32).reshape(p.k_pad // 4, p.m_pad, 4)
+    for m in range(k):
+        for cc in range(c):
+            for rr in range(r):
+                for ss in range(s):
+                    kp = (rr * s + ss) * c + cc
+                    assert packed[kp // 4, m, kp % 4] == wt[m, cc, rr, ss]
 
 
 def test_pool_out_matches_oracle():
