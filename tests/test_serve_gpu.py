@@ -48,6 +48,30 @@ def test_request_output_through_the_server_matches_oracle(cuda, sched_name, mode
     close(out, ref)
 
 
+@pytest.mark.parametrize("dispatch", ["hip", "direct"])
+def test_resident_input_mode_and_both_dispatch_paths_match_oracle(cuda, dispatch):
+    """Measurement mode (input uploaded once per instance, no host-to-device stage) and the HIP-launch fallback of
+    the model adapters must give the same answers as the default path."""
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    desc = models.describe("resnet18")
+    x = om.make_input(desc, 5, "normal")
+    ref = om.run(desc, x, seed=1)
+    old = {k: os.environ.get(k) for k in ("PAELLA_INPUT_RESIDENT", "PAELLA_DISPATCH")}
+    os.environ["PAELLA_INPUT_RESIDENT"] = "1"
+    os.environ["PAELLA_DISPATCH"] = dispatch
+    try:
+        with serve.Server(server_name("res" + dispatch), "full3", num_streams=8) as srv:
+            out, lat = serve.client_single(srv.name, serve.job_path("tvm_resnet18"), x, ref.size, n=4)
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    close(out, ref)
+
+
 @pytest.mark.parametrize("mem_marker", [True, False])
 def test_both_copy_completion_paths_on_the_gpu(cuda, mem_marker):
     from paella_amd import serve
