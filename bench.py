@@ -236,8 +236,12 @@ def main():
         log("[bench]     %-8s %3d launches %8.1f us  %7.3f GFLOP %8.2f MB  -> %6.2f TFLOP/s %7.1f GB/s" %
             (op, v["launches"], v["us"], v["flops"] / 1e9, v["bytes"] / 1e6, v["flops"] / (v["us"] * 1e-6) / 1e12, v["bytes"] / (v["us"] * 1e-6) / 1e9))
 
-    ring = ctypes.c_void_p()
     lib = _abi.ops()
+    peak = ctypes.c_double()
+    if lib.paella_mfma_peak_probe(ctypes.byref(peak)) == 0:
+        roofline["peak_measured"] = peak.value  # register-resident fp32 MFMA loop on this box; `peak` stays the published figure
+        log("[bench]   fp32 MFMA rate measured with a register-resident loop: %.1f TFLOP/s" % peak.value)
+    ring = ctypes.c_void_p()
     notify = {}
     if not args.roofline_only and lib.paella_ring_create(1024000, 1, ctypes.byref(ring)) == 0:
         us = ctypes.c_double()

@@ -52,6 +52,10 @@ int paella_ring_bench_drain(paella_ring* ring, unsigned blocks, unsigned vec_len
                             double* us_per_iter);
 int paella_ring_bench_pingpong(int warmup, int iters, double* flag_us, double* sync_us, double* flag_samples_us);
 
+/* Sustained fp32 MFMA rate of the device (v_mfma_f32_32x32x2_f32, register-resident operands, every SIMD busy):
+ * the measured denominator next to the published 157.3 TFLOP/s. */
+int paella_mfma_peak_probe(double* tflops);
+
 #ifdef __cplusplus
 }
 #endif

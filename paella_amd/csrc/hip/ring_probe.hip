@@ -63,6 +63,22 @@ __global__ void drain_bench_kernel(float* out, const float* in, unsigned count, 
 
 __global__ void empty_kernel() {}
 
+// Register-resident fp32 MFMA loop: four independent accumulator chains per wave, no memory traffic.
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void mfma_peak_kernel(float* sink, int iters) {
+    probe_f32x16 acc0 = {0}, acc1 = {0}, acc2 = {0}, acc3 = {0};
+    float a = 1.0f + threadIdx.x * 1e-6f, b = 1.0f - threadIdx.x * 1e-6f;
+    for (int i = 0; i < iters; ++i) {
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(b, a, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, a, acc2, 0, 0, 0);
+        acc3 = __builtin_amdgcn_mfma_f32_32x32x2f32(b, b, acc3, 0, 0, 0);
+    }
+    float v = 0.f;
+    for (int e = 0; e < 16; ++e) v += acc0[e] + acc1[e] + acc2[e] + acc3[e];
+    if (v == 123.456f) sink[0] = v;  // keeps the loop alive without a store in practice
+}
+
 __global__ void flag_kernel(int* flag) { __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM); }
 
 double now_us() {
@@ -202,6 +218,37 @@ int paella_ring_bench_pingpong(int warmup, int iters, double* flag_us, double* s
     hipStreamSynchronize(st);
     hipStreamDestroy(st);
     llis_hip_host_free(flag);
+    return 0;
+}
+
+int paella_mfma_peak_probe(double* tflops) {
+    if (!tflops) return -1;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, 0);
+    if (e != hipSuccess) return (int)e;
+    float* sink = nullptr;
+    e = hipMalloc(&sink, 64);
+    if (e != hipSuccess) return (int)e;
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    const int iters = 20000;
+    const unsigned blocks = (unsigned)prop.multiProcessorCount * 2;  // 8 waves per CU: two per SIMD
+    double best = 0;
+    for (int rep = 0; rep < 3; ++rep) {
+        hipEventRecord(e0, nullptr);
+        hipLaunchKernelGGL(mfma_peak_kernel, dim3(blocks), dim3(256), 0, nullptr, sink, iters);
+        hipEventRecord(e1, nullptr);
+        hipEventSynchronize(e1);
+        float ms = 0;
+        hipEventElapsedTime(&ms, e0, e1);
+        const double flops = (double)blocks * 4 /*waves*/ * iters * 4 /*mfma*/ * 4096.0;
+        if (ms > 0 && flops / (ms * 1e-3) / 1e12 > best) best = flops / (ms * 1e-3) / 1e12;
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    hipFree(sink);
+    *tflops = best;
     return 0;
 }
 
