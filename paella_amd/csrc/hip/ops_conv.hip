@@ -98,7 +98,7 @@ struct Frag {
 #define PAELLA_CONV_ABLATE 0
 #endif
 #ifndef PAELLA_CONV_DEPTH
-#define PAELLA_CONV_DEPTH 4
+#define PAELLA_CONV_DEPTH 2
 #endif
 #ifndef PAELLA_CONV_MINB
 #define PAELLA_CONV_MINB 1
@@ -285,8 +285,10 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     }
 
     // Software pipeline of depth D: D chunks of operands are in flight per wave; each slot is refilled with
-    // the chunk D ahead right after it has been consumed.  (Depth 8 was measured too: no faster alone, slower
-    // with several kernels in flight because of the registers it takes.)
+    // the chunk D ahead right after it has been consumed.  Shallow is better here: the small tile measured
+    // fastest at depth 2, alone (6.1 us for the 64-channel 56x56 layer against 6.4 at depth 4) and with many
+    // kernels in flight (2.4 against 2.7 us per kernel): fewer registers, so four workgroups fit a CU, and other
+    // waves hide the latency that a deeper pipeline would.
     constexpr int D = (MI * NI == 1) ? PAELLA_CONV_DEPTH : 4;
     if (c_begin < c_end) {
         Frag<MI, NI> frag[D];
