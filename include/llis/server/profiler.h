@@ -1,12 +1,15 @@
 #pragma once
 // Server-side recorder behind the PROFILER_CMD messages.  The wire protocol (sub-command enum, SAVE
 // carrying a path prefix) follows reference src/server/profiler.cpp:10-67 so a client's ProfilerClient
-// keeps working; recording covers kernel info and per-job event timelines, written on SAVE as
-// <prefix>_kernel_info.txt and <prefix>_job_events.txt in the reference's line formats
-// (reference src/server/profiler.cpp:76-131).  The other four files are created empty.
+// keeps working; recording covers kernel info, per-job event timelines, run_next() times and resource events,
+// written on SAVE as <prefix>_kernel_info.txt, _job_events.txt, _run_next_times.txt and _resource_events.txt in
+// the reference's line formats (reference src/server/profiler.cpp:76-131).  _block_exec_times.txt (needs the
+// optional per-block timing ring) and _kernel_block_mis_alloc.txt (written only by schedulers the reference
+// does not build) are created empty.
 
 #include <llis/ipc/defs.h>
 #include <llis/ipc/shm_channel.h>
+#include <llis/job/job.h>
 
 #include <chrono>
 #include <string>
@@ -22,6 +25,7 @@ class Profiler {
     using TimePoint = std::chrono::steady_clock::time_point;
 
     enum class JobEvent { JOB_SUBMITTED, KERNEL_SCHED_START, KERNEL_SCHED_ABORT, KERNEL_SUBMIT_START, KERNEL_SUBMIT_END, KERNEL_FINISHED, JOB_FINISHED };
+    enum class ResourceEvent { ACQUIRE, RELEASE, QUEUED };
 
     explicit Profiler(ipc::ShmChannelCpuReader* c2s_channel) : c2s_channel_(c2s_channel) {}
 
@@ -35,12 +39,22 @@ class Profiler {
     void record_kernel_info(TimePoint start, TimePoint end, unsigned num_blocks, unsigned num_threads_per_block, unsigned smem_size_per_block,
                             unsigned num_registers_per_thread, double priority, unsigned job_ref_id);
     void record_job_event(JobId job_id, JobEvent event);
+    bool recording_run_next_times() const { return run_next_times_flag_; }
+    void record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks);
+    // num workgroups of the job's running stage acquired or released (reference src/server/sm_resources.cpp:48,64)
+    void record_resource_event(job::Job* job, unsigned num, ResourceEvent event);
+    // the job's next stage has joined the ready queue (reference src/server/scheduler_full3.cpp:175,244,304)
+    void record_queued_resource_event(job::Job* job);
 
   private:
     ipc::ShmChannelCpuReader* c2s_channel_;
     bool kernel_info_flag_ = false;
     bool job_events_flag_ = false;
-    bool other_flags_[4] = {false, false, false, false};
+    bool run_next_times_flag_ = false;
+    bool resource_events_flag_ = false;
+    bool other_flags_[2] = {false, false};  // block exec times, kernel block mis-allocation: accepted, nothing recorded
+    std::vector<std::tuple<TimePoint, TimePoint, unsigned>> run_next_times_;
+    std::vector<std::tuple<JobId, std::string, ResourceEvent, TimePoint, unsigned, unsigned, unsigned, unsigned>> resource_events_;
     std::vector<std::tuple<TimePoint, TimePoint, unsigned, unsigned, unsigned, unsigned, double, unsigned>> kernel_info_;
     std::vector<std::vector<std::pair<JobEvent, TimePoint>>> jobs_events_cur_;
     std::vector<std::vector<std::pair<JobEvent, TimePoint>>> jobs_events_all_;

@@ -64,6 +64,7 @@ struct Options {
     unsigned num_jobs = 0, start_record_num = 0, seed = 1, sched_sleep = 0;
     unsigned warmup_jobs = 0;  // extra requests served (same arrival process) before the measured ones
     bool pin_threads = true;
+    std::string profile_prefix;  // non-empty: the server records everything during the measured phase and saves to this prefix
     // name-shaping switches (which parameters appear in the output file names, which one is the x column)
     bool n_iat = false, n_lns = false, n_con = false, n_n = false, n_srn = false, n_seed = false, n_fair = false, n_scheds = false;
     bool g_iat = false, g_lns = false, g_con = false, g_n = false, g_srn = false, g_seed = false, g_fair = false, g_scheds = false;
@@ -89,7 +90,27 @@ class LoadGenerator {
 
     void run() {
         if (opt_.warmup_jobs) phase(opt_.warmup_jobs, false);
+        // Server-side recording around the measured phase (the reference keeps these calls commented out in
+        // its monitor thread, reference app/client.cpp:101-121).
+        llis::client::ProfilerClient* prof = opt_.profile_prefix.empty() ? nullptr : client_->get_profiler_client();
+        if (prof) {
+            prof->set_record_kernel_info();
+            prof->set_record_block_exec_time();
+            prof->set_record_kernel_block_mis_alloc();
+            prof->set_record_run_next_times();
+            prof->set_record_job_events();
+            prof->set_record_resource_events();
+        }
         phase(opt_.num_jobs, true);
+        if (prof) {
+            prof->unset_record_kernel_info();
+            prof->unset_record_block_exec_time();
+            prof->unset_record_kernel_block_mis_alloc();
+            prof->unset_record_run_next_times();
+            prof->unset_record_job_events();
+            prof->unset_record_resource_events();
+            prof->save(opt_.profile_prefix);
+        }
     }
 
     double elapsed_us() const { return std::chrono::duration<double, std::micro>(end_time_ - start_time_).count(); }

@@ -1,6 +1,7 @@
 #include <llis/server/profiler.h>
 
 #include <cstdio>
+#include <typeinfo>
 
 namespace llis {
 namespace server {
@@ -21,8 +22,8 @@ void Profiler::handle_cmd() {
         case 4: job_events_flag_ = on; break;
         case 1: other_flags_[0] = on; break;
         case 2: other_flags_[1] = on; break;
-        case 3: other_flags_[2] = on; break;
-        case 5: other_flags_[3] = on; break;
+        case 3: run_next_times_flag_ = on; break;
+        case 5: resource_events_flag_ = on; break;
         default: std::fprintf(stderr, "[llis] unknown profiler command %u ignored\n", v); break;
     }
 }
@@ -44,6 +45,22 @@ void Profiler::record_job_event(JobId job_id, JobEvent event) {
     }
 }
 
+void Profiler::record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks) {
+    if (run_next_times_flag_) run_next_times_.emplace_back(start, end, num_blocks);
+}
+
+void Profiler::record_resource_event(job::Job* job, unsigned num, ResourceEvent event) {
+    if (!resource_events_flag_) return;
+    resource_events_.emplace_back(job->get_unique_id(), typeid(*job).name(), event, std::chrono::steady_clock::now(), num, job->get_cur_num_threads_per_block(),
+                                  job->get_cur_smem_size_per_block(), job->get_cur_num_registers_per_thread());
+}
+
+void Profiler::record_queued_resource_event(job::Job* job) {
+    if (!resource_events_flag_) return;
+    resource_events_.emplace_back(job->get_unique_id(), typeid(*job).name(), ResourceEvent::QUEUED, std::chrono::steady_clock::now(), job->get_num_blocks(),
+                                  job->get_num_threads_per_block(), job->get_smem_size_per_block(), job->get_num_registers_per_thread());
+}
+
 void Profiler::save(const std::string& prefix) {
     auto ns = [](TimePoint t) { return (long long)t.time_since_epoch().count(); };
     if (FILE* fp = std::fopen((prefix + "_kernel_info.txt").c_str(), "w")) {
@@ -60,11 +77,26 @@ void Profiler::save(const std::string& prefix) {
         }
         std::fclose(fp);
     }
-    for (const char* name : {"_block_exec_times.txt", "_kernel_block_mis_alloc.txt", "_run_next_times.txt", "_resource_events.txt"}) {
+    auto us = [](TimePoint t) { return std::chrono::duration<double, std::micro>(t.time_since_epoch()).count(); };
+    if (FILE* fp = std::fopen((prefix + "_run_next_times.txt").c_str(), "w")) {
+        for (const auto& r : run_next_times_)
+            std::fprintf(fp, "%f %f %f %u\n", us(std::get<0>(r)), us(std::get<1>(r)),
+                         std::chrono::duration<double, std::micro>(std::get<1>(r) - std::get<0>(r)).count(), std::get<2>(r));
+        std::fclose(fp);
+    }
+    if (FILE* fp = std::fopen((prefix + "_resource_events.txt").c_str(), "w")) {
+        for (const auto& r : resource_events_)
+            std::fprintf(fp, "%u %s %u %f %u %u %u %u\n", (unsigned)std::get<0>(r), std::get<1>(r).c_str(), (unsigned)std::get<2>(r), us(std::get<3>(r)), std::get<4>(r),
+                         std::get<5>(r), std::get<6>(r), std::get<7>(r));
+        std::fclose(fp);
+    }
+    for (const char* name : {"_block_exec_times.txt", "_kernel_block_mis_alloc.txt"}) {
         if (FILE* fp = std::fopen((prefix + name).c_str(), "w")) std::fclose(fp);
     }
     kernel_info_.clear();
     jobs_events_all_.clear();
+    run_next_times_.clear();
+    resource_events_.clear();
 }
 
 }  // namespace server

@@ -70,7 +70,13 @@ void SchedulerFifo2::schedule_job() {
         }
         job::Context::set_current_job(job);
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_START);
-        job->run_next();
+        if (profiler_->recording_run_next_times()) {
+            const auto t0 = std::chrono::steady_clock::now();
+            job->run_next();
+            profiler_->record_run_next_time(t0, std::chrono::steady_clock::now(), is_mem ? 0 : job->get_cur_num_blocks());
+        } else {
+            job->run_next();
+        }
         if (is_mem) post_mem_completion(job);
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);
     }

@@ -103,6 +103,7 @@ void SchedulerFull3::handle_new_job(std::unique_ptr<job::Job> owned) {
     if (!server_->has_job_stage_resource(job, next_stage)) server_->set_job_stage_resource(job, next_stage, 1);
     job->set_stage_lengths_resources(server_->get_job_remaining_rl(job, 0), server_->get_job_stage_lengths(job), server_->get_job_stage_resources(job));
     job->set_priority(take_priority(job));
+    if (!job->is_mem()) profiler_->record_queued_resource_event(job);
 
     job_queue_.push(job);
     ++num_jobs_;
@@ -129,6 +130,7 @@ void SchedulerFull3::requeue_or_finish(job::Job* job) {
         const unsigned next_stage = (unsigned)(job->get_cur_stage() + 1);
         if (!server_->has_job_stage_resource(job, next_stage)) server_->set_job_stage_resource(job, next_stage, 1);
         job->set_priority(take_priority(job));
+        if (!job->is_mem()) profiler_->record_queued_resource_event(job);
         job_queue_.push(job);
     } else {
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::JOB_FINISHED);
@@ -205,7 +207,13 @@ void SchedulerFull3::schedule_job() {
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_START);
         {
             LLIS_PHASE(kLaunch);
-            job->run_next();
+            if (profiler_->recording_run_next_times()) {
+                const auto t0 = std::chrono::steady_clock::now();
+                job->run_next();
+                profiler_->record_run_next_time(t0, std::chrono::steady_clock::now(), job->get_cur_num_blocks());
+            } else {
+                job->run_next();
+            }
             if (is_mem) post_mem_completion(job);
         }
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);

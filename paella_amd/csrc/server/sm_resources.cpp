@@ -1,3 +1,4 @@
+#include <llis/server/profiler.h>
 #include <llis/server/sm_resources.h>
 #include <llis/utils/error.h>
 
@@ -31,6 +32,7 @@ void SmResources::acquire(job::Job* job, int num) {
     nthrs_ -= threads * num;
     smem_ -= (long long)job->get_cur_smem_size_per_block() * num;
     nblocks_ -= num;
+    if (profiler_) profiler_->record_resource_event(job, (unsigned)num, Profiler::ResourceEvent::ACQUIRE);
 }
 
 void SmResources::release(job::Job* job, int num) {
@@ -39,6 +41,7 @@ void SmResources::release(job::Job* job, int num) {
     nthrs_ += threads * num;
     smem_ += (long long)job->get_cur_smem_size_per_block() * num;
     nblocks_ += num;
+    if (profiler_) profiler_->record_resource_event(job, (unsigned)num, Profiler::ResourceEvent::RELEASE);
 }
 
 double SmResources::dot(job::Job* job) const {

@@ -48,6 +48,37 @@ def test_load_generator_against_server_process(tmp_path, sched):
     assert not [f for f in os.listdir("/dev/shm") if name in f and "channel" in f]
 
 
+def test_profiler_files_have_the_reference_line_formats(tmp_path):
+    """--profile: the client switches every recording on around the measured phase and asks the server to save.
+    Line formats follow reference src/server/profiler.cpp:76-131."""
+    name = "ptprof%d" % os.getpid()
+    srv = start_server(name, "full3", FAKE_HIP_OP_US="20")
+    prof = str(tmp_path / "prof")
+    out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "200", "--dist", "exp", "--concurrency", "16",
+                          "--num_jobs", "60", "--seed", "1", "--prefix", str(tmp_path / "run"), "--no_pin", "--profile", prof,
+                          fake_job("fake_short"), "0.5", "8", fake_job("fake_mem3"), "0.5", "8"],
+                         env=fake_env(), capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert srv.wait(timeout=30) == 0
+    for suffix in ("kernel_info", "block_exec_times", "kernel_block_mis_alloc", "run_next_times", "job_events", "resource_events"):
+        assert os.path.exists("%s_%s.txt" % (prof, suffix)), suffix
+    kernel_info = [l.split() for l in open(prof + "_kernel_info.txt")]
+    assert kernel_info and all(len(l) == 8 and int(l[0]) <= int(l[1]) for l in kernel_info)
+    run_next = [l.split() for l in open(prof + "_run_next_times.txt")]
+    assert run_next and all(len(l) == 4 and abs(float(l[1]) - float(l[0]) - float(l[2])) < 1e-2 for l in run_next)
+    jobs = [l.split() for l in open(prof + "_job_events.txt")]
+    assert len(jobs) == 60
+    for l in jobs:  # pairs "event time"; a job starts with JOB_SUBMITTED (0) and ends with JOB_FINISHED (6), times non-decreasing
+        ev, t = [int(x) for x in l[0::2]], [float(x) for x in l[1::2]]
+        assert ev[0] == 0 and ev[-1] == 6 and t == sorted(t)
+    res = [l.split() for l in open(prof + "_resource_events.txt")]
+    assert res and all(len(l) == 8 and l[2] in ("0", "1", "2") for l in res)
+    acquired = sum(int(l[4]) for l in res if l[2] == "0")
+    released = sum(int(l[4]) for l in res if l[2] == "1")
+    assert acquired == released > 0   # every workgroup that was admitted has been given back
+    assert open(prof + "_block_exec_times.txt").read() == ""
+
+
 def test_arrival_process_is_reproducible_for_a_seed():
     """Same seed, same job mix => same sequence of job types (draw order: type first, then inter-arrival)."""
     counts = []
