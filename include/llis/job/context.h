@@ -20,7 +20,11 @@ class Context {
     static void set_gpu2sched_channel(ipc::Gpu2SchedChannel* channel) { gpu2sched_channel_ = channel->fork(); }
     static ipc::Gpu2SchedChannel* get_gpu2sched_channel() { return &gpu2sched_channel_; }
 
-    static void set_gpu2sched_block_time_channel(ipc::Gpu2SchedChannel* channel) { gpu2sched_block_time_channel_ = channel->fork(); }
+    // nullptr: the active scheduler collects no per-workgroup timing (a handle left by an earlier scheduler of
+    // this process must not survive it)
+    static void set_gpu2sched_block_time_channel(ipc::Gpu2SchedChannel* channel) {
+        gpu2sched_block_time_channel_ = channel ? channel->fork() : ipc::Gpu2SchedChannel();
+    }
     static ipc::Gpu2SchedChannel* get_gpu2sched_block_time_channel() { return &gpu2sched_block_time_channel_; }
 
     static void set_mem2sched_channel(ipc::ShmChannelCpuReader* channel) { mem2sched_channel_ = channel->fork(); }

@@ -8,14 +8,20 @@
 //   }
 //
 // Aggregation: lane (0,0,0) of each workgroup bumps a per-notifier counter that wraps at the grid size;
-// one message is sent per 16 workgroups plus one for the remainder, so a grid of n workgroups produces
-// exactly ceil(n/16) start messages and ceil(n/16) end messages whose `num` fields sum to n
+// one message is sent per noti_batch_size workgroups plus one for the remainder, so a grid of n workgroups
+// produces exactly ceil(n/batch) start messages and ceil(n/batch) end messages whose `num` fields sum to n
 // (reference include/llis/job/finished_block_notifier.h:18-94, alloc at src/job/finished_block_notifier.cu:21-46).
 //
 // Ordering on gfx950: a workgroup's results must be visible to a kernel that the scheduler launches on a
 // different stream as soon as the host has seen the end message.  Each workgroup therefore issues a
 // device-scope release before it bumps the end counter, the sender acquires at device scope after the
 // bump, and the message itself is a system-scope release store.
+//
+// Per-workgroup timing (optional, switched on when the array is created with a second ring): lane (0,0,0)
+// samples the 100 MHz wall clock on entry and on exit and sends both, 24 bits each, as one BlockStartEndTime
+// slot (reference LLIS_MEASURE_BLOCK_TIME, include/llis/job/finished_block_notifier.h:20-25,58-63,90-92; there a
+// compile-time switch, one sample pair shared by all workgroups of a kernel, SM clock / 256).  The entry
+// sample lives in LDS, so every workgroup reports its own pair; unit here: 10 ns.
 
 #include <llis/ipc/shm_primitive_channel.h>
 #include <llis/job/instrument_info.h>
@@ -32,8 +38,12 @@ class FinishedBlockNotifier {
     static constexpr unsigned noti_batch_size = 64;
 
     FinishedBlockNotifier() {}
-    explicit FinishedBlockNotifier(ipc::Gpu2SchedChannel* gpu2sched_channel) {
+    explicit FinishedBlockNotifier(ipc::Gpu2SchedChannel* gpu2sched_channel, ipc::Gpu2SchedChannel* block_time_channel = nullptr) {
         gpu2sched_channel_ = gpu2sched_channel->fork();
+        if (block_time_channel) {
+            block_time_channel_ = block_time_channel->fork();
+            measure_block_time_ = 1;
+        }
     }
     FinishedBlockNotifier(FinishedBlockNotifier&&) = default;
     FinishedBlockNotifier& operator=(FinishedBlockNotifier&&) = default;
@@ -41,8 +51,15 @@ class FinishedBlockNotifier {
 #if defined(__HIPCC__)
     __device__ __forceinline__ void start(JobId job_id) {
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
+            if (measure_block_time_) *entry_clock_slot() = (unsigned)wall_clock64() & 0xFFFFFFu;
             announce<false>(&agg_counter_start_, 1, job_id);
         }
+    }
+
+    // For kernels that skip start() (no start message wanted) and were told by their caller that timing is on:
+    // takes the entry sample without looking at the notifier.
+    __device__ __forceinline__ void begin_timing() {
+        if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) *entry_clock_slot() = (unsigned)wall_clock64() & 0xFFFFFFu;
     }
 
     // For arbitrary kernels: makes everything the workgroup wrote visible device-wide (cache write-back)
@@ -52,6 +69,7 @@ class FinishedBlockNotifier {
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             announce<true>(&agg_counter_end_, 0, job_id);
+            if (measure_block_time_) send_block_time();
         }
     }
 
@@ -64,16 +82,45 @@ class FinishedBlockNotifier {
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
             announce<false>(&agg_counter_end_, 0, job_id);
+            if (measure_block_time_) send_block_time();
+        }
+    }
+
+    // Same, for callers that know from elsewhere whether timing is on (the flag is then not read here).
+    __device__ __forceinline__ void end_written_through(JobId job_id, bool timed) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
+            announce<false>(&agg_counter_end_, 0, job_id);
+            if (timed && measure_block_time_) send_block_time();  // the member is looked at only when timing was asked for
         }
     }
 #endif
 
-    // Allocates `num` notifiers in device memory, all bound to the given ring.
-    static FinishedBlockNotifier* create_array(unsigned num, ipc::Gpu2SchedChannel* gpu2sched_channel);
+    // Allocates `num` notifiers in device memory, all bound to the given ring (and, when given, to the ring
+    // that receives per-workgroup timing samples).
+    static FinishedBlockNotifier* create_array(unsigned num, ipc::Gpu2SchedChannel* gpu2sched_channel,
+                                               ipc::Gpu2SchedChannel* block_time_channel = nullptr);
     static void free_array(FinishedBlockNotifier* ptr);
 
   private:
 #if defined(__HIPCC__)
+    // One word of LDS per kernel that carries the hooks: the workgroup's entry sample (only lane (0,0,0) touches it).
+    __device__ __forceinline__ static unsigned* entry_clock_slot() {
+        __shared__ unsigned entry_clock;
+        return &entry_clock;
+    }
+
+    __device__ __forceinline__ void send_block_time() {
+        const unsigned s = *entry_clock_slot();
+        const unsigned e = (unsigned)wall_clock64() & 0xFFFFFFu;
+        BlockStartEndTime t;  // 24 + 24 bits packed as in reference src/server/scheduler_full3.cpp:113-119
+        t.data[0] = (uint16_t)(s >> 8);
+        t.data[1] = (uint16_t)(((s & 0xFFu) << 8) | (e >> 16));
+        t.data[2] = (uint16_t)(e & 0xFFFFu);
+        block_time_channel_.write_relaxed(t);
+    }
+
     // ACQUIRE: the sender first acquires (device scope) what the other workgroups released before their bump.
     template <bool ACQUIRE>
     __device__ __forceinline__ void announce(unsigned* counter, uint8_t is_start, JobId job_id) {
@@ -98,8 +145,13 @@ class FinishedBlockNotifier {
     }
 #endif
 
+    // Read-only after creation ...
     ipc::Gpu2SchedChannel gpu2sched_channel_;
-    unsigned agg_counter_start_ = 0;
+    ipc::Gpu2SchedChannel block_time_channel_;
+    unsigned measure_block_time_ = 0;
+    // ... and, on a cache line of their own, the counters every workgroup bumps atomically: a load of the
+    // fields above must not queue behind those atomics.
+    alignas(128) unsigned agg_counter_start_ = 0;
     unsigned agg_counter_end_ = 0;
 };
 

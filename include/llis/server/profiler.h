@@ -3,9 +3,9 @@
 // carrying a path prefix) follows reference src/server/profiler.cpp:10-67 so a client's ProfilerClient
 // keeps working; recording covers kernel info, per-job event timelines, run_next() times and resource events,
 // written on SAVE as <prefix>_kernel_info.txt, _job_events.txt, _run_next_times.txt and _resource_events.txt in
-// the reference's line formats (reference src/server/profiler.cpp:76-131).  _block_exec_times.txt (needs the
-// optional per-block timing ring) and _kernel_block_mis_alloc.txt (written only by schedulers the reference
-// does not build) are created empty.
+// the reference's line formats (reference src/server/profiler.cpp:76-131), plus _block_exec_times.txt when the
+// server runs with --measure_block_time (entry and exit clock of every workgroup, 24 bits each, 10 ns units).
+// _kernel_block_mis_alloc.txt (written only by schedulers the reference does not build) is created empty.
 
 #include <llis/ipc/defs.h>
 #include <llis/ipc/shm_channel.h>
@@ -39,6 +39,7 @@ class Profiler {
     void record_kernel_info(TimePoint start, TimePoint end, unsigned num_blocks, unsigned num_threads_per_block, unsigned smem_size_per_block,
                             unsigned num_registers_per_thread, double priority, unsigned job_ref_id);
     void record_job_event(JobId job_id, JobEvent event);
+    void record_block_exec_time(unsigned long long start, unsigned long long end);
     bool recording_run_next_times() const { return run_next_times_flag_; }
     void record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks);
     // num workgroups of the job's running stage acquired or released (reference src/server/sm_resources.cpp:48,64)
@@ -52,7 +53,9 @@ class Profiler {
     bool job_events_flag_ = false;
     bool run_next_times_flag_ = false;
     bool resource_events_flag_ = false;
-    bool other_flags_[2] = {false, false};  // block exec times, kernel block mis-allocation: accepted, nothing recorded
+    bool block_exec_times_flag_ = false;
+    bool mis_alloc_flag_ = false;  // accepted, nothing records it
+    std::vector<std::pair<unsigned long long, unsigned long long>> block_exec_times_;
     std::vector<std::tuple<TimePoint, TimePoint, unsigned>> run_next_times_;
     std::vector<std::tuple<JobId, std::string, ResourceEvent, TimePoint, unsigned, unsigned, unsigned, unsigned>> resource_events_;
     std::vector<std::tuple<TimePoint, TimePoint, unsigned, unsigned, unsigned, unsigned, double, unsigned>> kernel_info_;

@@ -36,6 +36,9 @@ struct SchedulerOptions {
     // false = a runtime host callback writes the job pointer into the mem2sched byte ring.
     bool mem_marker = true;
     size_t ring_slots = GPU2SCHED_CHAN_SIZE;
+    // --measure_block_time: every workgroup also reports its entry and exit clock through a second ring; the
+    // profiler keeps the pairs while block-exec-time recording is on (reference: compile-time LLIS_MEASURE_BLOCK_TIME).
+    bool measure_block_time = false;
 };
 
 class Scheduler {
@@ -109,6 +112,7 @@ class StreamPoolScheduler : public Scheduler {
     static void mem_notification_callback(void* job);
 
     ipc::Gpu2SchedChannel gpu2sched_channel_;
+    ipc::Gpu2SchedChannel gpu2sched_block_time_channel_;  // connected only with options.measure_block_time
     ipc::ShmChannelCpuReader mem2sched_channel_;
     std::vector<void*> streams_;
     std::vector<unsigned> free_streams_;

@@ -31,6 +31,10 @@ extern "C" {
  * needs start messages only for kernels it admitted beyond the occupancy budget (to learn when they have
  * become fully resident); for every other kernel they are pure overhead.  Messages carry the id without the bit. */
 #define PAELLA_JOB_ID_NO_START 0x80000000u
+/* OR-ed into job_id by callers whose scheduler collects per-workgroup timing (second ring of the notifier):
+ * the kernel samples the clock on entry and exit and reports the pair.  Off: the kernel never looks. */
+#define PAELLA_JOB_ID_TIME_BLOCKS 0x40000000u
+#define PAELLA_JOB_ID_FLAGS (PAELLA_JOB_ID_NO_START | PAELLA_JOB_ID_TIME_BLOCKS)
 
 #define PAELLA_EINVAL (-1)   /* malformed descriptor */
 #define PAELLA_ENOSUP (-2)   /* shape class not implemented (e.g. grouped conv that is not depthwise), or facility unavailable */

@@ -34,6 +34,7 @@ typedef struct paella_server_options {
     int mem_marker;            /* 1: ring-marker kernel reports copy stages, 0: runtime host callback */
     int event_log;             /* 1: record the scheduler event log */
     int cpu;                   /* pin the serving thread to this CPU, -1 = do not pin */
+    int measure_block_time;    /* 1: --measure_block_time (per-workgroup entry/exit clocks for the profiler) */
 } paella_server_options;
 
 int paella_server_start(const paella_server_options* options, paella_server** out);
@@ -59,6 +60,7 @@ typedef struct paella_load_options {
     unsigned warmup_jobs;      /* served before the clock starts, beyond the one run per pooled instance */
     unsigned seed;
     int pin_threads;           /* pin monitor/submit threads to CPUs 0 and 2 like the reference client */
+    const char* profile_prefix; /* non-NULL: server-side recording around the measured phase, saved to this prefix */
 } paella_load_options;
 
 typedef struct paella_latency_stats {

@@ -108,7 +108,7 @@ template <int MI, int NI, int KW, bool TAP_MAJOR>
 __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
     CONV_TL(0);
     if (PAELLA_CONV_ABLATE & 16) return;
-    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
+    paella::hook_entry(p.notifier, p.job_id);
 
     // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
     extern __shared__ __align__(16) char smem[];
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     }
 
     CONV_TL(7);
-    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(p.notifier, p.job_id);
 #ifdef PAELLA_CONV_TIMELINE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     CONV_TL(8);
@@ -455,7 +455,7 @@ struct DwArgs {
 };
 
 __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
-    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
+    paella::hook_entry(p.notifier, p.job_id);
     const int c = blockIdx.y;
     const int pix = blockIdx.x * 256 + threadIdx.x;
     const int PQ = p.P * p.Q;
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
         const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
         store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
     }
-    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(p.notifier, p.job_id);
 }
 
 typedef void (*ConvKernel)(ConvArgs);

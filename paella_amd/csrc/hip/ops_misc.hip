@@ -44,7 +44,7 @@ __device__ __forceinline__ float wave_max(float v) {
 __global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                     const float* __restrict__ bias, float* __restrict__ y, int I, int O,
                                                     int act, uint32_t job_id, Notifier* notifier) {
-    if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
+    paella::hook_entry(notifier, job_id);
     const int lane = threadIdx.x & 63;
     const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (o < O) {
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x,
         acc = wave_sum(acc);
         if (lane == 0) store_out(y + o, act_apply(acc + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f));
     }
-    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(notifier, job_id);
 }
 
 // ------------------------------------------------------------------------------------------ pooling
@@ -77,7 +77,7 @@ struct PoolArgs {
 };
 
 __global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
-    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
+    paella::hook_entry(p.notifier, p.job_id);
     const int PQ = p.P * p.Q;
     const int idx = blockIdx.x * 256 + threadIdx.x;
     if (idx < p.C * PQ) {
@@ -121,13 +121,13 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
             store_out(p.y + idx, m);
         }
     }
-    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(p.notifier, p.job_id);
 }
 
 // One wave per channel.
 __global__ __launch_bounds__(256) void gap_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW,
                                                   uint32_t job_id, Notifier* notifier) {
-    if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
+    paella::hook_entry(notifier, job_id);
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (c < C) {
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void gap_kernel(const float* __restrict__ x, f
         acc = wave_sum(acc);
         if (lane == 0) store_out(y + c, acc / (float)HW);
     }
-    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(notifier, job_id);
 }
 
 // ------------------------------------------------------------------------------------------ elementwise
@@ -165,7 +165,7 @@ __device__ __forceinline__ float elt_one(const EltArgs& p, float a, float b, int
 
 template <bool VEC4>
 __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs p) {
-    if (p.notifier && !(p.job_id & PAELLA_JOB_ID_NO_START)) p.notifier->start(p.job_id);
+    paella::hook_entry(p.notifier, p.job_id);
     const size_t n = (size_t)p.C * p.HW;
     if (VEC4) {
         const size_t i4 = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -185,26 +185,26 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs p) {
         const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
         if (i < n) store_out(p.y + i, elt_one(p, p.a[i], p.b ? p.b[i] : 0.f, (int)(i / p.HW)));
     }
-    if (p.notifier) p.notifier->end_written_through(p.job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(p.notifier, p.job_id);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n,
                                                    uint32_t job_id, Notifier* notifier) {
-    if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
+    paella::hook_entry(notifier, job_id);
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i + 3 < n && n < ((size_t)1 << 30) && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
         store_out4(y, i, *reinterpret_cast<const float4*>(x + i));
     } else {
         for (size_t k = i; k < n && k < i + 4; ++k) store_out(y + k, x[k]);
     }
-    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(notifier, job_id);
 }
 
 // ------------------------------------------------------------------------------------------ softmax / LRN
 // One workgroup per row.
 __global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ x, float* __restrict__ y, int cols,
                                                       uint32_t job_id, Notifier* notifier) {
-    if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
+    paella::hook_entry(notifier, job_id);
     __shared__ float part[4];
     const float* xr = x + (size_t)blockIdx.x * cols;
     float* yr = y + (size_t)blockIdx.x * cols;
@@ -223,12 +223,12 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ 
     __syncthreads();
     s = (part[0] + part[1]) + (part[2] + part[3]);
     for (int i = threadIdx.x; i < cols; i += 256) store_out(yr + i, expf(xr[i] - m) / s);
-    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(notifier, job_id);
 }
 
 __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW, int size,
                                                   float alpha, float beta, float k, uint32_t job_id, Notifier* notifier) {
-    if (notifier && !(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id);
+    paella::hook_entry(notifier, job_id);
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx < (size_t)C * HW) {
         const int c = (int)(idx / HW);
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, f
         }
         store_out(y + idx, x[idx] / powf(k + alpha / (float)size * sq, beta));
     }
-    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_NO_START);
+    paella::hook_exit(notifier, job_id);
 }
 
 inline unsigned blocks_for(size_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }

@@ -8,6 +8,26 @@
 
 #include <hip/hip_runtime.h>
 
+#include "paella_ops.h"
+#include <llis/job/finished_block_notifier.h>
+
+namespace paella {
+// First statement of every operator kernel.  The start message is sent only when the scheduler asked for it
+// (job id without PAELLA_JOB_ID_NO_START); the entry clock sample for per-workgroup timing is taken when start()
+// runs (it knows from the notifier) or when the caller set PAELLA_JOB_ID_TIME_BLOCKS.
+__device__ __forceinline__ void hook_entry(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id) {
+    if (notifier) {
+        if (!(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id & ~PAELLA_JOB_ID_FLAGS);
+        else if (job_id & PAELLA_JOB_ID_TIME_BLOCKS) notifier->begin_timing();
+    }
+}
+
+// Last statement of every operator kernel (all results written with store_out / store_out4).
+__device__ __forceinline__ void hook_exit(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id) {
+    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_FLAGS, (job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0);
+}
+}  // namespace paella
+
 __device__ __forceinline__ void store_out(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Four consecutive floats at base[index .. index+3] (16-byte aligned) as ONE 16-byte write-through store.  Four

@@ -50,6 +50,7 @@ class ModelJob : public llis::job::CoroutineJob {
         // notification ring (fifo2, full3): the queues have no ordering of their own, and fifo relies on the stream.
         const char* resident = std::getenv("PAELLA_INPUT_RESIDENT");
         input_resident_ = resident && std::strcmp(resident, "1") == 0;
+        timed_ = llis::job::Context::get_gpu2sched_block_time_channel()->is_connected();  // server runs with --measure_block_time
         const char* dispatch = std::getenv("PAELLA_DISPATCH");
         direct_ = !(dispatch && std::strcmp(dispatch, "hip") == 0) && llis::job::Context::is_stage_by_stage();
         if (direct_) {
@@ -85,7 +86,7 @@ class ModelJob : public llis::job::CoroutineJob {
             set_num_registers_per_thread(d.vgprs);
             yield();
             // Only a kernel admitted beyond the occupancy budget ("unfit") needs its workgroup starts reported.
-            const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START);
+            const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
             void* target = stream();
             if (direct_) check(paella_direct_queue_shared(&target), "direct queue");
             check(paella_exec_launch_stage(exec_, s, target, id, get_finished_block_notifier()), "stage launch");
@@ -118,6 +119,7 @@ class ModelJob : public llis::job::CoroutineJob {
     void* io_ptr_ = nullptr;
     int num_stages_ = 0;
     bool direct_ = true;
+    bool timed_ = false;
     bool input_resident_ = false, input_uploaded_ = false;
 };
 

@@ -47,6 +47,7 @@ int paella_server_start(const paella_server_options* o, paella_server** out) {
         if (o->unfair > 0) so.unfair = o->unfair;
         so.sched_sleep = o->sched_sleep;
         so.mem_marker = o->mem_marker != 0;
+        so.measure_block_time = o->measure_block_time != 0;
         auto s = std::make_unique<paella_server>();
         s->scheduler = llis::server::SchedulerFactory::create(o->sched, so);
         s->server = std::make_unique<llis::server::Server>(o->name, s->scheduler.get());
@@ -111,6 +112,7 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         opt.warmup_jobs = o->warmup_jobs;
         opt.seed = o->seed;
         opt.pin_threads = o->pin_threads != 0;
+        if (o->profile_prefix) opt.profile_prefix = o->profile_prefix;
 
         std::vector<float> props_cum;
         std::vector<unsigned> max_outstanding;

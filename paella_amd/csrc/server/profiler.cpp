@@ -20,8 +20,8 @@ void Profiler::handle_cmd() {
     switch (v / 2) {
         case 0: kernel_info_flag_ = on; break;
         case 4: job_events_flag_ = on; break;
-        case 1: other_flags_[0] = on; break;
-        case 2: other_flags_[1] = on; break;
+        case 1: block_exec_times_flag_ = on; break;
+        case 2: mis_alloc_flag_ = on; break;
         case 3: run_next_times_flag_ = on; break;
         case 5: resource_events_flag_ = on; break;
         default: std::fprintf(stderr, "[llis] unknown profiler command %u ignored\n", v); break;
@@ -43,6 +43,10 @@ void Profiler::record_job_event(JobId job_id, JobEvent event) {
         jobs_events_all_.push_back(std::move(cur));
         cur.clear();
     }
+}
+
+void Profiler::record_block_exec_time(unsigned long long start, unsigned long long end) {
+    if (block_exec_times_flag_) block_exec_times_.emplace_back(start, end);
 }
 
 void Profiler::record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks) {
@@ -90,12 +94,15 @@ void Profiler::save(const std::string& prefix) {
                          std::get<5>(r), std::get<6>(r), std::get<7>(r));
         std::fclose(fp);
     }
-    for (const char* name : {"_block_exec_times.txt", "_kernel_block_mis_alloc.txt"}) {
-        if (FILE* fp = std::fopen((prefix + name).c_str(), "w")) std::fclose(fp);
+    if (FILE* fp = std::fopen((prefix + "_block_exec_times.txt").c_str(), "w")) {
+        for (const auto& b : block_exec_times_) std::fprintf(fp, "%llu %llu\n", b.first, b.second);
+        std::fclose(fp);
     }
+    if (FILE* fp = std::fopen((prefix + "_kernel_block_mis_alloc.txt").c_str(), "w")) std::fclose(fp);
     kernel_info_.clear();
     jobs_events_all_.clear();
     run_next_times_.clear();
+    block_exec_times_.clear();
     resource_events_.clear();
 }
 

@@ -48,7 +48,10 @@ StreamPoolScheduler::StreamPoolScheduler(const SchedulerOptions& options, size_t
         stream_index_[streams_[i]] = i;
         free_streams_.push_back(i);
     }
-    notifiers_raw_ = job::FinishedBlockNotifier::create_array(options.num_streams, &gpu2sched_channel_);
+    if (options.measure_block_time) gpu2sched_block_time_channel_.connect(std::string(), options.ring_slots);
+    job::Context::set_gpu2sched_block_time_channel(options.measure_block_time ? &gpu2sched_block_time_channel_ : nullptr);
+    notifiers_raw_ = job::FinishedBlockNotifier::create_array(options.num_streams, &gpu2sched_channel_,
+                                                              options.measure_block_time ? &gpu2sched_block_time_channel_ : nullptr);
     for (unsigned i = 0; i < options.num_streams; ++i) free_notifiers_.push_back(i);
 }
 
@@ -76,6 +79,13 @@ void StreamPoolScheduler::try_handle_block_start_finish() {
     }
     else {
         LLIS_PHASE(kIdle);
+    }
+    while (options_.measure_block_time && gpu2sched_block_time_channel_.can_read<job::BlockStartEndTime>()) {
+        // unpacking as in reference src/server/scheduler_full3.cpp:113-119
+        const job::BlockStartEndTime t = gpu2sched_block_time_channel_.read<job::BlockStartEndTime>();
+        const uint32_t start = (uint32_t)t.data[0] << 8 | (uint32_t)(t.data[1] >> 8);
+        const uint32_t end = (uint32_t)(t.data[1] & 0xFF) << 16 | t.data[2];
+        profiler_->record_block_exec_time(start, end);
     }
     if (mem2sched_channel_.can_read()) {
         LLIS_PHASE(kRing);

@@ -11,13 +11,14 @@ c_int, c_uint, c_float, c_double, c_char_p, c_void_p, c_size_t = (ctypes.c_int, 
 
 class ServerOptions(ctypes.Structure):
     _fields_ = [("name", c_char_p), ("sched", c_char_p), ("num_streams", c_uint), ("extra_kernels", c_uint), ("unfair", c_float),
-                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int)]
+                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int)]
 
 
 class LoadOptions(ctypes.Structure):
     _fields_ = [("server_name", c_char_p), ("num_types", c_int), ("job_paths", c_char_p * MAX_TYPES), ("proportions", c_float * MAX_TYPES),
                 ("max_outstanding", c_uint * MAX_TYPES), ("iat_us", c_double), ("dist_exp", c_int), ("ln_sigma", c_double),
-                ("concurrency", c_int), ("num_jobs", c_uint), ("warmup_jobs", c_uint), ("seed", c_uint), ("pin_threads", c_int)]
+                ("concurrency", c_int), ("num_jobs", c_uint), ("warmup_jobs", c_uint), ("seed", c_uint), ("pin_threads", c_int),
+                ("profile_prefix", c_char_p)]
 
 
 class LatencyStats(ctypes.Structure):
@@ -67,9 +68,9 @@ class Server:
     """`with Server('name', 'full3', num_streams=64) as s: ...`; s.event_log() after the block."""
 
     def __init__(self, name, sched, num_streams=500, extra_kernels=2, unfair=1e6, sched_sleep=0, mem_marker=True, event_log=False,
-                 cpu=-1):
+                 cpu=-1, measure_block_time=False):
         self.opts = ServerOptions(name.encode(), sched.encode(), num_streams, extra_kernels, unfair, sched_sleep, int(mem_marker),
-                                  int(event_log), cpu)
+                                  int(event_log), cpu, int(measure_block_time))
         self.name = name
         self.handle = c_void_p()
 
@@ -93,7 +94,7 @@ class Server:
 
 
 def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, seed=1, dist="exp", ln_sigma=2.0, pin_threads=False,
-               want_latencies=False):
+               want_latencies=False, profile_prefix=None):
     """jobs = [(path, proportion, max_outstanding), ...].  Returns a dict of the run's statistics."""
     import numpy as np
     o = LoadOptions()
@@ -107,6 +108,7 @@ def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, 
         o.max_outstanding[i] = mo
     o.iat_us, o.dist_exp, o.ln_sigma = iat_us, int(dist == "exp"), ln_sigma
     o.concurrency, o.num_jobs, o.warmup_jobs, o.seed, o.pin_threads = concurrency, num_jobs, warmup_jobs, seed, int(pin_threads)
+    o.profile_prefix = profile_prefix.encode() if profile_prefix else None
     res = LoadResult()
     lat = np.zeros(num_jobs, np.float64) if want_latencies else None
     if lib().paella_client_run(ctypes.byref(o), ctypes.byref(res), lat.ctypes.data if want_latencies else None) != 0:

@@ -138,6 +138,25 @@ def test_concurrent_dummy_jobs_replay_exactly(cuda, sched_name):
     assert sum(1 for e in actual if e[0] == "E") == 24 + 5  # plus one warm-up run per pooled instance
 
 
+def test_per_workgroup_timing_reaches_the_profiler(cuda, tmp_path):
+    """--measure_block_time: every workgroup of every kernel reports its entry and exit clock (24 bits, 10 ns units)
+    through the second ring; with block-exec-time recording on, the saved file has one line per workgroup."""
+    from paella_amd import serve
+    prof = str(tmp_path / "bt")
+    n = 6
+    with serve.Server(server_name("bt"), "full3", num_streams=8, measure_block_time=True) as srv:
+        serve.client_run(srv.name, [(serve.job_path("dummy_short"), 0.5, 2), (serve.job_path("tvm_mnist"), 0.5, 2)], 0.0, 2, n, profile_prefix=prof)
+    pairs = [tuple(int(v) for v in l.split()) for l in open(prof + "_block_exec_times.txt")]
+    assert pairs and all(0 <= s < (1 << 24) and 0 <= e < (1 << 24) for s, e in pairs)
+    dur = [((e - s) & 0xFFFFFF) * 10e-3 for s, e in pairs]  # microseconds
+    assert min(dur) >= 0 and max(dur) < 1e5
+    # dummy_short: 10 stages of 5 workgroups, about 15 ms of spinning in all -> its workgroups take > 100 us each,
+    # the small CNN's take a few microseconds: both kinds must be present
+    assert sum(d > 100 for d in dur) >= 5 and sum(d < 50 for d in dur) >= 5
+    kinfo = [l.split() for l in open(prof + "_kernel_info.txt")]
+    assert len(pairs) == sum(int(k[2]) for k in kinfo)  # one sample pair per workgroup of every recorded kernel
+
+
 def test_mixed_model_load_then_outputs_still_correct(cuda):
     """Small CNN : ResNet-18 = 9 : 1 Poisson load under full3, then a checked request of each model on the same
     server (the instances and their buffers were recycled by the load)."""
