@@ -63,7 +63,8 @@ int main(int argc, char** argv) {
                                      {"seed", required_argument, nullptr, 's'},        {"prefix", required_argument, nullptr, 'p'},
                                      {"fairness", required_argument, nullptr, 'f'},    {"sched_sleep", required_argument, nullptr, 'h'},
                                      {"dist", required_argument, nullptr, 'd'},        {"warmup", required_argument, nullptr, 'w'},        {"no_pin", no_argument, nullptr, 'P'},
-                                     {"profile", required_argument, nullptr, 'R'}};
+                                     {"profile", required_argument, nullptr, 'R'},
+                                     {"trace", required_argument, nullptr, 'T'}};
     for (int i = 0; i < 16; ++i) long_opts.push_back(option{flag_names[i], no_argument, &flag_slot, i + 1});
     long_opts.push_back(option{nullptr, 0, nullptr, 0});
 
@@ -84,13 +85,14 @@ int main(int argc, char** argv) {
             case 'w': opt.warmup_jobs = (unsigned)std::atoi(optarg); break;
             case 'P': opt.pin_threads = false; break;
             case 'R': opt.profile_prefix = optarg; break;
+            case 'T': opt.trace_path = optarg; break;
             default: return 2;
         }
     }
     if (opt.server_name.empty() || opt.iat < 0 || opt.concurrency <= 0 || opt.num_jobs == 0 || (argc - optind) < 3 || (argc - optind) % 3 != 0 ||
         (opt.dist != "exp" && opt.dist != "ln")) {
         std::fprintf(stderr, "usage: %s --server_name S --iat US [--dist exp|ln] [--ln_sigma X] --concurrency C --num_jobs N [--start_record_num R]\n"
-                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] job.so proportion max_outstanding ...\n", argv[0]);
+                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] [--trace FILE] job.so proportion max_outstanding ...\n", argv[0]);
         return 2;
     }
 

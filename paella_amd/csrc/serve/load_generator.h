@@ -64,6 +64,7 @@ struct Options {
     unsigned num_jobs = 0, start_record_num = 0, seed = 1, sched_sleep = 0;
     unsigned warmup_jobs = 0;  // extra requests served (same arrival process) before the measured ones
     bool pin_threads = true;
+    std::string trace_path;      // non-empty: replay "<type> <submit time us>" lines (llis_app_workload_pregen) instead of drawing
     std::string profile_prefix;  // non-empty: the server records everything during the measured phase and saves to this prefix
     // name-shaping switches (which parameters appear in the output file names, which one is the x column)
     bool n_iat = false, n_lns = false, n_con = false, n_n = false, n_srn = false, n_seed = false, n_fair = false, n_scheds = false;
@@ -192,7 +193,20 @@ class LoadGenerator {
         std::uniform_real_distribution<float> d_type(0, 1);
         const bool use_exp = opt_.dist == "exp";
 
-        double next_submit = 0;
+        // A pre-generated trace replaces the draws: request i is of trace_[i].first and due at trace_[i].second.
+        if (!opt_.trace_path.empty() && trace_.empty()) {
+            if (FILE* fp = std::fopen(opt_.trace_path.c_str(), "r")) {
+                unsigned type;
+                double when;
+                while (std::fscanf(fp, "%u %lf", &type, &when) == 2) trace_.emplace_back(type, when);
+                std::fclose(fp);
+            }
+            if (trace_.empty()) throw std::runtime_error("cannot read arrival trace " + opt_.trace_path);
+        }
+        const bool replay = !trace_.empty();
+        size_t trace_pos = 0;
+
+        double next_submit = replay ? trace_[0].second : 0;
         start_time_ = Clock::now();
         const double start_us = us_since_epoch(start_time_);
         unsigned submitted = 0;
@@ -206,7 +220,8 @@ class LoadGenerator {
                 while (num_outstanding_.load(std::memory_order_acquire) >= opt_.concurrency) {
                 }
             }
-            const unsigned type = (unsigned)(std::lower_bound(props_cum_.begin(), props_cum_.end(), d_type(gen)) - props_cum_.begin());
+            const unsigned type = replay ? trace_[trace_pos % trace_.size()].first
+                                         : (unsigned)(std::lower_bound(props_cum_.begin(), props_cum_.end(), d_type(gen)) - props_cum_.begin());
             const unsigned t = std::min<unsigned>(type, (unsigned)props_cum_.size() - 1);
             {
                 std::lock_guard<std::mutex> lk(mtx_);
@@ -220,7 +235,14 @@ class LoadGenerator {
             }
             num_outstanding_.fetch_add(1, std::memory_order_release);
             ++submitted;
-            if (opt_.iat > 0) next_submit += use_exp ? d_exp(gen) : d_ln(gen);
+            if (replay) {
+                // the trace wraps around (shifted by its own span) when more requests are asked for than it holds
+                ++trace_pos;
+                const double span = trace_.back().second + (trace_.size() > 1 ? trace_.back().second / (double)(trace_.size() - 1) : 0);
+                next_submit = trace_[trace_pos % trace_.size()].second + span * (double)(trace_pos / trace_.size());
+            } else if (opt_.iat > 0) {
+                next_submit += use_exp ? d_exp(gen) : d_ln(gen);
+            }
         }
     }
 
@@ -236,6 +258,7 @@ class LoadGenerator {
     std::vector<unsigned> outstanding_per_type_;
     std::atomic<int> num_outstanding_{0};
 
+    std::vector<std::pair<unsigned, double>> trace_;
     std::vector<double> latencies_;
     std::vector<std::vector<double>> latencies_per_type_;
     std::vector<unsigned> timeline_;

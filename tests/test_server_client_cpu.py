@@ -95,6 +95,36 @@ def test_arrival_process_is_reproducible_for_a_seed():
     assert counts[0] == counts[1] and abs(counts[0][0] - 100) < 40
 
 
+def test_pregenerated_trace_matches_the_live_arrival_process(tmp_path):
+    """llis_app_workload_pregen makes the same draws in the same order as the live generator (type first, then the
+    gap), writes the reference's file set, and a replay of its trace serves the same request mix."""
+    pre = subprocess.run([os.path.join(BIN, "llis_app_workload_pregen"), "--iat", "150", "--ln_sigma", "1.5", "--num_jobs", "300", "--seed", "7",
+                          "--pregen_prefix", str(tmp_path / "w"), "0.25", "0.75"], capture_output=True, text=True, timeout=60)
+    assert pre.returncode == 0, pre.stderr
+    trace_path = pre.stdout.strip()
+    assert os.path.basename(trace_path) == "w_iat150_lns1.5_n300_seed7.txt"
+    trace = [l.split() for l in open(trace_path)]
+    assert len(trace) == 300 and trace[0][1] == "0.000000"
+    times = [float(l[1]) for l in trace]
+    assert times == sorted(times) and 0.5 * 150 < times[-1] / 299 < 2.0 * 150
+    for t in (0, 1):
+        own = [l.split() for l in open(trace_path.replace(".txt", "_job%d.txt" % t))]
+        assert [l[1] for l in own] == [l[1] for l in trace if l[0] == str(t)] and all(l[0] == "0" for l in own)
+    counts = []
+    for mode in ("live", "trace"):
+        name = "pttr%d_%s" % (os.getpid(), mode)
+        srv = start_server(name, "fifo2")
+        extra = ["--trace", trace_path] if mode == "trace" else []
+        out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "150", "--dist", "ln", "--ln_sigma", "1.5",
+                              "--concurrency", "32", "--num_jobs", "300", "--seed", "7", "--prefix", str(tmp_path / mode), "--no_pin"] + extra +
+                             [fake_job("fake_short"), "0.25", "16", fake_job("fake_mem3"), "0.75", "16"],
+                             env=fake_env(), capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert srv.wait(timeout=30) == 0
+        counts.append(json.loads(out.stdout.strip().splitlines()[-1])["per_type_count"])
+    assert counts[0] == counts[1] == [sum(l[0] == "0" for l in trace), sum(l[0] == "1" for l in trace)]
+
+
 def test_unknown_scheduler_is_an_error_not_a_crash():
     out = subprocess.run([os.path.join(BIN, "llis_server"), "--name", "x", "--sched", "nope"], env=fake_env(), capture_output=True, text=True, timeout=30)
     assert out.returncode == 4 and "unknown scheduler" in out.stderr and "full3" in out.stderr
