@@ -41,6 +41,9 @@ const char* paella_model_names(void);
 int paella_model_io_bytes(const char* name, size_t* in_bytes, size_t* out_bytes);
 /* JSON description of the graph (buffers, weight tensors with stream/std/shape, nodes in stage order).
  * Writes at most cap bytes including the terminating NUL; *needed gets the full size. */
+/* Writes the I/O-shape sidecar of a model: input dims, -1, output dims, one per line (the format of the
+ * reference's sosp23_artifact/tvm_models_dim/<model>.dim). */
+int paella_model_write_dim(const char* name, const char* path);
 int paella_model_describe(const char* name, char* json, size_t cap, size_t* needed);
 /* Algorithmic totals of one forward pass. */
 int paella_model_totals(const char* name, double* macs, double* params, double* flops, double* bytes, int* stages);

@@ -23,6 +23,7 @@ MODEL_SYMBOLS = {
     "paella_exec_output": (c_void_p, [c_void_p]),
     "paella_exec_launch_stage": (c_int, [c_void_p, c_int, c_void_p, c_u32, c_void_p]),
     "paella_exec_forward": (c_int, [c_void_p, c_void_p]),
+    "paella_model_write_dim": (c_int, [ctypes.c_char_p, ctypes.c_char_p]),
 }
 
 

@@ -197,6 +197,19 @@ int paella_model_io_bytes(const char* name, size_t* in_bytes, size_t* out_bytes)
     return 0;
 }
 
+int paella_model_write_dim(const char* name, const char* path) {
+    const Graph* g = graph_of(name);
+    if (!g || !path) return PAELLA_EINVAL;
+    FILE* fp = std::fopen(path, "w");
+    if (!fp) return PAELLA_EINVAL;
+    // input dims, -1, output dims, one number per line (the sidecar the reference keeps next to each compiled
+    // model, reference sosp23_artifact/tvm_models_dim/*.dim); outputs without spatial extent are written as N x C
+    std::fprintf(fp, "1\n%d\n%d\n%d\n-1\n1\n%d\n", g->input.C, g->input.H, g->input.W, g->output.C);
+    if (g->output.H * g->output.W != 1) std::fprintf(fp, "%d\n%d\n", g->output.H, g->output.W);
+    std::fclose(fp);
+    return 0;
+}
+
 int paella_model_describe(const char* name, char* json, size_t cap, size_t* needed) {
     const Graph* g = graph_of(name);
     if (!g) return PAELLA_EINVAL;

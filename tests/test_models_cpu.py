@@ -91,3 +91,32 @@ def test_resnet18_oracle_equals_independent_torch_graph():
     got = om.run(desc, x, seed=2)
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4)
     assert np.abs(ref).max() > 0.1 and np.abs(ref).max() < 1e3
+
+
+def test_io_shapes_match_the_reference_dim_sidecars(tmp_path):
+    """The reference ships one .dim file per compiled model (input dims, -1, output dims).  The zoo's models must
+    have the same I/O shapes -- except Inception-v3, which the reference compiled at 224x224 and which is served
+    at 299x299 here on purpose (the BASELINE configuration) -- and paella_model_write_dim must reproduce the format."""
+    import json
+    import os
+    from paella_amd import _abi, models
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "tvm_models_dim.json")))["files"]
+    ours = {"densenet-9": "densenet121", "googlenet-9": "googlenet", "inception_v3": "inception_v3", "mnist-8": "mnist",
+            "mobilenetv2-7": "mobilenetv2", "resnet18-v2-7": "resnet18", "resnet34-v2-7": "resnet34", "resnet50-v2-7": "resnet50",
+            "squeezenet1.1-7": "squeezenet1_1"}
+    assert len(golden) == 9
+    for fname, dims in golden.items():
+        model = ours[fname.replace("-cuda-pack.so.dim", "")]
+        in_bytes, out_bytes = models.io_bytes(model)
+        want_in = list(dims["input"])
+        if model == "inception_v3":
+            assert want_in == [1, 3, 224, 224]
+            want_in = [1, 3, 299, 299]
+        assert in_bytes == 4 * int(np.prod(want_in)), model
+        assert out_bytes == 4 * int(np.prod(dims["output"])), model
+        path = str(tmp_path / (model + ".dim"))
+        assert _abi.ops().paella_model_write_dim(model.encode(), path.encode()) == 0
+        vals = [int(v) for v in open(path).read().split()]
+        cut = vals.index(-1)
+        assert vals[:cut] == want_in
+        assert int(np.prod(vals[cut + 1:])) == int(np.prod(dims["output"])) and vals[cut + 1:cut + 3] == dims["output"][:2]
