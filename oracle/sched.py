@@ -11,7 +11,7 @@ Restates (reference paths):
   Job counters    include/llis/job/job.h:138-191,278-292
 Pools of streams, notifiers and job ids are LIFO (scheduler_full3.cpp:206-207,280-287,391-396).
 
-Deliberate deviations shared with the product (documented in DESIGN.md): a stage whose length is not yet
+Deliberate deviations shared with the product: a stage whose length is not yet
 in the job's snapshot counts as zero remaining work (the reference indexes past the end of the snapshot);
 a job without stages is released without touching the id pool.
 

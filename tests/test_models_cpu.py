@@ -96,7 +96,7 @@ def test_resnet18_oracle_equals_independent_torch_graph():
 def test_io_shapes_match_the_reference_dim_sidecars(tmp_path):
     """The reference ships one .dim file per compiled model (input dims, -1, output dims).  The zoo's models must
     have the same I/O shapes -- except Inception-v3, which the reference compiled at 224x224 and which is served
-    at 299x299 here on purpose (the BASELINE configuration) -- and paella_model_write_dim must reproduce the format."""
+    at 299x299 here on purpose (the benchmark configuration) -- and paella_model_write_dim must reproduce the format."""
     import json
     import os
     from paella_amd import _abi, models

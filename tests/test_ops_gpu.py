@@ -27,7 +27,7 @@ def close(got, ref):
     assert np.all(err <= bound), "max err %g (bound there %g), %d bad of %d" % (err.max(), bound.flat[err.argmax()], (err > bound).sum(), err.size)
 
 
-# C, H, W, K, R, S, stride, pad, dil  -- the layer shapes of the BASELINE configs plus ragged edge cases
+# C, H, W, K, R, S, stride, pad, dil  -- the layer shapes of the benchmark models plus ragged edge cases
 CONV_SHAPES = [
     (1, 28, 28, 8, 5, 5, 1, 2, 1),          # small CNN conv1
     (8, 14, 14, 16, 5, 5, 1, 2, 1),         # small CNN conv2
@@ -190,7 +190,7 @@ def test_global_avgpool_eltwise_copy_softmax_lrn_parity(cuda):
 
 
 def test_conv_linearity_at_full_size(cuda):
-    """Size-independent property at a BASELINE-sized layer: conv(x, w1 + w2) == conv(x, w1) + conv(x, w2)."""
+    """Size-independent property at a full-size layer: conv(x, w1 + w2) == conv(x, w1) + conv(x, w2)."""
     from paella_amd import ops
     x = torch.tensor(rnd(1, 64, 112, 112), device=cuda)
     w1, w2 = rnd(64, 64, 3, 3, scale=0.05), rnd(64, 64, 3, 3, scale=0.05)
