@@ -8,8 +8,8 @@ computed here, independently of the GPU path.
 What it restates: the forward pass the reference obtains from `run_()` of a TVM-compiled model
 (reference jobs/tvm_mnist/tvm_mnist.cpp:41).  Pinning: the reference has no numeric outputs for any model,
 so (a) the operators are pinned in tests/test_oracle_ops.py, (b) the topologies are pinned through their
-published multiply-accumulate and parameter counts and, for the small CNN and ResNet-18, through an
-independent torch.nn.functional restatement in tests/test_models_cpu.py.
+published multiply-accumulate and parameter counts and through an independent torch.nn.functional
+restatement of each of the eleven models in tests/test_models_cpu.py.
 """
 import numpy as np
 

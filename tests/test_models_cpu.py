@@ -1,5 +1,5 @@
 """Model zoo on the CPU: topology totals against published counts, the seeded generator of the product against
-the oracle's, and an independent torch restatement of the small CNN and ResNet-18 against the oracle."""
+the oracle's, and an independent torch restatement of every model of the zoo against the oracle."""
 import numpy as np
 import pytest
 import torch
@@ -91,6 +91,241 @@ def test_resnet18_oracle_equals_independent_torch_graph():
     got = om.run(desc, x, seed=2)
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4)
     assert np.abs(ref).max() > 0.1 and np.abs(ref).max() < 1e3
+
+
+def _resnet_reference(name, bottleneck, layers, seed=2):
+    """Textbook ResNet (v1.5 bottleneck: the stride sits on the 3x3) written directly in torch; weights are taken
+    in the zoo's creation order: shortcut projection first, then the block's convs."""
+    desc = om.Desc(models.describe(name))
+    w = iter(_w(desc, seed))
+    nxt = lambda: next(w).double()
+    x = om.make_input(desc.d, 4)
+    t = torch.tensor(x).double()
+    t = F.max_pool2d(F.relu(F.conv2d(t, nxt(), nxt(), stride=2, padding=3)), 3, 2, 1)
+    for stage, planes in enumerate([64, 128, 256, 512]):
+        for block in range(layers[stage]):
+            stride = 2 if (stage > 0 and block == 0) else 1
+            out_ch = planes * (4 if bottleneck else 1)
+            identity = t
+            if stride != 1 or t.shape[1] != out_ch:
+                identity = F.conv2d(t, nxt(), nxt(), stride=stride)
+            if bottleneck:
+                y = F.relu(F.conv2d(t, nxt(), nxt()))
+                y = F.relu(F.conv2d(y, nxt(), nxt(), stride=stride, padding=1))
+                t = F.relu(F.conv2d(y, nxt(), nxt()) + identity)
+            else:
+                y = F.relu(F.conv2d(t, nxt(), nxt(), stride=stride, padding=1))
+                t = F.relu(F.conv2d(y, nxt(), nxt(), padding=1) + identity)
+    ref = F.linear(F.adaptive_avg_pool2d(t, 1).flatten(1), nxt(), nxt()).float().numpy().reshape(-1)
+    assert next(w, None) is None
+    return desc, x, ref
+
+
+@pytest.mark.parametrize("name,bottleneck,layers", [("resnet34", False, [3, 4, 6, 3]), ("resnet50", True, [3, 4, 6, 3])])
+def test_deeper_resnets_equal_independent_torch_graphs(name, bottleneck, layers):
+    desc, x, ref = _resnet_reference(name, bottleneck, layers)
+    np.testing.assert_allclose(om.run(desc, x, seed=2), ref, rtol=1e-4, atol=1e-4)
+    assert 0.05 < np.abs(ref).max() < 1e3
+
+
+def test_squeezenet_equals_independent_torch_graph():
+    desc = om.Desc(models.describe("squeezenet1_1"))
+    w = iter(_w(desc, 2))
+    nxt = lambda: next(w).double()
+    x = om.make_input(desc.d, 4)
+    t = torch.tensor(x).double()
+
+    def fire(t):
+        s = F.relu(F.conv2d(t, nxt(), nxt()))
+        return torch.cat([F.relu(F.conv2d(s, nxt(), nxt())), F.relu(F.conv2d(s, nxt(), nxt(), padding=1))], 1)
+
+    t = F.max_pool2d(F.relu(F.conv2d(t, nxt(), nxt(), stride=2)), 3, 2, ceil_mode=True)
+    t = fire(fire(t))
+    t = F.max_pool2d(t, 3, 2, ceil_mode=True)
+    t = fire(fire(t))
+    t = F.max_pool2d(t, 3, 2, ceil_mode=True)
+    t = fire(fire(fire(fire(t))))
+    assert t.shape == (1, 512, 13, 13)
+    ref = F.adaptive_avg_pool2d(F.relu(F.conv2d(t, nxt(), nxt())), 1).float().numpy().reshape(-1)
+    assert next(w, None) is None
+    np.testing.assert_allclose(om.run(desc, x, seed=2), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_mobilenetv2_equals_independent_torch_graph():
+    desc = om.Desc(models.describe("mobilenetv2"))
+    w = iter(_w(desc, 2))
+    nxt = lambda: next(w).double()
+    x = om.make_input(desc.d, 4)
+    t = torch.tensor(x).double()
+    relu6 = lambda v: torch.clamp(v, 0.0, 6.0)
+    t = relu6(F.conv2d(t, nxt(), nxt(), stride=2, padding=1))
+    for expand, out_ch, repeats, first_stride in [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]:
+        for i in range(repeats):
+            stride = first_stride if i == 0 else 1
+            y = t
+            if expand != 1:
+                y = relu6(F.conv2d(y, nxt(), nxt()))
+            y = relu6(F.conv2d(y, nxt(), nxt(), stride=stride, padding=1, groups=y.shape[1]))
+            y = F.conv2d(y, nxt(), nxt())
+            t = t + y if (stride == 1 and t.shape[1] == out_ch) else y
+    t = relu6(F.conv2d(t, nxt(), nxt()))
+    assert t.shape == (1, 1280, 7, 7)
+    ref = F.linear(F.adaptive_avg_pool2d(t, 1).flatten(1), nxt(), nxt()).float().numpy().reshape(-1)
+    assert next(w, None) is None
+    np.testing.assert_allclose(om.run(desc, x, seed=2), ref, rtol=1e-4, atol=1e-4)
+
+
+class _Torch:
+    """Weight cursor + the handful of layer shorthands the independent graphs below share."""
+
+    def __init__(self, name, seed=2):
+        self.desc = om.Desc(models.describe(name))
+        self._w = iter(_w(self.desc, seed))
+        self.x = om.make_input(self.desc.d, 4)
+        self.t = torch.tensor(self.x).double()
+
+    def nxt(self):
+        return next(self._w).double()
+
+    def conv(self, t, stride=1, padding=0, act=F.relu, groups=1):
+        y = F.conv2d(t, self.nxt(), self.nxt(), stride=stride, padding=padding, groups=groups)
+        return act(y) if act else y
+
+    def norm(self, t, act=F.relu):
+        y = t * self.nxt().view(1, -1, 1, 1) + self.nxt().view(1, -1, 1, 1)
+        return act(y) if act else y
+
+    def dense(self, t):
+        return F.linear(t.flatten(1), self.nxt(), self.nxt())
+
+    def check(self, ref, rtol=1e-4, atol=1e-4):
+        assert next(self._w, None) is None
+        ref = ref.float().numpy().reshape(-1)
+        np.testing.assert_allclose(om.run(self.desc, self.x, seed=2), ref, rtol=rtol, atol=atol)
+        assert np.isfinite(ref).all() and np.abs(ref).max() > 1e-4
+
+
+def test_googlenet_equals_independent_torch_graph():
+    g = _Torch("googlenet")
+    lrn = lambda t: F.local_response_norm(t, 5, alpha=1e-4, beta=0.75, k=1.0)
+    pool = lambda t: F.max_pool2d(t, 3, 2, ceil_mode=True)
+
+    def inception(t):
+        b1 = g.conv(t)
+        b3 = g.conv(g.conv(t), padding=1)
+        b5 = g.conv(g.conv(t), padding=2)
+        bp = g.conv(F.max_pool2d(t, 3, 1, 1))
+        return torch.cat([b1, b3, b5, bp], 1)
+
+    t = lrn(pool(g.conv(g.t, stride=2, padding=3)))
+    t = pool(lrn(g.conv(g.conv(t), padding=1)))
+    t = pool(inception(inception(t)))
+    assert t.shape == (1, 480, 14, 14)
+    for _ in range(5):
+        t = inception(t)
+    t = inception(inception(pool(t)))
+    assert t.shape == (1, 1024, 7, 7)
+    g.check(F.softmax(g.dense(F.adaptive_avg_pool2d(t, 1)), 1), atol=1e-6)
+
+
+def test_densenet121_equals_independent_torch_graph():
+    g = _Torch("densenet121")
+    t = F.max_pool2d(g.conv(g.t, stride=2, padding=3), 3, 2, 1)
+    for stage, layers in enumerate([6, 12, 24, 16]):
+        for _ in range(layers):
+            y = g.conv(g.norm(t))
+            t = torch.cat([t, g.conv(y, padding=1, act=None)], 1)
+        if stage < 3:
+            t = F.avg_pool2d(g.conv(g.norm(t), act=None), 2, 2)
+    assert t.shape == (1, 1024, 7, 7)
+    g.check(g.dense(F.adaptive_avg_pool2d(g.norm(t), 1)))
+
+
+def test_inception_v3_equals_independent_torch_graph():
+    g = _Torch("inception_v3")
+    avg = lambda t: F.avg_pool2d(t, 3, 1, 1)
+
+    def block_a(t):
+        b1 = g.conv(t)
+        b5 = g.conv(g.conv(t), padding=2)
+        b3 = g.conv(g.conv(g.conv(t), padding=1), padding=1)
+        return torch.cat([b1, b5, b3, g.conv(avg(t))], 1)
+
+    def block_b(t):
+        b3 = g.conv(t, stride=2)
+        bd = g.conv(g.conv(g.conv(t), padding=1), stride=2)
+        return torch.cat([b3, bd, F.max_pool2d(t, 3, 2)], 1)
+
+    def block_c(t):
+        b1 = g.conv(t)
+        b7 = g.conv(g.conv(g.conv(t), padding=(0, 3)), padding=(3, 0))
+        bd = g.conv(t)
+        for pad in [(3, 0), (0, 3), (3, 0), (0, 3)]:
+            bd = g.conv(bd, padding=pad)
+        return torch.cat([b1, b7, bd, g.conv(avg(t))], 1)
+
+    def block_d(t):
+        b3 = g.conv(g.conv(t), stride=2)
+        b7 = g.conv(g.conv(g.conv(g.conv(t), padding=(0, 3)), padding=(3, 0)), stride=2)
+        return torch.cat([b3, b7, F.max_pool2d(t, 3, 2)], 1)
+
+    def block_e(t):
+        b1 = g.conv(t)
+        y = g.conv(t)
+        b3 = [g.conv(y, padding=(0, 1)), g.conv(y, padding=(1, 0))]
+        y = g.conv(g.conv(t), padding=1)
+        bd = [g.conv(y, padding=(0, 1)), g.conv(y, padding=(1, 0))]
+        return torch.cat([b1] + b3 + bd + [g.conv(avg(t))], 1)
+
+    t = g.conv(g.conv(g.conv(g.t, stride=2)), padding=1)
+    t = F.max_pool2d(t, 3, 2)
+    t = F.max_pool2d(g.conv(g.conv(t)), 3, 2)
+    assert t.shape == (1, 192, 35, 35)
+    t = block_b(block_a(block_a(block_a(t))))
+    assert t.shape == (1, 768, 17, 17)
+    t = block_d(block_c(block_c(block_c(block_c(t)))))
+    t = block_e(block_e(t))
+    assert t.shape == (1, 2048, 8, 8)
+    g.check(g.dense(F.adaptive_avg_pool2d(t, 1)))
+
+
+def test_face_embedding_resnet100_equals_independent_torch_graph():
+    g = _Torch("arcfaceresnet100")
+
+    def conv_prelu(t, **kw):
+        w, b, slope = g.nxt(), g.nxt(), g.nxt()
+        return F.prelu(F.conv2d(t, w, b, **kw), slope)
+
+    t = conv_prelu(g.t, padding=1)
+    for units in [3, 13, 30, 3]:
+        for i in range(units):
+            stride = 2 if i == 0 else 1
+            shortcut = g.conv(t, stride=stride, act=None) if i == 0 else t
+            y = conv_prelu(g.norm(t, act=None), padding=1)
+            t = g.conv(y, stride=stride, padding=1, act=None) + shortcut
+    assert t.shape == (1, 512, 7, 7)
+    g.check(g.dense(g.norm(t, act=None)))
+
+
+def test_face_detector_scores_equal_independent_torch_graph():
+    g = _Torch("ultraface320")
+
+    def separable(t, stride=1, act=F.relu):
+        return g.conv(g.conv(t, stride=stride, padding=1, groups=t.shape[1]), act=act)
+
+    t = g.conv(g.t, stride=2, padding=1)
+    feats = []
+    for strides in [[1, 2, 1, 2, 1, 1, 1], [2, 1, 1], [2, 1]]:
+        for s in strides:
+            t = separable(t, s)
+        feats.append(t)
+    t = g.conv(g.conv(g.conv(t), stride=2, padding=1, groups=64))
+    feats.append(t)
+    assert [tuple(f.shape[1:]) for f in feats] == [(64, 30, 40), (128, 15, 20), (256, 8, 10), (256, 4, 5)]
+    # each head's [anchors*2][H][W] logits are laid flat one after the other; prior r is the pair (2r, 2r+1)
+    logits = torch.cat([separable(f, act=None).reshape(-1) for f in feats])
+    assert logits.numel() == 4420 * 2
+    g.check(F.softmax(logits.view(4420, 2), 1), atol=1e-6)
 
 
 def test_io_shapes_match_the_reference_dim_sidecars(tmp_path):
