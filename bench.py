@@ -39,9 +39,9 @@ def log(*a):
 CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 6.21e6}
 
 
-def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2):
+def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2, unfair=1e6):
     name = "bench%d_%s_%d" % (os.getpid(), sched, int(time.time() * 1000) % 100000)
-    with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4, extra_kernels=extra_kernels) as srv:
+    with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4, extra_kernels=extra_kernels, unfair=unfair) as srv:
         r = serve.client_run(srv.name, jobs, iat_us, concurrency, steps, warmup_jobs=warmup, seed=seed, dist="exp", pin_threads=True)
     return r
 
@@ -157,6 +157,8 @@ def main():
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mix", action="store_true", help="skip the small-CNN + Inception-v3 two-tenant arm")
+    ap.add_argument("--fairness-sweep", action="store_true",
+                    help="also sweep full3's deficit threshold over a ResNet-18 : Inception-v3 = 0.952 : 0.048 mix and report Jain's index")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel over a 64 MiB buffer five times (reference point for memory-traffic counters)")
     ap.add_argument("--roofline-only", action="store_true",
@@ -250,6 +252,45 @@ def main():
                 (rate, point["full3"]["small_cnn_p99_us"], point["full3"]["inception_v3_p99_us"],
                  point["fifo_multi_stream"]["small_cnn_p99_us"], point["fifo_multi_stream"]["inception_v3_p99_us"]))
 
+    # One client, one request at a time, small CNN, 10 000 requests, every request with its host-to-device and
+    # device-to-host copy: the latency floor of the full path (7 stages: 2 copies + 5 kernels, each with its notifications).
+    closed_loop = None
+    if not args.no_arms:
+        import numpy as np
+        os.environ["PAELLA_INPUT_RESIDENT"] = "0"
+        name = "bench%d_closed_%d" % (os.getpid(), int(time.time() * 1000) % 100000)
+        x = np.random.default_rng(1).random((1, 1, 28, 28), dtype=np.float32)
+        with serve.Server(name, "full3", num_streams=args.num_streams, cpu=4, extra_kernels=args.extra_kernels) as srv:
+            serve.client_single(srv.name, serve.job_path("tvm_mnist"), x, 10, n=500)
+            _, lat = serve.client_single(srv.name, serve.job_path("tvm_mnist"), x, 10, n=10000)
+        os.environ["PAELLA_INPUT_RESIDENT"] = "1"
+        lat = np.sort(lat)
+        closed_loop = {"workload": "small CNN 1x1x28x28, one client, one request outstanding, 10000 requests, copies included",
+                       "stages_per_request": models.totals("mnist")["stages"] + 2,
+                       "mean_us": float(lat.mean()), "p50_us": float(lat[len(lat) // 2]), "p99_us": float(lat[int(len(lat) * 0.99)]),
+                       "us_per_stage": float(lat.mean()) / (models.totals("mnist")["stages"] + 2)}
+        log("[bench]   small CNN closed loop: mean %.1f us, p50 %.1f us, p99 %.1f us per request (%d stages)" %
+            (closed_loop["mean_us"], closed_loop["p50_us"], closed_loop["p99_us"], closed_loop["stages_per_request"]))
+
+    # Deficit-threshold sweep over a two-model mix at saturation: latency of each model in the mix over its
+    # latency when served alone, and Jain's index over those slowdowns.
+    fairness_sweep = None
+    if args.fairness_sweep:
+        from paella_amd import fairness
+        fjobs = [(serve.job_path("tvm_resnet18"), 0.952, 119), (serve.job_path("tvm_inception_v3"), 0.048, 6)]
+        alone = []
+        for path, prop, cap in fjobs:
+            r = serve_arm(serve, "full3", args.num_streams, [(path, 1.0, cap)], cap, int(3000 * prop) + 1, 200, extra_kernels=args.extra_kernels)
+            alone.append(r["all"]["mean"])
+        fairness_sweep = {"workload": "ResNet-18 : Inception-v3 = 0.952 : 0.048, 119 + 6 outstanding, 3000 requests at saturation",
+                          "alone_mean_latency_us": alone, "points": []}
+        for f in (0.01, 1.0, 10.0, 50.0, 100.0, 500.0, 1000.0, 100000.0):
+            r = serve_arm(serve, "full3", args.num_streams, fjobs, 125, 3000, 300, extra_kernels=args.extra_kernels, unfair=f)
+            slow = [r["per_type"][i]["mean"] / alone[i] for i in range(2)]
+            fairness_sweep["points"].append({"unfair": f, "requests_per_s": r["throughput_rps"], "slowdown": slow, "jain_index": float(fairness.jain_index(slow))})
+            log("[bench]   unfair %-9g %.0f req/s, slowdown ResNet-18 %.2f, Inception-v3 %.2f, Jain index %.3f" %
+                (f, r["throughput_rps"], slow[0], slow[1], fairness_sweep["points"][-1]["jain_index"]))
+
     log("[bench] per-launch timing of the forward pass (kernel begin/end timestamps through HIP events)")
     rl = conv_roofline(models, hip, args.model, reps=50)
     achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
@@ -290,6 +331,25 @@ def main():
         if lib.paella_ring_bench_pingpong(100, 2000, ctypes.byref(flag), ctypes.byref(sync), None) == 0:
             notify["launch_plus_flag_store_us"] = flag.value
             notify["launch_plus_stream_sync_us"] = sync.value
+        # resident lane answering host pings through the ring: no launch in the way
+        import numpy as np
+        n_echo = 5000
+        rtt, one_way = np.zeros(n_echo), np.zeros(n_echo)
+        if lib.paella_ring_bench_echo(ring, 500, n_echo, rtt.ctypes.data, one_way.ctypes.data) == 0:
+            rtt.sort()
+            notify["echo_round_trip_us"] = {"p50": float(rtt[n_echo // 2]), "p99": float(rtt[int(n_echo * 0.99)]),
+                                            "what": "host flag store -> resident lane sees it -> ring message readable on the host"}
+            ow = np.sort(one_way[one_way > -1e29])
+            if len(ow):
+                # The translation interpolates between clock pairs the runtime samples itself and is good to a
+                # microsecond or two: a figure outside (0, round trip) says so.  The round trip is the hard bound.
+                notify["device_to_host_us_clock_translated"] = {
+                    "p50": float(ow[len(ow) // 2]), "p99": float(ow[int(len(ow) * 0.99)]),
+                    "inside_round_trip": bool(0.0 < ow[len(ow) // 2] < rtt[n_echo // 2]),
+                    "what": "host clock when the message became readable minus the lane's realtime counter just before the ring write, "
+                            "translated to the host clock by the runtime"}
+            log("[bench]   notification: echo round trip p50 %.2f / p99 %.2f us%s" % (rtt[n_echo // 2], rtt[int(n_echo * 0.99)],
+                ", device->host p50 %.2f / p99 %.2f us" % (ow[len(ow) // 2], ow[int(len(ow) * 0.99)]) if len(ow) else ""))
         lib.paella_ring_destroy(ring)
 
     cpu = None if args.no_cpu else cpu_baseline(args.model, args.cpu_seconds)
@@ -320,6 +380,8 @@ def main():
         "arms": arms,
         "poisson_sweep": sweep,
         "two_tenant_mix": mix,
+        "small_cnn_closed_loop": closed_loop,
+        "fairness_sweep": fairness_sweep,
         "direct_single_stream_rps": rl["direct_rps"],
         # per operator family, one forward pass, isolated launches: time, algorithmic work, and the rates they imply
         "per_op_us": {k: {"launches": v["launches"], "us": v["us"], "gflop": v["flops"] / 1e9, "mbytes": v["bytes"] / 1e6,

@@ -52,6 +52,15 @@ int paella_ring_bench_drain(paella_ring* ring, unsigned blocks, unsigned vec_len
                             double* us_per_iter);
 int paella_ring_bench_pingpong(int warmup, int iters, double* flag_us, double* sync_us, double* flag_samples_us);
 
+/* One-way notification latency without a kernel launch in the way (the reference has no counterpart; its probes
+ * above include the launch).  A resident one-lane kernel answers warmup + iters host pings: for each, the host
+ * raises a flag in host memory, the lane sees it, reads the device's realtime counter and sends one ring message.
+ *   round_trip_us[i]  host flag store -> message readable on the host (upper bound of the notification latency)
+ *   gpu_to_host_us[i] (may be NULL) host time at which the message became readable minus the lane's counter value
+ *                     translated to the host's clock by the runtime; -1e30 where the translation is unavailable.
+ * Both arrays hold `iters` doubles.  The lane's wait is bounded (20 s of device time) and ends early on error. */
+int paella_ring_bench_echo(paella_ring* ring, int warmup, int iters, double* round_trip_us, double* gpu_to_host_us);
+
 /* Sustained fp32 MFMA rate of the device (v_mfma_f32_32x32x2_f32, register-resident operands, every SIMD busy):
  * the measured denominator next to the published 157.3 TFLOP/s. */
 int paella_mfma_peak_probe(double* tflops);

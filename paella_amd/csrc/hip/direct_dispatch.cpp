@@ -302,6 +302,18 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     hsa_signal_store_screlease(hq->doorbell_signal, (hsa_signal_value_t)index);
 }
 
+bool direct_system_clock(uint64_t* now_ticks, uint64_t* ticks_per_second) {
+    if (!ensure_runtime()) return false;
+    if (now_ticks && hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP, now_ticks) != HSA_STATUS_SUCCESS) return false;
+    if (ticks_per_second && hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, ticks_per_second) != HSA_STATUS_SUCCESS) return false;
+    return true;
+}
+
+bool direct_device_tick_to_system(uint64_t device_tick, uint64_t* system_tick) {
+    if (!ensure_runtime() || !system_tick) return false;
+    return hsa_amd_profiling_convert_tick_to_system_domain(g_rt.gpu, device_tick, system_tick) == HSA_STATUS_SUCCESS;
+}
+
 }  // namespace paella
 
 // ---- C-ABI --------------------------------------------------------------------------------------

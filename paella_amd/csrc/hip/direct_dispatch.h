@@ -57,4 +57,10 @@ inline void pack_args(char* buf, size_t& offset, const T& first, const Rest&... 
 
 constexpr size_t kMaxExplicitArgBytes = 256;
 
+// Clock bridge for latency probes: the host's reading of the system timestamp, its frequency, and the
+// translation of a device realtime-counter value (what wall_clock64() returns in a kernel) into that domain.
+// False if the runtime is unavailable.
+bool direct_system_clock(uint64_t* now_ticks, uint64_t* ticks_per_second);
+bool direct_device_tick_to_system(uint64_t device_tick, uint64_t* system_tick);
+
 }  // namespace paella

@@ -7,6 +7,7 @@
 #include <new>
 #include <vector>
 
+#include "direct_dispatch.h"
 #include "paella_hip.h"
 #include "paella_ring.h"
 #include <llis/ipc/shm_primitive_channel.h>
@@ -80,6 +81,26 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(float* sink, int iters) 
 }
 
 __global__ void flag_kernel(int* flag) { __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM); }
+
+// One lane answers `total` host pings: waits (bounded by a tick budget, and by a negative value of the flag) until
+// the host has raised *go above i, reads the realtime counter, sends one ring message, keeps the counter value.
+__global__ void echo_kernel(Gpu2SchedChannel channel, const int* go, unsigned long long* stamps, int total, unsigned long long budget_ticks) {
+    const unsigned long long t_start = wall_clock64();
+    for (int i = 0; i < total; ++i) {
+        for (;;) {
+            const int seen = __hip_atomic_load(go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (seen > i) break;
+            if (seen < 0 || wall_clock64() - t_start > budget_ticks) return;
+        }
+        const unsigned long long g = wall_clock64();
+        InstrumentInfo info;
+        info.is_start = 0;
+        info.num = 1;
+        info.job_id = (llis::JobId)(i & 0xFFFF);
+        channel.write(info);
+        stamps[i] = g;
+    }
+}
 
 double now_us() {
     return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -218,6 +239,65 @@ int paella_ring_bench_pingpong(int warmup, int iters, double* flag_us, double* s
     hipStreamSynchronize(st);
     hipStreamDestroy(st);
     llis_hip_host_free(flag);
+    return 0;
+}
+
+int paella_ring_bench_echo(paella_ring* r, int warmup, int iters, double* round_trip_us, double* gpu_to_host_us) {
+    if (!r || warmup < 0 || iters <= 0 || iters + warmup > 200000 || !round_trip_us) return -1;
+    const int total = warmup + iters;
+    uint64_t hz = 0;
+    const bool have_clock = paella::direct_system_clock(nullptr, &hz) && hz > 0;
+    hipStream_t st;
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
+    if (e != hipSuccess) return (int)e;
+    void* p = nullptr;
+    int rc = llis_hip_host_alloc_coherent(&p, 64);
+    if (rc) return rc;
+    int* go = reinterpret_cast<int*>(p);
+    __atomic_store_n(go, 0, __ATOMIC_RELEASE);
+    unsigned long long* stamps = nullptr;
+    e = hipMalloc(&stamps, sizeof(unsigned long long) * total);
+    if (e != hipSuccess) {
+        llis_hip_host_free(go);
+        return (int)e;
+    }
+    std::vector<uint64_t> seen_at(total, 0);
+    std::vector<double> rtt(total, 0);
+    // the kernel gives up after 20 s of realtime-counter ticks (100 MHz) whatever the host does
+    hipLaunchKernelGGL(echo_kernel, dim3(1), dim3(1), 0, st, r->channel.fork(), go, stamps, total, 2000000000ull);
+    int done = 0;
+    for (; done < total; ++done) {
+        const double h0 = now_us();
+        __atomic_store_n(go, done + 1, __ATOMIC_RELEASE);
+        unsigned spins = 0;
+        bool got = true;
+        while (!r->channel.can_read<InstrumentInfo>()) {
+            if ((++spins & 0xFFFF) == 0 && now_us() - h0 > 2e6) {
+                got = false;
+                break;
+            }
+        }
+        if (!got) break;
+        if (have_clock) paella::direct_system_clock(&seen_at[done], nullptr);
+        rtt[done] = now_us() - h0;
+        r->channel.read<InstrumentInfo>();
+    }
+    if (done < total) __atomic_store_n(go, -1, __ATOMIC_RELEASE);  // releases the kernel
+    hipStreamSynchronize(st);
+    std::vector<unsigned long long> g(total, 0);
+    hipMemcpy(g.data(), stamps, sizeof(unsigned long long) * total, hipMemcpyDeviceToHost);
+    hipFree(stamps);
+    hipStreamDestroy(st);
+    llis_hip_host_free(go);
+    if (done < total) return -1;
+    for (int i = 0; i < iters; ++i) {
+        round_trip_us[i] = rtt[warmup + i];
+        if (gpu_to_host_us) {
+            uint64_t sys = 0;
+            const bool ok = have_clock && paella::direct_device_tick_to_system(g[warmup + i], &sys);
+            gpu_to_host_us[i] = ok ? ((double)seen_at[warmup + i] - (double)sys) * 1e6 / (double)hz : -1e30;
+        }
+    }
     return 0;
 }
 

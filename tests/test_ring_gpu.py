@@ -134,3 +134,23 @@ def test_notify_latency_probes_report_sane_numbers(ring):
     _abi.check(lib.paella_ring_bench_pingpong(50, 500, ctypes.byref(flag), ctypes.byref(sync), None))
     assert 0.5 < flag.value < 2000.0 and 0.5 < sync.value < 5000.0
     print("ring drain 64 blocks: %.2f us/iter; flag ping-pong %.2f us; stream sync %.2f us" % (us.value, flag.value, sync.value))
+
+
+def test_resident_echo_measures_the_notification_without_a_launch(ring):
+    """A resident lane answers host pings through the ring: every ping is answered in order, the round trip is a
+    few microseconds, and where the runtime can translate the device clock the one-way figure lies inside it."""
+    lib, h = ring
+    n = 2000
+    rtt = np.zeros(n, np.float64)
+    one_way = np.zeros(n, np.float64)
+    from paella_amd import _abi
+    _abi.check(lib.paella_ring_bench_echo(h, 200, n, rtt.ctypes.data, one_way.ctypes.data))
+    assert np.all(rtt > 0) and 0.3 < np.median(rtt) < 200.0
+    assert lib.paella_ring_can_read(h) == 0
+    have = one_way > -1e29
+    print("echo round trip p50 %.2f us p99 %.2f us; device->host p50 %.2f us p99 %.2f us (%d of %d samples translated)" %
+          (np.median(rtt), np.sort(rtt)[int(n * 0.99)], np.median(one_way[have]) if have.any() else float("nan"),
+           np.sort(one_way[have])[int(have.sum() * 0.99)] if have.any() else float("nan"), have.sum(), n))
+    if have.any():
+        # the translation interpolates between clock samples taken by the runtime: allow it a few microseconds
+        assert np.median(one_way[have]) < np.median(rtt) + 5.0 and np.median(one_way[have]) > -5.0

@@ -173,6 +173,37 @@ def test_mixed_model_load_then_outputs_still_correct(cuda):
             close(out, om.run(desc, x, seed=1))
 
 
+MIXES = {
+    # small CNN : Inception-v3 = 9 : 1
+    "two_tenants": ([("mnist", "tvm_mnist", 0.9), ("inception_v3", "tvm_inception_v3", 0.1)], 400.0, 600),
+    # MobileNetV2 + ResNet-50 at equal rates
+    "mobilenet_resnet50": ([("mobilenetv2", "tvm_mobilenet", 0.5), ("resnet50", "tvm_resnet50", 0.5)], 600.0, 400),
+    # eight models, uniform
+    "eight_models": ([(m, "tvm_" + m, 0.125) for m in ("densenet121", "googlenet", "squeezenet1_1", "resnet34", "ultraface320",
+                                                       "arcfaceresnet100")] + [("mobilenetv2", "tvm_mobilenet", 0.125), ("mnist", "tvm_mnist", 0.125)],
+                     1500.0, 400),
+}
+
+
+@pytest.mark.parametrize("mix", sorted(MIXES))
+def test_benchmark_mixes_serve_and_every_model_still_answers_correctly(cuda, mix):
+    """The multi-model configurations of the benchmark under open-loop Poisson arrivals and full3: every request
+    completes, every model gets its share, and afterwards one checked request per model on the same server."""
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    types, iat_us, n = MIXES[mix]
+    with serve.Server(server_name(mix), "full3", num_streams=64, extra_kernels=16) as srv:
+        r = serve.client_run(srv.name, [(serve.job_path(job), prop, 4) for _, job, prop in types], iat_us, 16, n, warmup_jobs=4 * len(types), seed=1)
+        assert r["all"]["count"] == n
+        counts = [r["per_type"][i]["count"] for i in range(len(types))]
+        assert sum(counts) == n and min(counts) > 0.4 * n * min(p for _, _, p in types), counts
+        for model, job, _ in types:
+            desc = models.describe(model)
+            x = om.make_input(desc, 41, "uniform" if model == "mnist" else "normal")
+            out, _ = serve.client_single(srv.name, serve.job_path(job), x, models.io_bytes(model)[1] // 4, n=1)
+            close(out, om.run(desc, x, seed=1))
+
+
 def test_stream_order_independence_of_results(cuda):
     """Stages of one request issued on different streams, each only after the previous stage's end message was
     read from the ring, give the same bits as the single-stream forward: the end hook's ordering is sufficient."""
