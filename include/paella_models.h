@@ -10,7 +10,13 @@
  * interleave stages of different requests.
  *
  * Model names: mnist, resnet18, resnet34, resnet50, mobilenetv2, inception_v3, squeezenet1_1, googlenet,
- * densenet121, ultraface320, arcfaceresnet100.
+ * densenet121, ultraface320, arcfaceresnet100 -- or "onnx:<path>" for an ONNX file, which is imported on first use
+ * (graph and trained weights; batch 1, fp32) where the reference compiles it with TVM
+ * (reference sosp23_artifact/setup/onnx2tvm_all.sh:15-23).  Every entry point below takes either kind of name; for an
+ * imported model the seed is ignored.  Operators read: Conv, BatchNormalization, Relu, Clip, PRelu, LeakyRelu, Add, Sub,
+ * Mul, Div (with constants), MaxPool, AveragePool, GlobalAveragePool, GlobalMaxPool, Gemm, MatMul, Concat, Softmax, LRN,
+ * Flatten, Reshape, Squeeze, Unsqueeze, Dropout, Identity, Constant, and Shape/Gather/Cast over static shapes; a file that
+ * needs anything else makes the call fail (PAELLA_EINVAL) with the reason on stderr.
  *
  * Seeded weights: tensor number t of a model (creation order, listed by paella_model_describe) is filled
  * with value_i = float(normal_i * std_t), normal_i = sqrt(-2 ln u1) cos(2 pi u2),

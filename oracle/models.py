@@ -17,13 +17,18 @@ from . import ops
 
 
 class Desc:
-    def __init__(self, d):
+    def __init__(self, d, external=None):
+        """external(idx) -> array supplies the values of weight tensors marked "external" (imported models carry
+        their own weights instead of seeded ones); tests pass what they read back from the importer."""
         self.d = d
         self.name = d["name"]
+        self.external = external
 
     def weight(self, idx, seed):
         w = self.d["weights"][idx]
         shape = tuple(w["shape"])
+        if w["fill"] == "external":
+            return np.asarray(self.external(idx), np.float32).reshape(shape)
         if w["fill"] == "normal":
             return ops.fill_normal(shape, seed, idx, w["a"])
         if w["fill"] == "uniform":

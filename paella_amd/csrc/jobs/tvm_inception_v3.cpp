@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMInceptionV3Job, "inception_v3")
+PAELLA_DEFINE_MODEL_JOB(TVMInceptionV3Job, "inception_v3", "inception_v3")

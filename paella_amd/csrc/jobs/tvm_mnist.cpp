@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMMnistJob, "mnist")
+PAELLA_DEFINE_MODEL_JOB(TVMMnistJob, "mnist", "mnist-8")

@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMMobilenetJob, "mobilenetv2")
+PAELLA_DEFINE_MODEL_JOB(TVMMobilenetJob, "mobilenetv2", "mobilenetv2-7")

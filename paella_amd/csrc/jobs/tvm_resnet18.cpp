@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMResnet18Job, "resnet18")
+PAELLA_DEFINE_MODEL_JOB(TVMResnet18Job, "resnet18", "resnet18-v2-7")

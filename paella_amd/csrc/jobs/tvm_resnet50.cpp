@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMResnet50, "resnet50")
+PAELLA_DEFINE_MODEL_JOB(TVMResnet50, "resnet50", "resnet50-v2-7")

@@ -2,4 +2,4 @@
 // client command lines keep working; there is no TVM underneath).
 #include "models/model_job.h"
 
-PAELLA_DEFINE_MODEL_JOB(TVMSqueezeNet11Job, "squeezenet1_1")
+PAELLA_DEFINE_MODEL_JOB(TVMSqueezeNet11Job, "squeezenet1_1", "squeezenet1.1-7")

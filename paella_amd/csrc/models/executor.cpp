@@ -59,7 +59,8 @@ const Graph* graph_of(const char* name) {
     if (it != g_graphs.end()) return it->second.get();
     auto g = std::make_unique<Graph>();
     try {
-        if (!build_model(name, g.get())) return nullptr;
+        if (std::strncmp(name, "onnx:", 5) == 0) *g = import_onnx(name + 5, name);
+        else if (!build_model(name, g.get())) return nullptr;
     } catch (const std::exception& e) {
         std::fprintf(stderr, "paella_models: %s: %s\n", name, e.what());
         return nullptr;

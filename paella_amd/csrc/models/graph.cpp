@@ -1,5 +1,6 @@
 #include "graph.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <stdexcept>
@@ -263,6 +264,11 @@ inline double u01(uint64_t seed, uint64_t stream, uint64_t idx) {
 
 void fill_weight(const WeightTensor& t, uint64_t seed, uint64_t stream, float* out) {
     const size_t n = t.numel();
+    if (t.fill == Fill::External) {
+        if (!t.data || t.data->size() != n) throw std::logic_error("external weight tensor without values");
+        std::copy(t.data->begin(), t.data->end(), out);
+        return;
+    }
     const double two_pi = 6.283185307179586476925286766559;
     for (size_t i = 0; i < n; ++i) {
         switch (t.fill) {
@@ -278,6 +284,8 @@ void fill_weight(const WeightTensor& t, uint64_t seed, uint64_t stream, float* o
                 break;
             case Fill::Constant:
                 out[i] = (float)t.a;
+                break;
+            case Fill::External:
                 break;
         }
     }
@@ -314,7 +322,7 @@ std::string describe_json(const Graph& g) {
         const WeightTensor& w = g.weights[i];
         s += i ? ", {\"shape\": [" : "{\"shape\": [";
         for (size_t d = 0; d < w.shape.size(); ++d) s += (d ? ", " : "") + std::to_string(w.shape[d]);
-        const char* fill = w.fill == Fill::Normal ? "normal" : w.fill == Fill::Uniform ? "uniform" : "constant";
+        const char* fill = w.fill == Fill::Normal ? "normal" : w.fill == Fill::Uniform ? "uniform" : w.fill == Fill::Constant ? "constant" : "external";
         std::snprintf(buf, sizeof(buf), "], \"fill\": \"%s\", \"a\": %.17g, \"b\": %.17g}", fill, w.a, w.b);
         s += buf;
     }

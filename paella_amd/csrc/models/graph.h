@@ -8,6 +8,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -27,12 +28,13 @@ struct View {
     size_t numel() const { return (size_t)C * H * W; }
 };
 
-enum class Fill { Normal, Uniform, Constant };
+enum class Fill { Normal, Uniform, Constant, External };
 
 struct WeightTensor {
     std::vector<int> shape;
     Fill fill = Fill::Normal;
     double a = 0, b = 0;  // Normal: std = a; Uniform: [a, b); Constant: a
+    std::shared_ptr<std::vector<float>> data;  // External: the values themselves (imported models); the seed is ignored
     size_t numel() const {
         size_t n = 1;
         for (int d : shape) n *= (size_t)d;
@@ -111,6 +113,10 @@ class GraphBuilder {
     Graph g_;
     double bias_std_;
 };
+
+// Reads an ONNX file into a graph with the file's own weights (throws std::runtime_error with the reason when the
+// file uses something the operators do not cover).
+Graph import_onnx(const std::string& path, const std::string& name);
 
 // Zoo: returns false for an unknown name.
 bool build_model(const std::string& name, Graph* out);

@@ -28,8 +28,23 @@ namespace paella {
 
 class ModelJob : public llis::job::CoroutineJob {
   public:
-    explicit ModelJob(const char* model_name) : name_(model_name) {
-        if (paella_model_io_bytes(model_name, &in_bytes_, &out_bytes_) != 0) throw std::invalid_argument(std::string("unknown model ") + model_name);
+    // onnx_stem: file name (without ".onnx") of the model's ONNX zoo file.  If $LLIS_MODELS_DIR/<stem>.onnx is readable
+    // the adapter serves that file -- its graph and trained weights -- instead of the built-in seeded model; the
+    // reference looks in the same directory for "<stem>-cuda_llis-pack.so" (reference jobs/tvm_mnist/tvm_mnist.cpp:27).
+    explicit ModelJob(const char* model_name, const char* onnx_stem = nullptr) : name_(resolve(model_name, onnx_stem)) {
+        if (paella_model_io_bytes(name_.c_str(), &in_bytes_, &out_bytes_) != 0) throw std::invalid_argument("cannot load model " + name_);
+    }
+
+    static std::string resolve(const char* model_name, const char* onnx_stem) {
+        const char* dir = std::getenv("LLIS_MODELS_DIR");
+        if (dir && *dir && onnx_stem) {
+            const std::string path = std::string(dir) + "/" + onnx_stem + ".onnx";
+            if (FILE* f = std::fopen(path.c_str(), "rb")) {
+                std::fclose(f);
+                return "onnx:" + path;
+            }
+        }
+        return model_name;
     }
 
     size_t get_input_size() override { return in_bytes_; }
@@ -125,9 +140,9 @@ class ModelJob : public llis::job::CoroutineJob {
 
 }  // namespace paella
 
-#define PAELLA_DEFINE_MODEL_JOB(ClassName, model_name)                                                   \
+#define PAELLA_DEFINE_MODEL_JOB(ClassName, model_name, onnx_stem)                                        \
     class ClassName : public paella::ModelJob {                                                          \
       public:                                                                                            \
-        ClassName() : paella::ModelJob(model_name) {}                                                    \
+        ClassName() : paella::ModelJob(model_name, onnx_stem) {}                                         \
     };                                                                                                   \
     extern "C" __attribute__((visibility("default"))) llis::job::Job* init_job() { return new ClassName(); }

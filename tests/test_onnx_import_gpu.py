@@ -1,0 +1,85 @@
+"""ONNX import on the GPU: files written by torch's own ONNX exporter, imported, executed by the HIP operators through
+the C-ABI executor and through a job adapter under the server, against torch's forward pass of the original network.
+Tolerance |got - ref| <= 1e-4 + 1e-3 |ref| (fp32)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import _onnx_writer as ow
+import _torch_nets as nets
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+
+
+def close(got, ref, what):
+    ref = np.asarray(ref, np.float64).reshape(-1)
+    err = np.abs(got.astype(np.float64) - ref)
+    assert got.shape == ref.shape and np.isfinite(got).all()
+    assert np.all(err <= ATOL + RTOL * np.abs(ref)), "%s: max err %g" % (what, err.max())
+    assert np.abs(ref).max() > 1e-3
+
+
+def export(tmp_path, name, module, x):
+    path = tmp_path / (name + ".onnx")
+    if not ow.export_torch(module, x, str(path)):
+        pytest.skip("torch's TorchScript ONNX exporter is not usable here")
+    with torch.no_grad():
+        return str(path), module(x).numpy()
+
+
+def run_on_gpu(path, x):
+    from paella_amd import models
+    ex = models.Exec("onnx:" + path)
+    try:
+        ex.set_input(x)
+        ex.forward()
+        return ex.get_output()
+    finally:
+        ex.close()
+
+
+@pytest.mark.parametrize("net", sorted(nets.NETS))
+def test_imported_networks_match_torch(cuda, tmp_path, net):
+    make, shape = nets.NETS[net]
+    module = nets.randomize(make(), seed=21)
+    x = torch.randn(shape, generator=torch.Generator().manual_seed(6))
+    path, ref = export(tmp_path, net, module, x)
+    print("case", net, flush=True)
+    close(run_on_gpu(path, x.numpy()), ref, net)
+
+
+def test_resnet18_at_full_size_from_its_onnx_file(cuda, tmp_path):
+    """torchvision's ResNet-18 layout with batch norms, 224 x 224, 1000 classes: 20 convs after folding, no elementwise stage."""
+    from paella_amd import models
+    module = nets.randomize(nets.ResNet((2, 2, 2, 2), 64, 1000), seed=4)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(2))
+    path, ref = export(tmp_path, "resnet18_torchvision_layout", module, x)
+    d = models.describe("onnx:" + path)
+    ops = [n["op"] for n in d["nodes"]]
+    assert ops.count("conv") == 20 and ops.count("eltwise") == 0 and len(ops) == 23
+    assert models.totals("onnx:" + path)["macs"] == 1_814_073_344
+    close(run_on_gpu(path, x.numpy()), ref, "resnet18")
+
+
+def test_adapter_serves_the_onnx_file_found_in_the_models_directory(cuda, tmp_path):
+    """$LLIS_MODELS_DIR/resnet18-v2-7.onnx replaces the built-in ResNet-18 behind the tvm_resnet18 adapter: request
+    sizes, graph and weights come from the file."""
+    from paella_amd import serve
+    module = nets.randomize(nets.ResNet((1, 1), 16, 12), seed=8)
+    x = torch.randn(1, 3, 64, 64, generator=torch.Generator().manual_seed(3))
+    path, ref = export(tmp_path, "resnet18-v2-7", module, x)
+    before = os.environ.get("LLIS_MODELS_DIR")
+    os.environ["LLIS_MODELS_DIR"] = str(tmp_path)
+    try:
+        with serve.Server("gt%d_onnx" % os.getpid(), "full3", num_streams=8) as srv:
+            out, _ = serve.client_single(srv.name, serve.job_path("tvm_resnet18"), x.numpy(), 12, n=3)
+    finally:
+        if before is None:
+            del os.environ["LLIS_MODELS_DIR"]
+        else:
+            os.environ["LLIS_MODELS_DIR"] = before
+    close(out, ref, "served")
