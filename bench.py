@@ -144,6 +144,83 @@ def cpu_baseline(model, budget_s):
             "sample": "%d %s forward passes (batch 1, fp32, same graph and seeded weights) with the float-accumulate CPU oracle, %.1f s" % (n, model, dt)}
 
 
+def torch_cpu_baseline(model, budget_s):
+    """The same graph and seeded weights through torch's CPU operators (oneDNN), all host threads: the stronger CPU
+    figure, standing in for the reference's TVM-llvm target, which cannot exist offline."""
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+    from oracle import models as om
+    from paella_amd import models
+    d = models.describe(model)
+    desc = om.Desc(d)
+    W = {i: torch.from_numpy(desc.weight(i, 1)) for i in range(len(d["weights"]))}
+    bufs = [torch.zeros(b["C"] * b["H"] * b["W"]) for b in d["buffers"]]
+
+    def get(v):
+        return None if v["buf"] < 0 else bufs[v["buf"]][v["off"]:v["off"] + v["C"] * v["H"] * v["W"]].view(1, v["C"], v["H"], v["W"])
+
+    def act(y, n):
+        a = n["act"]
+        if a == 1:
+            return F.relu(y)
+        if a == 2:
+            return torch.clamp(y, 0.0, 6.0)
+        if a == 3:
+            return F.prelu(y, W[n["slope"]])
+        if a == 4:
+            return torch.clamp(y, n["lo"], n["hi"])
+        return y
+
+    def forward(x):
+        get(d["input"]).copy_(x)
+        for n in d["nodes"]:
+            xin, x2, op = get(n["x"]), get(n["x2"]), n["op"]
+            if op == "conv":
+                y = F.conv2d(xin, W[n["w"]], W[n["bias"]] if n["bias"] >= 0 else None, tuple(n["stride"]), tuple(n["pad"]), tuple(n["dil"]), n["groups"])
+                y = act(y + x2 if x2 is not None else y, n)
+            elif op == "dense":
+                y = act(F.linear(xin.reshape(1, -1), W[n["w"]], W[n["bias"]]), n)
+            elif op == "pool":
+                if n["avg"]:
+                    y = F.avg_pool2d(xin, tuple(n["k"]), tuple(n["stride"]), tuple(n["pad"]), bool(n["ceil"]), bool(n["count_include_pad"]))
+                else:
+                    y = F.max_pool2d(xin, tuple(n["k"]), tuple(n["stride"]), tuple(n["pad"]), 1, bool(n["ceil"]))
+            elif op == "gap":
+                y = xin.mean((2, 3), keepdim=True)
+            elif op == "eltwise":
+                y = xin
+                if n["scale"] >= 0:
+                    y = y * W[n["scale"]].view(1, -1, 1, 1)
+                if n["shift"] >= 0:
+                    y = y + W[n["shift"]].view(1, -1, 1, 1)
+                y = act(y + x2 if x2 is not None else y, n)
+            elif op == "softmax":
+                y = F.softmax(xin.reshape(n["rows"], n["cols"]), 1)
+            elif op == "lrn":
+                y = F.local_response_norm(xin, n["size"], n["alpha"], n["beta"], n["k"])
+            else:
+                raise ValueError(op)
+            get(n["y"]).copy_(y.reshape(get(n["y"]).shape))
+        return get(d["output"]).reshape(-1).clone()
+
+    x = torch.from_numpy(om.make_input(d, 1))
+    with torch.no_grad():
+        out = forward(x)
+        ref = om.run(desc, x.numpy(), seed=1, fast=True)
+        if not np.allclose(out.numpy(), ref, rtol=1e-2, atol=1e-3):
+            return None  # not the same computation: do not report a time for it
+        n, t0 = 0, time.perf_counter()
+        while True:
+            forward(x)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt >= budget_s or n >= 2000:
+                break
+    return {"value": n / dt, "unit": "requests/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d %s forward passes (batch 1, fp32, same graph and seeded weights) through torch's CPU operators, %.1f s" % (n, model, dt)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -353,6 +430,15 @@ def main():
         lib.paella_ring_destroy(ring)
 
     cpu = None if args.no_cpu else cpu_baseline(args.model, args.cpu_seconds)
+    cpu_torch = None
+    if not args.no_cpu:
+        try:
+            cpu_torch = torch_cpu_baseline(args.model, min(args.cpu_seconds, 8.0))
+        except Exception as ex:  # torch missing or an operator it lacks: the oracle figure stands alone
+            log("[bench]   torch CPU baseline unavailable: %s" % ex)
+        if cpu and cpu_torch:
+            log("[bench]   CPU: oracle %.2f req/s on %d threads, torch CPU operators %.1f req/s on %d threads" %
+                (cpu["value"], cpu["cores"], cpu_torch["value"], cpu_torch["cores"]))
 
     out = {
         "metric": METRIC,
@@ -377,6 +463,7 @@ def main():
                        if len(sweep) > 1 else None),
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "cpu_baseline_torch": cpu_torch,
         "arms": arms,
         "poisson_sweep": sweep,
         "two_tenant_mix": mix,
