@@ -11,7 +11,9 @@ namespace job {
 
 #if defined(__HIPCC__)
 
-// Compute-unit id of the calling wave, folded to 8 bits: (XCC_ID << 5 | SE_ID << 3 | CU_ID) & 0xFF.
+// Compute-unit id of the calling wave in 8 bits: XCC_ID << 5 | SE_ID << 3 | (CU_ID & 7).  Each of an XCD's four shader
+// engines exposes eight consecutive CU_ID values (0..7 or 1..8 on MI355X), so the low three bits tell them apart and the
+// id is dense over the 256 compute units, with the XCD in the top three bits.
 __device__ __forceinline__ unsigned current_cu_id() {
     unsigned hw_id, xcc_id;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));

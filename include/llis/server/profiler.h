@@ -5,7 +5,8 @@
 // written on SAVE as <prefix>_kernel_info.txt, _job_events.txt, _run_next_times.txt and _resource_events.txt in
 // the reference's line formats (reference src/server/profiler.cpp:76-131), plus _block_exec_times.txt when the
 // server runs with --measure_block_time (entry and exit clock of every workgroup, 24 bits each, 10 ns units).
-// _kernel_block_mis_alloc.txt (written only by schedulers the reference does not build) is created empty.
+// _kernel_block_mis_alloc.txt holds what GpuResources::reconcile() reports (the reference only writes it from a
+// scheduler it does not build); it is empty when no per-compute-unit model is in use.
 
 #include <llis/ipc/defs.h>
 #include <llis/ipc/shm_channel.h>
@@ -40,6 +41,11 @@ class Profiler {
                             unsigned num_registers_per_thread, double priority, unsigned job_ref_id);
     void record_job_event(JobId job_id, JobEvent event);
     void record_block_exec_time(unsigned long long start, unsigned long long end);
+    // one kernel's placement prediction against what its workgroups reported: workgroups, mispredicted workgroups,
+    // compute units they had been predicted on (reference src/server/profiler.cpp:146-150, file format :93-97)
+    void record_kernel_block_mis_alloc(unsigned total, unsigned total_wrong_prediction, unsigned total_wrong_prediction_cus);
+    // the reference's spelling of the same call
+    void recrod_kernel_block_mis_alloc(unsigned total, unsigned wrong, unsigned wrong_sm) { record_kernel_block_mis_alloc(total, wrong, wrong_sm); }
     bool recording_run_next_times() const { return run_next_times_flag_; }
     void record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks);
     // num workgroups of the job's running stage acquired or released (reference src/server/sm_resources.cpp:48,64)
@@ -54,7 +60,8 @@ class Profiler {
     bool run_next_times_flag_ = false;
     bool resource_events_flag_ = false;
     bool block_exec_times_flag_ = false;
-    bool mis_alloc_flag_ = false;  // accepted, nothing records it
+    bool mis_alloc_flag_ = false;
+    std::vector<std::tuple<unsigned, unsigned, unsigned>> mis_alloc_;
     std::vector<std::pair<unsigned long long, unsigned long long>> block_exec_times_;
     std::vector<std::tuple<TimePoint, TimePoint, unsigned>> run_next_times_;
     std::vector<std::tuple<JobId, std::string, ResourceEvent, TimePoint, unsigned, unsigned, unsigned, unsigned>> resource_events_;

@@ -169,6 +169,81 @@ class SmResources:
         self.free = [f + x for f, x in zip(self.free, self._need(st, n))]
 
 
+class GpuResources:
+    """Per-compute-unit budget with the XCD-aware placement prediction (restates include/llis/server/gpu_resources.h;
+    accounting as reference src/server/gpu_resources.cpp:38-64, reconciliation as reference
+    src/server/scheduler_full.cpp:98-121).  A stage is a Stage (regs, smem, threads, blocks).  The placement rule is
+    this build's own (the reference's table is for another vendor's part): workgroup i of a dispatch goes to XCD
+    (first + i) mod xcds, inside it to the compute unit with the most free threads, searching from a pointer that
+    moves past the last choice."""
+
+    def __init__(self, cus, xcds, regs, smem, threads, blocks):
+        self.cus = [SmResources(regs, smem, threads, blocks) for _ in range(cus)]
+        self.xcds, self.per = xcds, cus // xcds
+        self.next_cu = [0] * xcds
+        self.next_xcd = 0
+
+    @staticmethod
+    def _full(r):
+        return any(f <= 0 for f in r.free)
+
+    @staticmethod
+    def _room(r, st):
+        if GpuResources._full(r):
+            return 0
+        n = r.free[3]
+        if st.threads > 0:
+            if st.regs * st.threads > 0:
+                n = min(n, r.free[0] // (st.regs * st.threads))
+            n = min(n, r.free[2] // st.threads)
+        if st.smem > 0:
+            n = min(n, r.free[1] // st.smem)
+        return max(n, 0)
+
+    def num_full(self):
+        return sum(self._full(r) for r in self.cus)
+
+    def fits(self, st):
+        for x in range(self.xcds):
+            lane = (x - self.next_xcd) % self.xcds
+            share = (st.blocks - lane + self.xcds - 1) // self.xcds if st.blocks > lane else 0
+            if sum(self._room(r, st) for r in self.cus[x * self.per:(x + 1) * self.per]) < share:
+                return False
+        return True
+
+    def choose(self, st):
+        """Returns {cu: workgroups predicted there}; acquires them."""
+        predicted = {}
+        for i in range(st.blocks):
+            x = (self.next_xcd + i) % self.xcds
+            best, best_room = None, None
+            for k in range(self.per):
+                c = x * self.per + (self.next_cu[x] + k) % self.per
+                room = -1 if self._full(self.cus[c]) else self.cus[c].free[2]
+                if best is None or room > best_room:
+                    best, best_room = c, room
+            self.next_cu[x] = (best % self.per + 1) % self.per
+            self.cus[best].acquire(st, 1)
+            predicted[best] = predicted.get(best, 0) + 1
+        self.next_xcd = (self.next_xcd + st.blocks) % self.xcds
+        return predicted
+
+    def observe_start(self, st, predicted, cu):
+        if predicted.get(cu, 0) > 0:
+            predicted[cu] -= 1
+        else:
+            self.cus[cu].acquire(st, 1)
+
+    def reconcile(self, st, predicted):
+        wrong = sum(predicted.values())
+        wrong_cus = sum(1 for n in predicted.values() if n > 0)
+        for cu, n in predicted.items():
+            if n > 0:
+                self.cus[cu].release(st, n)
+        predicted.clear()
+        return wrong, wrong_cus
+
+
 # Budget the scripted test device reports: 256 CUs x {131072 regs, 160 KiB LDS, 2048 threads, 32 workgroups}.
 FAKE_BUDGET = (256 * 131072, 256 * 163840, 256 * 2048, 256 * 32)
 

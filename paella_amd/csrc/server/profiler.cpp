@@ -49,6 +49,10 @@ void Profiler::record_block_exec_time(unsigned long long start, unsigned long lo
     if (block_exec_times_flag_) block_exec_times_.emplace_back(start, end);
 }
 
+void Profiler::record_kernel_block_mis_alloc(unsigned total, unsigned total_wrong_prediction, unsigned total_wrong_prediction_cus) {
+    if (mis_alloc_flag_) mis_alloc_.emplace_back(total, total_wrong_prediction, total_wrong_prediction_cus);
+}
+
 void Profiler::record_run_next_time(TimePoint start, TimePoint end, unsigned num_blocks) {
     if (run_next_times_flag_) run_next_times_.emplace_back(start, end, num_blocks);
 }
@@ -98,7 +102,11 @@ void Profiler::save(const std::string& prefix) {
         for (const auto& b : block_exec_times_) std::fprintf(fp, "%llu %llu\n", b.first, b.second);
         std::fclose(fp);
     }
-    if (FILE* fp = std::fopen((prefix + "_kernel_block_mis_alloc.txt").c_str(), "w")) std::fclose(fp);
+    if (FILE* fp = std::fopen((prefix + "_kernel_block_mis_alloc.txt").c_str(), "w")) {
+        for (const auto& m : mis_alloc_) std::fprintf(fp, "%u %u %u\n", std::get<0>(m), std::get<1>(m), std::get<2>(m));
+        std::fclose(fp);
+    }
+    mis_alloc_.clear();
     kernel_info_.clear();
     jobs_events_all_.clear();
     run_next_times_.clear();
