@@ -288,8 +288,25 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     // the chunk D ahead right after it has been consumed.  Shallow is better here: the small tile measured
     // fastest at depth 2, alone (6.1 us for the 64-channel 56x56 layer against 6.4 at depth 4) and with many
     // kernels in flight (2.4 against 2.7 us per kernel): fewer registers, so four workgroups fit a CU, and other
-    // waves hide the latency that a deeper pipeline would.
+    // waves hide the latency that a deeper pipeline would.  Three slots with the refill issued ahead of the current
+    // chunk's matrix instructions were no better either (23.8 against 24.9 TFLOP/s over a ResNet-18 pass): the loop is
+    // bound by what the compute unit's vector cache can take in -- each wave fetches its own 32 x 8 operand
+    // fragments, 147 KB per workgroup for a 64-channel 3x3 layer -- not by exposed latency.
     constexpr int D = (MI * NI == 1) ? PAELLA_CONV_DEPTH : 4;
+    auto compute = [&](const Frag<MI, NI>& f) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const float av = t == 0 ? f.a[mi].x : t == 1 ? f.a[mi].y : t == 2 ? f.a[mi].z : f.a[mi].w;
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * f.b[ni][t];
+                    else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
+                }
+            }
+        }
+    };
     if (c_begin < c_end) {
         Frag<MI, NI> frag[D];
 #pragma unroll
@@ -297,20 +314,6 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
             load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
         }
-        auto compute = [&](const Frag<MI, NI>& f) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int mi = 0; mi < MI; ++mi) {
-                    const float av = t == 0 ? f.a[mi].x : t == 1 ? f.a[mi].y : t == 2 ? f.a[mi].z : f.a[mi].w;
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * f.b[ni][t];
-                        else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
-                    }
-                }
-            }
-        };
         CONV_TL(2);
         const int n = c_end - c_begin;
         const int c_main_end = c_begin + (n / D) * D;
@@ -334,21 +337,33 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     }
 
     CONV_TL(3);
-    auto epilogue = [&](int rr, float v) {
-        int m, pix;
-        out_coords(wave * RPW + rr, m, pix);
-        if (m < p.K && pix < p.PQ) {
-            const size_t o = (size_t)m * p.PQ + pix;
+    // Finishes the wave's RPW outputs.  Every operand load comes first, then the arithmetic, then the stores back
+    // to back: a load between two stores would make the compiler wait for the earlier store as well (one counter
+    // covers both), and a write-through store takes about 0.3 us to be acknowledged.
+    auto epilogue_all = [&](float (&v)[RPW]) {
+        size_t o[RPW];
+        bool ok[RPW];
+        float sl[RPW];
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {
+            int m, pix;
+            out_coords(wave * RPW + rr, m, pix);
+            ok[rr] = m < p.K && pix < p.PQ;
+            o[rr] = (size_t)m * p.PQ + pix;
+            sl[rr] = (ok[rr] && p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
             if (kPrefetchEpilogue) {
-                v += bias_v[rr];
-                v += res_v[rr];
-            } else {
-                if (p.bias) v += p.bias[m];
-                if (p.residual) v += p.residual[o];
+                v[rr] += bias_v[rr];
+                v[rr] += res_v[rr];
+            } else if (ok[rr]) {
+                if (p.bias) v[rr] += p.bias[m];
+                if (p.residual) v[rr] += p.residual[o[rr]];
             }
-            const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
-            store_out(p.y + o, apply_act(v, p.act, sl, p.lo, p.hi));
         }
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) v[rr] = apply_act(v[rr], p.act, sl[rr], p.lo, p.hi);
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr)
+            if (ok[rr]) store_out(p.y + o[rr], v[rr]);
     };
 
     float mine[RPW];
@@ -385,8 +400,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
         return;
     }
     if (p.splits == 1) {
-#pragma unroll
-        for (int rr = 0; rr < RPW; ++rr) epilogue(rr, mine[rr]);
+        epilogue_all(mine);
     } else {
         // Deterministic split-k: every workgroup parks its partial tile in the workspace (write-through),
         // bumps the tile's counter, and the workgroup that arrives last adds the partials in split order and
@@ -422,8 +436,7 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
 #pragma unroll
                     for (int rr = 0; rr < RPW; ++rr) v[rr] += t[u][rr];
             }
-#pragma unroll
-            for (int rr = 0; rr < RPW; ++rr) epilogue(rr, v[rr]);
+            epilogue_all(v);
             if (threadIdx.x == 0) __hip_atomic_store(p.ws_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
