@@ -398,6 +398,16 @@ def main():
     if lib.paella_mfma_peak_probe(ctypes.byref(peak)) == 0:
         roofline["peak_measured"] = peak.value  # register-resident fp32 MFMA loop on this box; `peak` stays the published figure
         log("[bench]   fp32 MFMA rate measured with a register-resident loop: %.1f TFLOP/s" % peak.value)
+    floor = ctypes.c_double()
+    if lib.paella_empty_kernel_probe(200, ctypes.byref(floor)) == 0 and floor.value > 0:
+        # what the same time stamps report for a kernel that does nothing: every launch pays it, so at batch 1 the
+        # 20 conv launches of a pass cannot beat flops / (20 x floor) however fast the kernels are
+        bound = rl["conv_flops"] / (rl["conv_launches"] * floor.value * 1e-6) / 1e12
+        roofline["empty_kernel_us"] = floor.value
+        roofline["launch_bound_tflops"] = bound
+        roofline["frac_of_launch_bound"] = achieved / bound
+        log("[bench]   an empty kernel takes %.2f us by the same time stamps: launch-bound ceiling %.1f TFLOP/s, conv at %.0f%% of it" %
+            (floor.value, bound, 100 * achieved / bound))
     ring = ctypes.c_void_p()
     notify = {}
     if not args.roofline_only and lib.paella_ring_create(1024000, 1, ctypes.byref(ring)) == 0:

@@ -61,6 +61,10 @@ int paella_ring_bench_pingpong(int warmup, int iters, double* flag_us, double* s
  * Both arrays hold `iters` doubles.  The lane's wait is bounded (20 s of device time) and ends early on error. */
 int paella_ring_bench_echo(paella_ring* ring, int warmup, int iters, double* round_trip_us, double* gpu_to_host_us);
 
+/* Duration of a kernel that does nothing (256 workgroups of 256 lanes), between the begin and end time stamps the
+ * device records for it: the floor under every per-launch figure measured the same way.  Median of `iters` launches. */
+int paella_empty_kernel_probe(int iters, double* median_us);
+
 /* Sustained fp32 MFMA rate of the device (v_mfma_f32_32x32x2_f32, register-resident operands, every SIMD busy):
  * the measured denominator next to the published 157.3 TFLOP/s. */
 int paella_mfma_peak_probe(double* tflops);

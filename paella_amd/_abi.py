@@ -109,6 +109,7 @@ RING_SYMBOLS = {
     "paella_ring_drain": (c_size_t, [c_void_p, c_void_p, c_size_t, c_double]),
     "paella_ring_bench_drain": (c_int, [c_void_p, c_uint, c_uint, c_int, c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_pingpong": (c_int, [c_int, c_int, ctypes.POINTER(c_double), ctypes.POINTER(c_double), c_void_p]),
+    "paella_empty_kernel_probe": (c_int, [c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_echo": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "paella_mfma_peak_probe": (c_int, [ctypes.POINTER(c_double)]),
 }

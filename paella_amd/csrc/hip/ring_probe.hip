@@ -1,7 +1,9 @@
 // Stand-alone exercisers and latency probes for the GPU->host notification ring (see include/paella_ring.h).
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <new>
@@ -298,6 +300,31 @@ int paella_ring_bench_echo(paella_ring* r, int warmup, int iters, double* round_
             gpu_to_host_us[i] = ok ? ((double)seen_at[warmup + i] - (double)sys) * 1e6 / (double)hz : -1e30;
         }
     }
+    return 0;
+}
+
+int paella_empty_kernel_probe(int iters, double* median_us) {
+    if (iters <= 0 || iters > 100000 || !median_us) return -1;
+    hipStream_t st;
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
+    if (e != hipSuccess) return (int)e;
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    std::vector<float> us;
+    for (int it = -10; it < iters; ++it) {
+        // the extended launch stamps the events with the kernel's own begin and end time on the device
+        hipExtLaunchKernelGGL(empty_kernel, dim3(256), dim3(256), 0, st, e0, e1, 0);
+        hipStreamSynchronize(st);
+        float ms = 0;
+        if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && it >= 0) us.push_back(ms * 1e3f);
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    hipStreamDestroy(st);
+    if (us.empty()) return -1;
+    std::sort(us.begin(), us.end());
+    *median_us = us[us.size() / 2];
     return 0;
 }
 
