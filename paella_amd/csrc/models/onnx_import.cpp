@@ -209,6 +209,8 @@ Tensor parse_tensor(Reader r) {
             default: r.skip(wire);
         }
     }
+    for (int64_t d : t.dims)
+        if (d < 0 || d > (int64_t)1 << 32) fail("tensor '" + t.name + "' has an impossible dimension");
     const size_t n = t.numel();
     auto need = [&](size_t have, size_t elem) {
         if (have != n * elem) fail("tensor '" + t.name + "' holds " + std::to_string(have / elem) + " values for " + std::to_string(n) + " elements");
@@ -225,9 +227,9 @@ Tensor parse_tensor(Reader r) {
             }
             break;
         case kDouble:
-            t.f.resize(n);
             if (raw) {
                 need(raw_len, 8);
+                t.f.resize(n);
                 for (size_t k = 0; k < n; ++k) {
                     double v;
                     std::memcpy(&v, raw + 8 * k, 8);
@@ -235,13 +237,14 @@ Tensor parse_tensor(Reader r) {
                 }
             } else {
                 need(double_data.size(), 1);
+                t.f.resize(n);
                 for (size_t k = 0; k < n; ++k) t.f[k] = (float)double_data[k];
             }
             break;
         case kFloat16:
-            t.f.resize(n);
             if (raw) {
                 need(raw_len, 2);
+                t.f.resize(n);
                 for (size_t k = 0; k < n; ++k) {
                     uint16_t h;
                     std::memcpy(&h, raw + 2 * k, 2);
@@ -249,6 +252,7 @@ Tensor parse_tensor(Reader r) {
                 }
             } else {
                 need(int_data.size(), 1);
+                t.f.resize(n);
                 for (size_t k = 0; k < n; ++k) t.f[k] = half_to_float((uint16_t)int_data[k]);
             }
             break;
@@ -263,9 +267,9 @@ Tensor parse_tensor(Reader r) {
             }
             break;
         case kInt32:
-            t.i.resize(n);
             if (raw) {
                 need(raw_len, 4);
+                t.i.resize(n);
                 for (size_t k = 0; k < n; ++k) {
                     int32_t v;
                     std::memcpy(&v, raw + 4 * k, 4);
@@ -944,7 +948,10 @@ class Importer {
                 else known *= d;
                 shape.push_back(d);
             }
-            if (infer >= 0) shape[(size_t)infer] = (int64_t)x.v.numel() / known;
+            if (infer >= 0) {
+                if (known <= 0) fail(n.label() + ": cannot infer a dimension next to a zero-sized one");
+                shape[(size_t)infer] = (int64_t)x.v.numel() / known;
+            }
         } else if (n.op == "Squeeze" || n.op == "Unsqueeze") {
             std::vector<int64_t> axes = n.getints("axes");
             if (axes.empty() && n.in.size() > 1 && !n.in[1].empty()) axes = init_i(n, n.in[1]).i;

@@ -246,3 +246,12 @@ def test_garbage_and_missing_files_are_errors(tmp_path, capfd):
         with pytest.raises(RuntimeError):
             models.describe(name)
     assert "onnx import" in capfd.readouterr().err
+    # a tensor whose dims promise far more data than the file holds must be refused before anything is allocated for it
+    b = ow.Builder(np.random.default_rng(0))
+    lie = ow._len(1, ow._varint(1 << 30) + ow._varint(1 << 30)) + ow._int(2, 11) + ow._len(9, b"\0" * 8) + ow._str(8, "w")
+    b.inits.append(lie)
+    b.nodes.append(ow.node("Conv", ["x", "w"], ["y"], kernel_shape=[3, 3]))
+    b.save(str(tmp_path / "lie.onnx"), [("x", [1, 3, 8, 8])], [("y", [1, 4, 6, 6])])
+    with pytest.raises(RuntimeError):
+        models.describe("onnx:" + str(tmp_path / "lie.onnx"))
+    assert "holds" in capfd.readouterr().err
