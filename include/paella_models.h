@@ -70,6 +70,13 @@ int paella_exec_destroy(paella_exec* e);
 /* Device pointers of the request's input and output tensors. */
 void* paella_exec_input(paella_exec* e);
 void* paella_exec_output(paella_exec* e);
+/* Makes the stages read the request's input from / write its output to memory of the caller instead of the request's own
+ * device buffers -- pinned host memory the device can address, 16-byte aligned, at least the model's input / output
+ * size: small tensors then cross PCIe inside the first / last kernel and need no copy stage of their own.  NULL restores
+ * the device buffer.  PAELLA_ENOSUP if the graph cannot do without the buffer (a stage reads the output back, or writes
+ * into the input buffer).  No counterpart in the reference, whose adapters always copy (jobs/tvm_mnist/tvm_mnist.cpp:38-46). */
+int paella_exec_bind_input(paella_exec* e, void* device_visible);
+int paella_exec_bind_output(paella_exec* e, void* device_visible);
 /* Issues stage i on `stream`; notifier may be NULL. */
 int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier);
 /* All stages back to back on one stream, un-instrumented (plain single-stream serving). */

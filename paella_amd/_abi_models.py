@@ -19,6 +19,8 @@ MODEL_SYMBOLS = {
     "paella_model_stage_work": (c_int, [c_void_p, c_int, ctypes.POINTER(c_char_p), _pd, _pd]),
     "paella_exec_create": (c_int, [c_void_p, ctypes.POINTER(c_void_p)]),
     "paella_exec_destroy": (c_int, [c_void_p]),
+    "paella_exec_bind_input": (c_int, [c_void_p, c_void_p]),
+    "paella_exec_bind_output": (c_int, [c_void_p, c_void_p]),
     "paella_exec_input": (c_void_p, [c_void_p]),
     "paella_exec_output": (c_void_p, [c_void_p]),
     "paella_exec_launch_stage": (c_int, [c_void_p, c_int, c_void_p, c_u32, c_void_p]),

@@ -43,7 +43,14 @@ struct paella_exec {
     const paella_model* m = nullptr;
     float* arena = nullptr;
     void* workspace = nullptr;
-    float* ptr(const View& v) const { return v.buf < 0 ? nullptr : arena + m->g.buffers[v.buf].offset + v.off; }
+    float* in_bound = nullptr;   // caller's memory standing for the input / output buffer (paella_exec_bind_*)
+    float* out_bound = nullptr;
+    float* ptr(const View& v) const {
+        if (v.buf < 0) return nullptr;
+        if (in_bound && v.buf == m->g.input.buf) return in_bound + v.off;
+        if (out_bound && v.buf == m->g.output.buf) return out_bound + v.off;
+        return arena + m->g.buffers[v.buf].offset + v.off;
+    }
 };
 
 namespace {
@@ -300,6 +307,31 @@ int paella_exec_destroy(paella_exec* e) {
     llis_hip_device_free(e->arena);
     if (e->workspace) llis_hip_device_free(e->workspace);
     delete e;
+    return 0;
+}
+
+int paella_exec_bind_input(paella_exec* e, void* p) {
+    if (!e || ((uintptr_t)p & 15)) return PAELLA_EINVAL;
+    const Graph& g = e->m->g;
+    if (p) {
+        if (g.input.off != 0) return PAELLA_ENOSUP;
+        for (const Node& n : g.nodes)
+            if (n.y.buf == g.input.buf) return PAELLA_ENOSUP;   // something writes into the input buffer (a concatenation re-based onto it)
+    }
+    e->in_bound = reinterpret_cast<float*>(p);
+    return 0;
+}
+
+int paella_exec_bind_output(paella_exec* e, void* p) {
+    if (!e || ((uintptr_t)p & 15)) return PAELLA_EINVAL;
+    const Graph& g = e->m->g;
+    if (p) {
+        const Buffer& b = g.buffers[g.output.buf];
+        if (g.output.off != 0 || g.output.numel() != (size_t)b.C * b.H * b.W || g.output.buf == g.input.buf) return PAELLA_ENOSUP;
+        for (const Node& n : g.nodes)
+            if (n.x.buf == g.output.buf || n.x2.buf == g.output.buf) return PAELLA_ENOSUP;   // a stage reads it back
+    }
+    e->out_bound = reinterpret_cast<float*>(p);
     return 0;
 }
 

@@ -8,6 +8,9 @@
 // Differences, on purpose:
 //  * the device-to-host stage copies the model OUTPUT (the reference copies its input buffer back);
 //  * PAELLA_INPUT_RESIDENT=1 (measurement only) drops the host-to-device stage: the input stays in device memory;
+//  * a tensor of at most PAELLA_ZERO_COPY_BYTES (default 64 KiB) gets no copy stage: the first kernel reads the input
+//    from, the last kernel writes the output to, the pinned staging buffer across PCIe (the small CNN then has 5 stages
+//    instead of 7, ResNet-18 no device-to-host stage); pre-notify moves to the last kernel;
 //  * request buffers in the client's shared-memory pool cannot be registered with the runtime on this
 //    platform, so both copies go through a per-instance pinned staging buffer (filled on the server
 //    thread just before the H2D copy is issued, drained in on_complete()).
@@ -57,7 +60,8 @@ class ModelJob : public llis::job::CoroutineJob {
         check(paella_model_get(name_.c_str(), seed, &model_), "paella_model_get");
         check(paella_exec_create(model_, &exec_), "paella_exec_create");
         void* p = nullptr;
-        check(llis_hip_host_alloc_pinned(&p, in_bytes_ + out_bytes_), "pinned staging");
+        out_off_ = (in_bytes_ + 255) / 256 * 256;
+        check(llis_hip_host_alloc_pinned(&p, out_off_ + out_bytes_), "pinned staging");
         staging_ = reinterpret_cast<char*>(p);
         num_stages_ = paella_model_num_stages(model_);
         // Kernels go out as AQL packets on the operator library's own queues unless PAELLA_DISPATCH=hip; the
@@ -65,6 +69,10 @@ class ModelJob : public llis::job::CoroutineJob {
         // notification ring (fifo2, full3): the queues have no ordering of their own, and fifo relies on the stream.
         const char* resident = std::getenv("PAELLA_INPUT_RESIDENT");
         input_resident_ = resident && std::strcmp(resident, "1") == 0;
+        const char* zc = std::getenv("PAELLA_ZERO_COPY_BYTES");
+        const size_t zero_copy_limit = zc ? std::strtoull(zc, nullptr, 10) : 65536;
+        zero_in_ = !input_resident_ && in_bytes_ <= zero_copy_limit && paella_exec_bind_input(exec_, staging_) == 0;
+        zero_out_ = out_bytes_ <= zero_copy_limit && paella_exec_bind_output(exec_, staging_ + out_off_) == 0;
         timed_ = llis::job::Context::get_gpu2sched_block_time_channel()->is_connected();  // server runs with --measure_block_time
         const char* dispatch = std::getenv("PAELLA_DISPATCH");
         direct_ = !(dispatch && std::strcmp(dispatch, "hip") == 0) && llis::job::Context::is_stage_by_stage();
@@ -79,7 +87,9 @@ class ModelJob : public llis::job::CoroutineJob {
 
     void body(void* io_ptr) override {
         io_ptr_ = io_ptr;
-        if (!input_resident_) {
+        if (zero_in_) {
+            // no stage of its own: staged just before the first kernel is issued, below
+        } else if (!input_resident_) {
             set_is_mem();
             yield();
             std::memcpy(staging_, io_ptr, in_bytes_);
@@ -99,7 +109,9 @@ class ModelJob : public llis::job::CoroutineJob {
             set_num_threads_per_block(d.block);
             set_smem_size_per_block(d.lds_bytes);
             set_num_registers_per_thread(d.vgprs);
+            if (zero_out_ && s == num_stages_ - 1) set_pre_notify();
             yield();
+            if (zero_in_ && s == 0) std::memcpy(staging_, io_ptr, in_bytes_);
             // Only a kernel admitted beyond the occupancy budget ("unfit") needs its workgroup starts reported.
             const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
             void* target = stream();
@@ -107,14 +119,15 @@ class ModelJob : public llis::job::CoroutineJob {
             check(paella_exec_launch_stage(exec_, s, target, id, get_finished_block_notifier()), "stage launch");
         }
 
+        if (zero_out_) return;
         set_is_mem();
         set_pre_notify();
         yield();
-        check(llis_hip_memcpy_async(staging_ + in_bytes_, paella_exec_output(exec_), out_bytes_, LLIS_HIP_D2H, stream()), "D2H");
+        check(llis_hip_memcpy_async(staging_ + out_off_, paella_exec_output(exec_), out_bytes_, LLIS_HIP_D2H, stream()), "D2H");
     }
 
     // The output sits right after the input bytes of the request slot (what the client library reads).
-    void on_complete() override { std::memcpy(reinterpret_cast<char*>(io_ptr_) + in_bytes_, staging_ + in_bytes_, out_bytes_); }
+    void on_complete() override { std::memcpy(reinterpret_cast<char*>(io_ptr_) + in_bytes_, staging_ + out_off_, out_bytes_); }
 
   private:
     void* stream() { return reinterpret_cast<void*>(get_cuda_stream()); }
@@ -127,7 +140,7 @@ class ModelJob : public llis::job::CoroutineJob {
     }
 
     std::string name_;
-    size_t in_bytes_ = 0, out_bytes_ = 0;
+    size_t in_bytes_ = 0, out_bytes_ = 0, out_off_ = 0;
     paella_model* model_ = nullptr;
     paella_exec* exec_ = nullptr;
     char* staging_ = nullptr;
@@ -136,6 +149,7 @@ class ModelJob : public llis::job::CoroutineJob {
     bool direct_ = true;
     bool timed_ = false;
     bool input_resident_ = false, input_uploaded_ = false;
+    bool zero_in_ = false, zero_out_ = false;
 };
 
 }  // namespace paella

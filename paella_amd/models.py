@@ -80,6 +80,11 @@ class Exec:
         check(_abi.hip().llis_hip_memcpy(out.ctypes.data, self.lib.paella_exec_output(self.handle), out.nbytes, 2), "D2H")
         return out
 
+    def bind_io(self, in_ptr=None, out_ptr=None):
+        """Device-visible host memory (addresses) in place of the request's input / output device buffers; None restores."""
+        check(self.lib.paella_exec_bind_input(self.handle, ctypes.c_void_p(in_ptr)), "paella_exec_bind_input")
+        check(self.lib.paella_exec_bind_output(self.handle, ctypes.c_void_p(out_ptr)), "paella_exec_bind_output")
+
     def forward(self, stream=None):
         check(self.lib.paella_exec_forward(self.handle, stream), "paella_exec_forward")
 

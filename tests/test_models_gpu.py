@@ -82,3 +82,38 @@ def test_different_seeds_and_inputs_give_different_outputs(cuda):
         outs.append(ex.get_output())
         ex.close()
     assert not np.allclose(outs[0], outs[1]) and not np.allclose(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("name", ["mnist", "googlenet", "ultraface320"])
+def test_input_and_output_bound_to_pinned_host_memory_give_the_same_bits(cuda, name):
+    """The first stage reading the input from, and the last writing the output to, host memory across PCIe (what the
+    job adapters do for small tensors) changes no bit of the result."""
+    from paella_amd import _abi, models
+    hip = _abi.hip()
+    desc = models.describe(name)
+    x = om.make_input(desc, 13, "uniform" if name == "mnist" else "normal")
+    ex = models.Exec(name, seed=2)
+    host = ctypes.c_void_p()
+    out_off = (ex.in_bytes + 255) // 256 * 256
+    _abi.check(hip.llis_hip_host_alloc_pinned(ctypes.byref(host), out_off + ex.out_bytes))
+    try:
+        ex.set_input(x)
+        ex.forward()
+        want = ex.get_output()
+        ctypes.memmove(host.value, np.ascontiguousarray(x, np.float32).ctypes.data, ex.in_bytes)
+        ctypes.memset(host.value + out_off, 0xFF, ex.out_bytes)
+        ex.set_input(np.zeros_like(x))                      # the device-side input buffer must not be what is read
+        ex.bind_io(host.value, host.value + out_off)
+        for i in range(ex.num_stages):
+            ex.launch_stage(i)
+        _abi.check(hip.llis_hip_device_synchronize())
+        got = np.frombuffer((ctypes.c_char * ex.out_bytes).from_address(host.value + out_off), np.float32).copy()
+        np.testing.assert_array_equal(got, want)
+        ex.bind_io(None, None)
+        ex.set_input(x)
+        ex.forward()
+        np.testing.assert_array_equal(ex.get_output(), want)
+        assert ex.lib.paella_exec_bind_input(ex.handle, ctypes.c_void_p(host.value + 4)) == -1     # misaligned
+    finally:
+        ex.close()
+        hip.llis_hip_host_free(host)

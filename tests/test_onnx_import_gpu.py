@@ -83,3 +83,23 @@ def test_adapter_serves_the_onnx_file_found_in_the_models_directory(cuda, tmp_pa
         else:
             os.environ["LLIS_MODELS_DIR"] = before
     close(out, ref, "served")
+
+
+def test_output_that_a_later_stage_reads_back_cannot_be_bound_to_host_memory(cuda, tmp_path):
+    """The graph's output tensor also feeds a pooling stage: the executor must keep it in device memory."""
+    import ctypes
+    from paella_amd import _abi, models
+    b = ow.Builder(np.random.default_rng(1))
+    y1 = b.op("Relu", [b.op("Conv", ["x", b.const(b.randn(4, 3, 3, 3))], kernel_shape=[3, 3])])
+    b.op("GlobalAveragePool", [y1])
+    path = str(tmp_path / "readback.onnx")
+    b.save(path, [("x", [1, 3, 8, 8])], [(y1, [1, 4, 6, 6])])
+    ex = models.Exec("onnx:" + path)
+    host = ctypes.c_void_p()
+    _abi.check(_abi.hip().llis_hip_host_alloc_pinned(ctypes.byref(host), 4096))
+    try:
+        assert ex.lib.paella_exec_bind_output(ex.handle, host) == -2
+        assert ex.lib.paella_exec_bind_input(ex.handle, host) == 0
+    finally:
+        ex.close()
+        _abi.hip().llis_hip_host_free(host)

@@ -173,6 +173,23 @@ def test_mixed_model_load_then_outputs_still_correct(cuda):
             close(out, om.run(desc, x, seed=1))
 
 
+@pytest.mark.parametrize("model,job", [("mnist", "tvm_mnist"), ("resnet18", "tvm_resnet18")])
+def test_copy_stages_still_serve_when_zero_copy_is_switched_off(cuda, model, job):
+    """PAELLA_ZERO_COPY_BYTES=0: every request goes host-to-device copy -> kernels -> device-to-host copy (pre-notify), the
+    reference's stage sequence; same results."""
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    os.environ["PAELLA_ZERO_COPY_BYTES"] = "0"
+    try:
+        desc = models.describe(model)
+        x = om.make_input(desc, 23, "uniform" if model == "mnist" else "normal")
+        with serve.Server(server_name("copies"), "full3", num_streams=8) as srv:
+            out, _ = serve.client_single(srv.name, serve.job_path(job), x, models.io_bytes(model)[1] // 4, n=3)
+        close(out, om.run(desc, x, seed=1))
+    finally:
+        del os.environ["PAELLA_ZERO_COPY_BYTES"]
+
+
 MIXES = {
     # small CNN : Inception-v3 = 9 : 1
     "two_tenants": ([("mnist", "tvm_mnist", 0.9), ("inception_v3", "tvm_inception_v3", 0.1)], 400.0, 600),
