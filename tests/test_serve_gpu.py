@@ -174,12 +174,13 @@ def test_mixed_model_load_then_outputs_still_correct(cuda):
 
 
 @pytest.mark.parametrize("model,job", [("mnist", "tvm_mnist"), ("resnet18", "tvm_resnet18")])
-def test_copy_stages_still_serve_when_zero_copy_is_switched_off(cuda, model, job):
-    """PAELLA_ZERO_COPY_BYTES=0: every request goes host-to-device copy -> kernels -> device-to-host copy (pre-notify), the
-    reference's stage sequence; same results."""
+def test_reference_stage_sequence_still_serves_when_the_shortcuts_are_switched_off(cuda, model, job):
+    """PAELLA_ZERO_COPY_BYTES=0 and PAELLA_GROUP_THREADS=0: every request goes host-to-device copy -> one stage per kernel
+    -> device-to-host copy (pre-notify), the reference's stage sequence; same results."""
     from paella_amd import models, serve
     os.environ["LLIS_MODEL_SEED"] = "1"
     os.environ["PAELLA_ZERO_COPY_BYTES"] = "0"
+    os.environ["PAELLA_GROUP_THREADS"] = "0"
     try:
         desc = models.describe(model)
         x = om.make_input(desc, 23, "uniform" if model == "mnist" else "normal")
@@ -188,6 +189,7 @@ def test_copy_stages_still_serve_when_zero_copy_is_switched_off(cuda, model, job
         close(out, om.run(desc, x, seed=1))
     finally:
         del os.environ["PAELLA_ZERO_COPY_BYTES"]
+        del os.environ["PAELLA_GROUP_THREADS"]
 
 
 MIXES = {
