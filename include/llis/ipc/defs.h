@@ -1,6 +1,6 @@
 #pragma once
-// Identifier types and the client->server wire enums.  Numeric values are part of the IPC protocol and
-// match reference include/llis/ipc/defs.h:7-37 so a reference-built client can talk to this server.
+// Identifier types and the client->server wire enums.  The numeric values are part of the IPC protocol: they
+// equal those of reference include/llis/ipc/defs.h:7-37, so a reference-built client can talk to this server.
 
 #include <cstdint>
 
@@ -11,31 +11,35 @@ using JobRefId = uint32_t;
 using JobInstanceRefId = uint32_t;
 using JobId = uint32_t;
 
+// First word of every message on the client->server ring.
 enum class MsgType : uint32_t {
-    REGISTER_CLIENT = 0,
-    REGISTER_JOB = 1,
-    LAUNCH_JOB = 2,
-    GROW_POOL = 3,
-    CUDA_PROFILER_START = 4,
+    REGISTER_CLIENT = 0,      // {u32 temporary id}                         -> u32 client id on the temporary reply ring
+    REGISTER_JOB = 1,         // {u32 client, str library path, str pool}   -> u32 job reference id
+    LAUNCH_JOB = 2,           // {u32 job reference, i32 pool, size_t offset, void* client-side handle}
+    GROW_POOL = 3,            // {u32 job reference, size_t bytes}
+    CUDA_PROFILER_START = 4,  // (names kept from the reference; they switch the device profiler range on / off)
     CUDA_PROFILER_STOP = 5,
-    PROFILER_CMD = 6,
+    PROFILER_CMD = 6,         // {u32 ProfilerMsgType [, str path]}
     EXIT_CMD = 7,
 };
 
+// Sub-command of PROFILER_CMD.  Every record kind has a "set" (even) and an "unset" (odd) value; SAVE comes last.
+#define LLIS_PROFILER_RECORD_KINDS(X) \
+    X(KERNEL_INFO, 0)                 \
+    X(BLOCK_EXEC_TIME, 1)             \
+    X(KERNEL_BLOCK_MIS_ALLOC, 2)      \
+    X(RUN_NEXT_TIMES, 3)              \
+    X(JOB_EVENTS, 4)                  \
+    X(RESOURCE_EVENTS, 5)
+
 enum class ProfilerMsgType : uint32_t {
-    SET_RECORD_KERNEL_INFO = 0,
-    UNSET_RECORD_KERNEL_INFO = 1,
-    SET_RECORD_BLOCK_EXEC_TIME = 2,
-    UNSET_RECORD_BLOCK_EXEC_TIME = 3,
-    SET_RECORD_KERNEL_BLOCK_MIS_ALLOC = 4,
-    UNSET_RECORD_KERNEL_BLOCK_MIS_ALLOC = 5,
-    SET_RECORD_RUN_NEXT_TIMES = 6,
-    UNSET_RECORD_RUN_NEXT_TIMES = 7,
-    SET_RECORD_JOB_EVENTS = 8,
-    UNSET_RECORD_JOB_EVENTS = 9,
-    SET_RECORD_RESOURCE_EVENTS = 10,
-    UNSET_RECORD_RESOURCE_EVENTS = 11,
+#define LLIS_PROFILER_MSG(kind, index) SET_RECORD_##kind = 2 * (index), UNSET_RECORD_##kind = 2 * (index) + 1,
+    LLIS_PROFILER_RECORD_KINDS(LLIS_PROFILER_MSG)
+#undef LLIS_PROFILER_MSG
     SAVE = 12,
 };
+
+static_assert((uint32_t)ProfilerMsgType::UNSET_RECORD_RESOURCE_EVENTS == 11 && (uint32_t)ProfilerMsgType::SET_RECORD_RUN_NEXT_TIMES == 6,
+              "profiler sub-commands are wire values");
 
 }  // namespace llis

@@ -1,10 +1,12 @@
 #pragma once
-// What the server keeps per registered client: its completion ring and its wake-up socket address
-// (reference include/llis/server/client_connection.h:10-37).
+// What the server keeps per registered client: the ring its completions go to, the datagram socket it is woken on,
+// and the wake-ups it is still owed (reference include/llis/server/client_connection.h:10-37 holds the first two).
 
 #include <llis/ipc/defs.h>
 #include <llis/ipc/shm_channel.h>
 #include <llis/ipc/unix_datagram_socket.h>
+
+#include <utility>
 
 namespace llis {
 namespace server {
@@ -13,18 +15,41 @@ class ClientConnection {
   public:
     explicit ClientConnection(ClientId client_id) : client_id_(client_id) {}
 
-    void use_s2c_channel(ipc::ShmChannelCpuWriter&& channel) { s2c_channel_ = std::move(channel); }
-    void use_s2c_socket(ipc::UnixDatagramSocket&& sock) { s2c_socket_ = std::move(sock); }
-
-    ipc::ShmChannelCpuWriter* get_s2c_channel() { return &s2c_channel_; }
-    ipc::UnixDatagramSocket* get_s2c_socket() { return &s2c_socket_; }
     ClientId get_client_id() const { return client_id_; }
 
-    // Wake-ups that could not be delivered yet because the client's socket queue was full.
-    unsigned owed_wakeups = 0;
+    void use_s2c_channel(ipc::ShmChannelCpuWriter&& channel) { s2c_channel_ = std::move(channel); }
+    void use_s2c_socket(ipc::UnixDatagramSocket&& sock) { s2c_socket_ = std::move(sock); }
+    ipc::ShmChannelCpuWriter* get_s2c_channel() { return &s2c_channel_; }
+    ipc::UnixDatagramSocket* get_s2c_socket() { return &s2c_socket_; }
+
+    // One-byte poke that gets the client out of wait().  The kernel queues only a handful of datagrams per socket, and
+    // a client with many requests in flight that is slow to call wait() must not stall the serving thread: the poke
+    // never blocks, and one that did not fit is owed (they are all the same byte, so order does not matter).
+    // Returns true if the poke is owed rather than sent.
+    bool wake() {
+        if (owed_wakeups_ == 0 && poke()) return false;
+        ++owed_wakeups_;
+        return true;
+    }
+
+    // Sends as many owed pokes as fit now; returns how many went out.
+    unsigned retry_wakeups() {
+        unsigned sent = 0;
+        while (owed_wakeups_ != 0 && poke()) {
+            --owed_wakeups_;
+            ++sent;
+        }
+        return sent;
+    }
 
   private:
+    bool poke() {
+        const bool byte = true;
+        return s2c_socket_.try_write(&byte, sizeof(byte));
+    }
+
     ClientId client_id_;
+    unsigned owed_wakeups_ = 0;
     ipc::ShmChannelCpuWriter s2c_channel_;
     ipc::UnixDatagramSocket s2c_socket_;
 };

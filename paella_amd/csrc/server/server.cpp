@@ -46,13 +46,7 @@ void Server::poll_once() {
 
 void Server::retry_owed_wakeups() {
     polls_since_retry_ = 0;
-    const bool msg = true;
-    for (auto& conn : client_connections_) {
-        while (conn->owed_wakeups != 0 && conn->get_s2c_socket()->try_write(&msg, sizeof(msg))) {
-            --conn->owed_wakeups;
-            --total_owed_wakeups_;
-        }
-    }
+    for (auto& conn : client_connections_) total_owed_wakeups_ -= conn->retry_wakeups();
 }
 
 void Server::handle_c2s() {
@@ -123,15 +117,8 @@ void Server::handle_grow_pool() {
 }
 
 void Server::notify_job_starts(job::Job* job) {
-    // The kernel queues only a handful of datagrams per socket; a client that has many requests in flight
-    // and is slow to call wait() must not stall or kill the serving thread, so the poke is non-blocking and
-    // undelivered ones are retried from the poll loop (order does not matter: they are all the same byte).
-    const bool msg = true;
-    ClientConnection* conn = client_connections_[job->get_client_id()].get();
-    if (conn->owed_wakeups != 0 || !conn->get_s2c_socket()->try_write(&msg, sizeof(msg))) {
-        ++conn->owed_wakeups;
-        ++total_owed_wakeups_;
-    }
+    // never blocks: a poke that does not fit the client's socket queue is retried from the poll loop
+    if (client_connections_[job->get_client_id()]->wake()) ++total_owed_wakeups_;
 }
 
 void Server::notify_job_ends(job::Job* job) {
