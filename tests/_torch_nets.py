@@ -180,7 +180,40 @@ class FaceStyle(nn.Module):
         return self.fc(torch.flatten(x, 1))
 
 
+class PreActBlock(nn.Module):
+    """ResNet v2 unit (the layout of the resnet*-v2-7 zoo files): norm and relu come BEFORE each conv, the shortcut
+    branches off after the first norm+relu when it projects, and nothing follows the addition."""
+
+    def __init__(self, cin, cout, stride):
+        super().__init__()
+        self.bn1, self.conv1 = nn.BatchNorm2d(cin), nn.Conv2d(cin, cout, 3, stride, 1, bias=False)
+        self.bn2, self.conv2 = nn.BatchNorm2d(cout), nn.Conv2d(cout, cout, 3, 1, 1, bias=False)
+        self.project = nn.Conv2d(cin, cout, 1, stride, bias=False) if (stride != 1 or cin != cout) else None
+
+    def forward(self, x):
+        a = F.relu(self.bn1(x))
+        shortcut = x if self.project is None else self.project(a)
+        y = self.conv1(a)
+        y = self.conv2(F.relu(self.bn2(y)))
+        return y + shortcut
+
+
+class ResNetV2Style(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.bn_data = nn.BatchNorm2d(3)
+        self.conv0, self.bn0 = nn.Conv2d(3, 8, 7, 2, 3, bias=False), nn.BatchNorm2d(8)
+        self.blocks = nn.Sequential(PreActBlock(8, 8, 1), PreActBlock(8, 16, 2), PreActBlock(16, 16, 1))
+        self.bn_last, self.fc = nn.BatchNorm2d(16), nn.Linear(16, 11)
+
+    def forward(self, x):
+        x = F.max_pool2d(F.relu(self.bn0(self.conv0(self.bn_data(x)))), 3, 2, 1)
+        x = F.relu(self.bn_last(self.blocks(x)))
+        return self.fc(torch.flatten(F.adaptive_avg_pool2d(x, 1), 1))
+
+
 NETS = {
+    "resnet_v2_style": (ResNetV2Style, (1, 3, 40, 40)),
     "resnet_style": (lambda: ResNet((1, 2), 8, 10), (1, 3, 32, 32)),
     "squeeze_style": (SqueezeStyle, (1, 3, 47, 47)),
     "mobile_style": (MobileStyle, (1, 3, 32, 32)),
