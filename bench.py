@@ -234,6 +234,8 @@ def main():
     ap.add_argument("--no-arms", action="store_true", help="skip the comparison arms and the Poisson sweep")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mix", action="store_true", help="skip the small-CNN + Inception-v3 two-tenant arm")
+    ap.add_argument("--mem-notify", choices=["marker", "hostfunc"], default="marker",
+                    help="how the end of a copy stage reaches the scheduler in the timed arms: ring-marker kernel or host callback")
     ap.add_argument("--fairness-sweep", action="store_true",
                     help="also sweep full3's deficit threshold over a ResNet-18 : Inception-v3 = 0.952 : 0.048 mix and report Jain's index")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -280,11 +282,13 @@ def main():
         args.no_arms = args.no_cpu = True
         main_run, value = None, None
     else:
-        main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup, extra_kernels=args.extra_kernels)
+        main_run = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, args.steps, args.warmup, extra_kernels=args.extra_kernels,
+                             mem_marker=args.mem_notify == "marker")
         value = main_run["throughput_rps"]
         log("[bench]   %.1f req/s" % value)
         os.environ["PAELLA_INPUT_RESIDENT"] = "0"
-        r = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, max(500, args.steps // 2), args.warmup // 2, extra_kernels=args.extra_kernels)
+        r = serve_arm(serve, "full3", args.num_streams, jobs, args.concurrency, max(500, args.steps // 2), args.warmup // 2, extra_kernels=args.extra_kernels,
+                      mem_marker=args.mem_notify == "marker")
         pcie_inclusive = r["throughput_rps"]
         log("[bench]   %.1f req/s with the host-to-device copy of every request's input" % pcie_inclusive)
         os.environ["PAELLA_INPUT_RESIDENT"] = "1"
@@ -408,13 +412,14 @@ def main():
         log("[bench]   fp32 MFMA rate measured with a register-resident loop: %.1f TFLOP/s" % peak.value)
     floor = ctypes.c_double()
     if lib.paella_empty_kernel_probe(200, ctypes.byref(floor)) == 0 and floor.value > 0:
-        # what the same time stamps report for a kernel that does nothing: every launch pays it, so at batch 1 the
-        # 20 conv launches of a pass cannot beat flops / (20 x floor) however fast the kernels are
+        # what the same time stamps report for a kernel that does nothing (the profiler's kernel trace gives 1.4 us for
+        # it): every per-launch figure taken this way contains it, so measured like this the 20 conv launches of a pass
+        # cannot show more than flops / (20 x floor) however fast the kernels are
         bound = rl["conv_flops"] / (rl["conv_launches"] * floor.value * 1e-6) / 1e12
         roofline["empty_kernel_us"] = floor.value
         roofline["launch_bound_tflops"] = bound
         roofline["frac_of_launch_bound"] = achieved / bound
-        log("[bench]   an empty kernel takes %.2f us by the same time stamps: launch-bound ceiling %.1f TFLOP/s, conv at %.0f%% of it" %
+        log("[bench]   an empty kernel is %.2f us long by the same time stamps: ceiling of this measurement %.1f TFLOP/s, conv at %.0f%% of it" %
             (floor.value, bound, 100 * achieved / bound))
     ring = ctypes.c_void_p()
     notify = {}
