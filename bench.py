@@ -449,7 +449,8 @@ def main():
                     "what": "host clock when the message became readable minus the lane's realtime counter just before the ring write, "
                             "translated to the host clock by the runtime"}
             log("[bench]   notification: echo round trip p50 %.2f / p99 %.2f us%s" % (rtt[n_echo // 2], rtt[int(n_echo * 0.99)],
-                ", device->host p50 %.2f / p99 %.2f us" % (ow[len(ow) // 2], ow[int(len(ow) * 0.99)]) if len(ow) else ""))
+                "" if not len(ow) else (", device->host p50 %.2f / p99 %.2f us" % (ow[len(ow) // 2], ow[int(len(ow) * 0.99)])) +
+                ("" if 0.0 < ow[len(ow) // 2] < rtt[n_echo // 2] else " (outside the round trip: the runtime's clock translation is off by more than that here)")))
         lib.paella_ring_destroy(ring)
 
     cpu = None if args.no_cpu else cpu_baseline(args.model, args.cpu_seconds)

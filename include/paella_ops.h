@@ -91,6 +91,29 @@ int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const voi
                          const float* residual, const float* slope, float* y, void* workspace,
                          void* stream, uint32_t job_id, void* notifier);
 
+/* Two convs that do not depend on each other as ONE launch: the first problem's workgroups followed by the
+ * second's, so that layers whose own grids are far below the 256 CUs (the 1x1 projection beside a residual block's
+ * first 3x3 conv, parallel branches of an inception module) fill the device together and cost one dispatch.  No
+ * counterpart in the reference, whose generated code launches every operator by itself.  Both plans must be MFMA
+ * plans with mi == ni == 1 and the same kw and k_order (paella_conv2d_pair_dims returns PAELLA_ENOSUP otherwise; a
+ * plan can be forced to that shape with tile_hint); neither conv may read or overwrite what the other writes, and
+ * two split plans need separate workspaces.  The results are bit-identical to two paella_conv2d_launch calls.
+ * The hooks report one kernel of dims->grid workgroups. */
+typedef struct paella_conv_operands {
+    const paella_conv_plan* plan;
+    const float* x;
+    const void* blob_dev;
+    const float* bias;
+    const float* residual;
+    const float* slope;
+    float* y;
+    void* workspace;
+} paella_conv_operands;
+
+int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_plan* second, paella_launch_dims* dims);
+int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second,
+                              void* stream, uint32_t job_id, void* notifier);
+
 /* ---------------------------------------------------------------- dense (O3) */
 
 /* y[o] = act(bias[o] + sum_i x[i] * w[o][i]); w is the plain [O][I] row-major matrix. */

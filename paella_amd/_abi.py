@@ -26,6 +26,10 @@ class ConvPlan(ctypes.Structure):
                 ("flops", c_double), ("bytes", c_double)]
 
 
+class ConvOperands(ctypes.Structure):
+    _fields_ = [("plan", ctypes.POINTER(ConvPlan))] + [(n, c_void_p) for n in ("x", "blob_dev", "bias", "residual", "slope", "y", "workspace")]
+
+
 class PoolDesc(ctypes.Structure):
     _fields_ = [(n, c_int) for n in ("C", "H", "W", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w",
                                      "ceil_mode", "is_avg", "count_include_pad")]
@@ -73,6 +77,8 @@ OPS_SYMBOLS = {
     "paella_conv2d_plan": (c_int, [ctypes.POINTER(ConvDesc), c_int, c_int, ctypes.POINTER(ConvPlan)]),
     "paella_conv2d_pack": (c_int, [ctypes.POINTER(ConvPlan), c_void_p, c_void_p]),
     "paella_conv2d_launch": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 7 + _TAIL),
+    "paella_conv2d_pair_dims": (c_int, [ctypes.POINTER(ConvPlan), ctypes.POINTER(ConvPlan), ctypes.POINTER(LaunchDims)]),
+    "paella_conv2d_launch_pair": (c_int, [ctypes.POINTER(ConvOperands), ctypes.POINTER(ConvOperands)] + _TAIL),
     "paella_dense_dims": (c_int, [c_int, c_int, ctypes.POINTER(LaunchDims)]),
     "paella_dense_launch": (c_int, [c_void_p] * 4 + [c_int] * 3 + _TAIL),
     "paella_pool_out": (c_int, [c_int] * 5),

@@ -34,7 +34,7 @@ int g_direct_queue_count = 0;
 namespace {
 
 constexpr uint32_t kQueuePackets = 4096;       // ring size (power of two)
-constexpr uint32_t kKernargSlotBytes = 512;    // one slot per packet index: explicit args <= 256 + implicit block 256
+constexpr uint32_t kKernargSlotBytes = 768;    // one slot per packet index: explicit args <= 448 + implicit block 256
 constexpr size_t kImplicitBytes = 256;
 
 struct Runtime {
@@ -235,6 +235,7 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     char* ka = q->kernargs + (size_t)slot * kKernargSlotBytes;
     // The implicit block starts at the next 8-byte boundary; a kernel that uses none of it has a shorter segment.
     const size_t implicit_at = (explicit_bytes + 7) & ~(size_t)7;
+    static_assert(kMaxExplicitArgBytes + kImplicitBytes <= kKernargSlotBytes, "a slot holds the largest argument block");
     if (explicit_bytes > kernel->kernarg_bytes) {
         std::fprintf(stderr, "[paella] direct dispatch: %zu argument bytes for a kernel that takes %u\n", explicit_bytes, kernel->kernarg_bytes);
         std::abort();

@@ -104,8 +104,9 @@ struct Frag {
 #define PAELLA_CONV_MINB 1
 #endif
 
+// One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
 template <int MI, int NI, int KW, bool TAP_MAJOR>
-__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
+__device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid) {
     CONV_TL(0);
     if (PAELLA_CONV_ABLATE & 16) return;
     paella::hook_entry(p.notifier, p.job_id);
@@ -126,9 +127,9 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     int tile_n, tile_m, split;
     {
         const unsigned total = (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits);
-        const unsigned xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+        const unsigned xcd = bid & 7u, j = bid >> 3;
         const unsigned q = total >> 3, r = total & 7u;
-        const unsigned w = p.slab_major == 2 ? blockIdx.x : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
+        const unsigned w = p.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
         if (p.slab_major) {
             const unsigned slab = w / (unsigned)p.n_tiles_n;
             tile_n = (int)(w - slab * (unsigned)p.n_tiles_n);
@@ -449,6 +450,28 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
 #endif
 }
 
+template <int MI, int NI, int KW, bool TAP_MAJOR>
+__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
+    conv_tile<MI, NI, KW, TAP_MAJOR>(p, blockIdx.x);
+}
+
+// Two independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
+// projection beside a residual block's first 3x3, the parallel branches of an inception module) share a grid, the
+// first problem's workgroups followed by the second's.  Both use the smallest tile and the same wave count; the
+// hooks see one kernel of first_grid + second grid workgroups.
+struct ConvPairArgs {
+    ConvArgs first, second;
+    unsigned first_grid;
+};
+
+template <int KW, bool TAP_MAJOR>
+__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_pair_kernel(ConvPairArgs g) {
+    const bool second = blockIdx.x >= g.first_grid;  // the same for the whole workgroup
+    ConvArgs p = g.first;
+    if (second) p = g.second;
+    conv_tile<1, 1, KW, TAP_MAJOR>(p, second ? blockIdx.x - g.first_grid : blockIdx.x);
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Depthwise conv (groups == C == K): HBM-bound, one thread per output pixel, taps from L1/L2.
 
@@ -641,6 +664,106 @@ extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, 
     return 0;
 }
 
+namespace {
+
+// Kernel arguments of one MFMA conv (plan->kind == 0).
+int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias, const float* residual,
+              const float* slope, float* y, void* workspace, uint32_t job_id, llis::job::FinishedBlockNotifier* nf, ConvArgs& a) {
+    if (!plan || !x || !blob_dev || !y || plan->kind != 0) return PAELLA_EINVAL;
+    const paella_conv_desc& d = plan->d;
+    if (d.act == PAELLA_ACT_PRELU && !slope) return PAELLA_EINVAL;
+    const int PQ = plan->P * plan->Q;
+    a.x = x;
+    a.wpk = reinterpret_cast<const float4*>(blob_dev);
+    a.w_bytes = (unsigned)plan->blob_bytes;
+    a.kdim = d.C * d.R * d.S; a.RS = d.R * d.S; a.S = d.S; a.dh = d.dil_h; a.dw = d.dil_w;
+    a.CB = d.C / 8;
+    a.bias = bias;
+    a.residual = residual;
+    a.slope = slope;
+    a.y = y;
+    a.H = d.H; a.W = d.W; a.Q = plan->Q; a.PQ = PQ;
+    a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
+    a.K = d.K; a.m_pad = plan->m_pad; a.nchunks = plan->k_pad / 8;
+    a.splits = plan->splits;
+    a.chunks_per_split = (a.nchunks + plan->splits - 1) / plan->splits;
+    a.ws_partials = nullptr;
+    a.ws_counters = nullptr;
+    if (plan->splits > 1) {
+        if (!workspace) return PAELLA_EINVAL;
+        // counters first (they must be zero before the first launch; the kernel leaves them at zero)
+        a.ws_counters = reinterpret_cast<unsigned*>(workspace);
+        a.ws_partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kMaxSplitTiles * sizeof(unsigned));
+    }
+    a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
+    a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
+    a.job_id = job_id;
+    a.notifier = nf;
+    a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
+    a.n_tiles_m = plan->m_pad / (32 * plan->mi);
+    // Weights outweigh the input: keep the workgroups that read one slab of weights on one XCD.
+    a.slab_major = (double)d.K * d.C * d.R * d.S > (double)d.C * d.H * d.W ? 1 : 0;
+    if (const char* force = std::getenv("PAELLA_CONV_ORDER")) a.slab_major = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : a.slab_major));
+    return 0;
+}
+
+int allow_lds(const void* kern, unsigned lds_bytes) {
+    if (lds_bytes <= 65536) return 0;
+    return (int)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+}
+
+typedef void (*ConvPairKernel)(ConvPairArgs);
+
+ConvPairKernel pick_pair_kernel(int kw, int k_order) {
+    switch (kw) {
+        case 1: return k_order ? conv_mfma_pair_kernel<1, true> : conv_mfma_pair_kernel<1, false>;
+        case 2: return k_order ? conv_mfma_pair_kernel<2, true> : conv_mfma_pair_kernel<2, false>;
+        case 4: return k_order ? conv_mfma_pair_kernel<4, true> : conv_mfma_pair_kernel<4, false>;
+        case 8: return k_order ? conv_mfma_pair_kernel<8, true> : conv_mfma_pair_kernel<8, false>;
+        default: return nullptr;
+    }
+}
+
+}  // namespace
+
+extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* a, const paella_conv_plan* b, paella_launch_dims* dims) {
+    if (!a || !b) return PAELLA_EINVAL;
+    if (a->kind != 0 || b->kind != 0 || a->mi != 1 || a->ni != 1 || b->mi != 1 || b->ni != 1 || a->kw != b->kw || a->k_order != b->k_order)
+        return PAELLA_ENOSUP;
+    if (dims) {
+        dims->grid = a->dims.grid + b->dims.grid;
+        dims->block = a->dims.block;
+        dims->lds_bytes = a->dims.lds_bytes > b->dims.lds_bytes ? a->dims.lds_bytes : b->dims.lds_bytes;
+        dims->vgprs = a->dims.vgprs;
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_pair_kernel(a->kw, a->k_order))) == hipSuccess && attr.numRegs > 0)
+            dims->vgprs = (unsigned)attr.numRegs;
+        else
+            (void)hipGetLastError();
+    }
+    return 0;
+}
+
+extern "C" int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second, void* stream, uint32_t job_id,
+                                         void* notifier) {
+    if (!first || !second) return PAELLA_EINVAL;
+    paella_launch_dims dims;
+    if (int rc = paella_conv2d_pair_dims(first->plan, second->plan, &dims)) return rc;
+    if (first->plan->splits > 1 && second->plan->splits > 1 && first->workspace == second->workspace) return PAELLA_EINVAL;
+    auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
+    ConvPairArgs g;
+    if (int rc = fill_args(first->plan, first->x, first->blob_dev, first->bias, first->residual, first->slope, first->y, first->workspace, job_id, nf, g.first))
+        return rc;
+    if (int rc = fill_args(second->plan, second->x, second->blob_dev, second->bias, second->residual, second->slope, second->y, second->workspace, job_id,
+                           nf, g.second))
+        return rc;
+    g.first_grid = first->plan->dims.grid;
+    ConvPairKernel kern = pick_pair_kernel(first->plan->kw, first->plan->k_order);
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
+    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
+    return (int)hipGetLastError();
+}
+
 extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
                                     const float* residual, const float* slope, float* y, void* workspace, void* stream,
                                     uint32_t job_id, void* notifier) {
@@ -654,45 +777,9 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
         ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order);
         if (!kern) return PAELLA_EINVAL;
         ConvArgs a;
-        a.x = x;
-        a.wpk = reinterpret_cast<const float4*>(blob_dev);
-        a.w_bytes = (unsigned)plan->blob_bytes;
-        a.kdim = d.C * d.R * d.S; a.RS = d.R * d.S; a.S = d.S; a.dh = d.dil_h; a.dw = d.dil_w;
-        a.CB = d.C / 8;
-        a.bias = bias;
-        a.residual = residual;
-        a.slope = slope;
-        a.y = y;
-        a.H = d.H; a.W = d.W; a.Q = plan->Q; a.PQ = PQ;
-        a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
-        a.K = d.K; a.m_pad = plan->m_pad; a.nchunks = plan->k_pad / 8;
-        a.splits = plan->splits;
-        a.chunks_per_split = (a.nchunks + plan->splits - 1) / plan->splits;
-        a.ws_partials = nullptr;
-        a.ws_counters = nullptr;
-        if (plan->splits > 1) {
-            if (!workspace) return PAELLA_EINVAL;
-            const size_t n_tiles = (size_t)((PQ + 32 * plan->ni - 1) / (32 * plan->ni)) * (plan->m_pad / (32 * plan->mi));
-            // counters first (they must be zero before the first launch; the kernel leaves them at zero)
-            a.ws_counters = reinterpret_cast<unsigned*>(workspace);
-            a.ws_partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kMaxSplitTiles * sizeof(unsigned));
-            (void)n_tiles;
-        }
-        a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
-        a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
-        a.job_id = job_id;
-        a.notifier = nf;
-        a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
-        a.n_tiles_m = plan->m_pad / (32 * plan->mi);
-        // Weights outweigh the input: keep the workgroups that read one slab of weights on one XCD.
-        a.slab_major = (double)d.K * d.C * d.R * d.S > (double)d.C * d.H * d.W ? 1 : 0;
-        if (const char* force = std::getenv("PAELLA_CONV_ORDER")) a.slab_major = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : a.slab_major));
-        dim3 grid((unsigned)(a.n_tiles_n * a.n_tiles_m * plan->splits), 1, 1);
-        if (plan->dims.lds_bytes > 65536) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->dims.lds_bytes);
-            if (e != hipSuccess) return (int)e;
-        }
-        paella::launch(kern, grid, dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
+        if (int rc = fill_args(plan, x, blob_dev, bias, residual, slope, y, workspace, job_id, nf, a)) return rc;
+        if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
+        paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
         return (int)hipGetLastError();
     }
     DwArgs a;

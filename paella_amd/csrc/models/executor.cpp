@@ -7,6 +7,7 @@
 #include "paella_models.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -31,12 +32,24 @@ struct StagePlan {
     const float* shift = nullptr;
 };
 
+// One launch: an operator, or two convs that do not depend on each other sharing a grid.
+struct Launch {
+    int first = -1, second = -1;  // node indices; second < 0: a single operator
+    paella_launch_dims dims{};
+};
+
 struct paella_model {
     Graph g;
-    size_t workspace_bytes = 0;  // largest conv workspace of any stage (stages of one request never overlap)
+    // Split-reduction scratch of a request (stages of one request never overlap).  Every conv expects arrival
+    // counters that read zero at the head of its workspace and partial tiles behind them, so the second convs of
+    // pairs get an area of their own: a first conv's partial tiles never land on a second conv's counters.
+    size_t workspace_bytes = 0;
+    size_t ws_second = 0;        // byte offset of that area
     uint64_t seed = 0;
+    bool pairing = true;
     char* weights_dev = nullptr;
-    std::vector<StagePlan> stages;
+    std::vector<StagePlan> plans;   // one per node
+    std::vector<Launch> stages;     // in execution order
 };
 
 struct paella_exec {
@@ -56,7 +69,14 @@ struct paella_exec {
 namespace {
 
 std::mutex g_mtx;
-std::map<std::pair<std::string, uint64_t>, std::unique_ptr<paella_model>> g_models;
+std::map<std::pair<std::string, uint64_t>, std::unique_ptr<paella_model>> g_models;  // name + '|' + pairing -> model
+
+// Whether models built now put two independent convs into one launch (the environment is read at every build, so
+// a process can hold both forms of a model).
+bool pairing_enabled() {
+    const char* env = std::getenv("PAELLA_CONV_PAIRS");
+    return !(env && env[0] == '0');
+}
 std::map<std::string, std::unique_ptr<Graph>> g_graphs;
 
 const Graph* graph_of(const char* name) {
@@ -82,16 +102,74 @@ unsigned vgprs_or(const char* family, unsigned fallback) {
     return paella_kernel_vgprs(family, &v) == 0 && v > 0 ? v : fallback;
 }
 
+int log2_ceil(int v) {
+    int b = 0;
+    while ((1 << b) < v) ++b;
+    return b;
+}
+
+// Lays the nodes out as launches.  Two consecutive MFMA convs on the smallest tile go out as one launch when
+// neither reads or overwrites what the other writes and at least one of them would leave CUs idle by itself
+// (PAELLA_CONV_PAIRS=0 switches this off).  The one with fewer waves per workgroup is re-planned to the other's
+// count; its packed weights do not depend on that.
+void pair_up(paella_model* m) {
+    const Graph& g = m->g;
+    const bool enabled = m->pairing;
+    auto overlap = [&](const View& a, const View& b) {
+        if (a.buf < 0 || b.buf < 0) return false;
+        const size_t a0 = g.buffers[a.buf].offset + a.off, b0 = g.buffers[b.buf].offset + b.off;
+        return a0 < b0 + b.numel() && b0 < a0 + a.numel();
+    };
+    auto independent = [&](const Node& a, const Node& b) {
+        return !overlap(a.y, b.x) && !overlap(a.y, b.x2) && !overlap(a.y, b.y) && !overlap(b.y, a.x) && !overlap(b.y, a.x2);
+    };
+    auto small_tile = [](const StagePlan& st) { return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1; };
+    m->stages.clear();
+    size_t ws_first = 0, ws_second = 0;
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        Launch l;
+        l.first = (int)i;
+        l.dims = m->plans[i].dims;
+        if (enabled && i + 1 < g.nodes.size() && small_tile(m->plans[i]) && small_tile(m->plans[i + 1]) &&
+            m->plans[i].conv.k_order == m->plans[i + 1].conv.k_order && independent(g.nodes[i], g.nodes[i + 1]) &&
+            (m->plans[i].dims.grid <= 256 || m->plans[i + 1].dims.grid <= 256)) {
+            StagePlan a = m->plans[i], b = m->plans[i + 1];
+            const int kw = a.conv.kw > b.conv.kw ? a.conv.kw : b.conv.kw;
+            bool ok = true;
+            for (StagePlan* st : {&a, &b}) {
+                if (st->conv.kw == kw) continue;
+                const int hint = log2_ceil(st->conv.splits) << 12 | 1 << 8 | 1 << 4 | log2_ceil(kw);
+                ok = ok && paella_conv2d_plan(&st->node->conv, st->node->x2.buf >= 0, hint, &st->conv) == 0;
+                st->dims = st->conv.dims;
+            }
+            paella_launch_dims dims{};
+            if (ok && a.conv.blob_bytes == m->plans[i].conv.blob_bytes && b.conv.blob_bytes == m->plans[i + 1].conv.blob_bytes &&
+                paella_conv2d_pair_dims(&a.conv, &b.conv, &dims) == 0) {
+                m->plans[i] = a;
+                m->plans[i + 1] = b;
+                l.second = (int)i + 1;
+                l.dims = dims;
+                if (b.conv.workspace_bytes > ws_second) ws_second = b.conv.workspace_bytes;
+                ++i;
+            }
+        }
+        if (g.nodes[l.first].op == Op::Conv && m->plans[l.first].conv.workspace_bytes > ws_first) ws_first = m->plans[l.first].conv.workspace_bytes;
+        m->stages.push_back(l);
+    }
+    m->ws_second = align256(ws_first);
+    m->workspace_bytes = ws_second ? m->ws_second + ws_second : ws_first;
+}
+
 int build(paella_model* m) {
     const Graph& g = m->g;
     // Pass 1: plan every node and lay out the weight arena.
     std::vector<size_t> tensor_off(g.weights.size(), (size_t)-1);
     std::vector<size_t> blob_off(g.nodes.size(), (size_t)-1);
     size_t total = 0;
-    m->stages.resize(g.nodes.size());
+    m->plans.resize(g.nodes.size());
     for (size_t i = 0; i < g.nodes.size(); ++i) {
         const Node& n = g.nodes[i];
-        StagePlan& st = m->stages[i];
+        StagePlan& st = m->plans[i];
         st.node = &n;
         int rc = 0;
         switch (n.op) {
@@ -108,7 +186,6 @@ int build(paella_model* m) {
                 }
                 blob_off[i] = total;
                 total += align256(st.conv.blob_bytes);
-                if (st.conv.workspace_bytes > m->workspace_bytes) m->workspace_bytes = st.conv.workspace_bytes;
                 break;
             case Op::Dense:
                 rc = paella_dense_dims(n.dense_in, n.dense_out, &st.dims);
@@ -157,6 +234,8 @@ int build(paella_model* m) {
         }
     }
 
+    pair_up(m);
+
     // Pass 2: generate, pack, upload.
     std::vector<char> host(total, 0);
     std::vector<float> tmp;
@@ -169,7 +248,7 @@ int build(paella_model* m) {
         if (n.op != Op::Conv) continue;
         tmp.resize(g.weights[n.w].numel());
         fill_weight(g.weights[n.w], m->seed, (uint64_t)n.w, tmp.data());
-        int rc = paella_conv2d_pack(&m->stages[i].conv, tmp.data(), host.data() + blob_off[i]);
+        int rc = paella_conv2d_pack(&m->plans[i].conv, tmp.data(), host.data() + blob_off[i]);
         if (rc) return rc;
     }
     void* dev = nullptr;
@@ -180,7 +259,7 @@ int build(paella_model* m) {
     m->weights_dev = reinterpret_cast<char*>(dev);
     for (size_t i = 0; i < g.nodes.size(); ++i) {
         const Node& n = g.nodes[i];
-        StagePlan& st = m->stages[i];
+        StagePlan& st = m->plans[i];
         auto at = [&](int id) -> const float* { return id >= 0 ? reinterpret_cast<const float*>(m->weights_dev + tensor_off[id]) : nullptr; };
         st.w = n.op == Op::Conv ? (const void*)(m->weights_dev + blob_off[i]) : (const void*)at(n.w);
         st.bias = at(n.bias);
@@ -257,12 +336,14 @@ int paella_model_get(const char* name, uint64_t seed, paella_model** out) {
     const Graph* g = graph_of(name);
     if (!g || !out) return PAELLA_EINVAL;
     std::lock_guard<std::mutex> lk(g_mtx);
-    auto key = std::make_pair(std::string(name), seed);
+    const bool pairing = pairing_enabled();
+    auto key = std::make_pair(std::string(name) + (pairing ? "|pairs" : "|single"), seed);
     auto it = g_models.find(key);
     if (it == g_models.end()) {
         auto m = std::make_unique<paella_model>();
         m->g = *g;
         m->seed = seed;
+        m->pairing = pairing;
         if (int rc = build(m.get())) return rc;
         it = g_models.emplace(key, std::move(m)).first;
     }
@@ -280,10 +361,18 @@ int paella_model_stage_dims(const paella_model* m, int stage, paella_launch_dims
 
 int paella_model_stage_work(const paella_model* m, int stage, const char** op, double* flops, double* bytes) {
     if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
-    if (op) *op = m->stages[stage].op;
-    if (flops) *flops = m->stages[stage].flops;
-    if (bytes) *bytes = m->stages[stage].bytes;
+    const Launch& l = m->stages[stage];
+    const StagePlan& a = m->plans[l.first];
+    const StagePlan* b = l.second >= 0 ? &m->plans[l.second] : nullptr;
+    if (op) *op = a.op;
+    if (flops) *flops = a.flops + (b ? b->flops : 0);
+    if (bytes) *bytes = a.bytes + (b ? b->bytes : 0);
     return 0;
+}
+
+int paella_model_stage_operators(const paella_model* m, int stage) {
+    if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
+    return m->stages[stage].second >= 0 ? 2 : 1;
 }
 
 int paella_exec_create(const paella_model* m, paella_exec** out) {
@@ -340,8 +429,17 @@ void* paella_exec_output(paella_exec* e) { return e ? e->ptr(e->m->g.output) : n
 
 int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier) {
     if (!e || stage < 0 || (size_t)stage >= e->m->stages.size()) return PAELLA_EINVAL;
-    const StagePlan& st = e->m->stages[stage];
+    const Launch& l = e->m->stages[stage];
+    const StagePlan& st = e->m->plans[l.first];
     const Node& n = *st.node;
+    if (l.second >= 0) {
+        const StagePlan& st2 = e->m->plans[l.second];
+        const Node& n2 = *st2.node;
+        const paella_conv_operands a{&st.conv, e->ptr(n.x), st.w, st.bias, e->ptr(n.x2), st.slope, e->ptr(n.y), e->workspace};
+        const paella_conv_operands b{&st2.conv, e->ptr(n2.x), st2.w, st2.bias, e->ptr(n2.x2), st2.slope, e->ptr(n2.y),
+                                     e->workspace ? static_cast<char*>(e->workspace) + e->m->ws_second : nullptr};
+        return paella_conv2d_launch_pair(&a, &b, stream, job_id, notifier);
+    }
     const float* x = e->ptr(n.x);
     const float* x2 = e->ptr(n.x2);
     float* y = e->ptr(n.y);

@@ -65,6 +65,9 @@ class Exec:
         check(self.lib.paella_model_stage_dims(self.model, i, ctypes.byref(d)), "paella_model_stage_dims")
         return d
 
+    def stage_operators(self, i):
+        return self.lib.paella_model_stage_operators(self.model, i)
+
     def stage_work(self, i):
         op, f, b = ctypes.c_char_p(), ctypes.c_double(), ctypes.c_double()
         check(self.lib.paella_model_stage_work(self.model, i, ctypes.byref(op), f, b), "paella_model_stage_work")

@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from . import _abi
-from ._abi import ConvDesc, ConvPlan, LaunchDims, PoolDesc, check
+from ._abi import ConvDesc, ConvOperands, ConvPlan, LaunchDims, PoolDesc, check
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_PRELU, ACT_CLIP = range(5)
 
@@ -63,6 +63,30 @@ class Conv2d:
                                             ctypes.c_void_p(self.workspace.data_ptr()) if self.workspace is not None else None,
                                             _stream(stream), job_id, notifier), "paella_conv2d_launch")
         return y
+
+
+    def operands(self, x, residual=None, out=None):
+        p = self.plan
+        assert x.shape == (1, p.d.C, p.d.H, p.d.W), (tuple(x.shape), p.d.C, p.d.H, p.d.W)
+        y = out if out is not None else torch.empty((1, p.d.K, p.P, p.Q), device=x.device, dtype=torch.float32)
+        data = lambda t: None if t is None else _ptr(t).value
+        ops = ConvOperands(ctypes.pointer(p), data(x), self.blob.data_ptr(), data(self.bias), data(residual), data(self.slope), data(y),
+                           None if self.workspace is None else self.workspace.data_ptr())
+        return ops, y
+
+
+def conv2d_pair(first, x1, second, x2, residual1=None, residual2=None, stream=None, job_id=0, notifier=None):
+    """Two independent Conv2d layers as one launch (paella_conv2d_launch_pair); returns both outputs."""
+    a, y1 = first.operands(x1, residual1)
+    b, y2 = second.operands(x2, residual2)
+    check(first.lib.paella_conv2d_launch_pair(ctypes.byref(a), ctypes.byref(b), _stream(stream), job_id, notifier), "paella_conv2d_launch_pair")
+    return y1, y2
+
+
+def pair_dims(first, second):
+    d = LaunchDims()
+    rc = first.lib.paella_conv2d_pair_dims(ctypes.byref(first.plan), ctypes.byref(second.plan), ctypes.byref(d))
+    return rc, d
 
 
 def dense(x, w, bias=None, act=ACT_NONE, stream=None, job_id=0, notifier=None):

@@ -60,15 +60,58 @@ def test_every_intermediate_of_resnet18_matches(cuda):
         arena_in = ex.lib.paella_exec_input(ex.handle)
         base = arena_in - 4 * 0  # the input is buffer 0 at arena offset 0
         offsets = np.cumsum([0] + [((b["C"] * b["H"] * b["W"] + 63) // 64) * 64 for b in desc["buffers"]])
-        for i, node in enumerate(desc["nodes"]):
-            ex.launch_stage(i)
-            v = node["y"]
-            n = v["C"] * v["H"] * v["W"]
-            out = np.empty(n, np.float32)
-            _abi.check(_abi.hip().llis_hip_memcpy(out.ctypes.data, base + 4 * int(offsets[v["buf"]] + v["off"]), out.nbytes, 2))
-            assert_close(out, keep[i].reshape(-1), "%s stage %d (%s)" % (name, i, node["op"]))
+        i = 0
+        for stage in range(ex.num_stages):
+            ex.launch_stage(stage)
+            for _ in range(ex.stage_operators(stage)):  # a stage is one operator, or two convs in one launch
+                node = desc["nodes"][i]
+                v = node["y"]
+                n = v["C"] * v["H"] * v["W"]
+                out = np.empty(n, np.float32)
+                _abi.check(_abi.hip().llis_hip_memcpy(out.ctypes.data, base + 4 * int(offsets[v["buf"]] + v["off"]), out.nbytes, 2))
+                assert_close(out, keep[i].reshape(-1), "%s operator %d (%s)" % (name, i, node["op"]))
+                i += 1
+        assert i == len(desc["nodes"])
     finally:
         ex.close()
+
+
+@pytest.mark.parametrize("name,pairs", [("resnet18", 3), ("resnet50", None), ("inception_v3", None), ("googlenet", None), ("mnist", 0)])
+def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pairs):
+    """Two independent convs sharing a launch (a residual block's first conv and its projection, branches of an
+    inception module) against the same model built with one launch per operator.  A paired conv may run with more
+    waves per workgroup than it would alone, which changes its summation order: the outputs agree within the fp32
+    tolerance, not bit for bit (two launches with the same plans do: see the operator tests)."""
+    import os
+    from paella_amd import models
+    desc = models.describe(name)
+    x = om.make_input(desc, 17, "uniform" if name == "mnist" else "normal")
+    outs, stages = {}, {}
+    before = os.environ.get("PAELLA_CONV_PAIRS")
+    try:
+        for setting in ("0", "1"):
+            os.environ["PAELLA_CONV_PAIRS"] = setting
+            ex = models.Exec(name, seed=9)
+            try:
+                stages[setting] = [ex.stage_operators(i) for i in range(ex.num_stages)]
+                ex.set_input(x)
+                ex.forward()
+                outs[setting] = ex.get_output()
+            finally:
+                ex.close()
+    finally:
+        if before is None:
+            del os.environ["PAELLA_CONV_PAIRS"]
+        else:
+            os.environ["PAELLA_CONV_PAIRS"] = before
+    assert stages["0"] == [1] * len(desc["nodes"])
+    assert sum(stages["1"]) == len(desc["nodes"])
+    print("case", name, "pairs", stages["1"].count(2), "of", len(desc["nodes"]), "operators", flush=True)
+    if pairs is None:
+        assert stages["1"].count(2) >= 1
+    else:
+        assert stages["1"].count(2) == pairs
+    assert_close(outs["1"], outs["0"], name)
 
 
 def test_different_seeds_and_inputs_give_different_outputs(cuda):

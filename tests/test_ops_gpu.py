@@ -108,6 +108,56 @@ def test_conv2d_is_deterministic(cuda):
         assert torch.equal(conv(xd).cpu(), a)
 
 
+# (first conv, second conv): C, H, W, K, R, stride, pad, tile_hint -- both on the 32 x 32 tile with the same wave count
+PAIRS = [
+    ((64, 56, 56, 128, 3, 2, 1, 0x1113), (64, 56, 56, 128, 1, 2, 0, 0x113)),     # residual block entry and its projection: split 3x3 + tiny 1x1
+    ((256, 14, 14, 512, 3, 2, 1, 0x3113), (256, 14, 14, 512, 1, 2, 0, 0x1113)),  # both split over the reduction
+    ((192, 35, 35, 64, 1, 1, 0, 0x112), (192, 35, 35, 48, 1, 1, 0, 0x112)),      # two branches of an inception module
+    ((5, 9, 11, 7, 3, 1, 1, 0x111), (3, 13, 7, 40, 3, 1, 1, 0x111)),             # reduction order (c, r, s), different inputs
+    ((24, 20, 20, 33, 3, 1, 1, 0x110), (16, 9, 9, 70, 1, 1, 0, 0x110)),          # one wave per workgroup
+]
+
+
+@pytest.mark.parametrize("pair", PAIRS)
+def test_two_convs_in_one_launch_equal_two_launches_bit_for_bit(cuda, pair):
+    from paella_amd import ops
+    convs, xs, res, refs = [], [], [], []
+    for idx, (c, h, w, k, r, stride, pad, hint) in enumerate(pair):
+        x = rnd(1, c, h, w)
+        wt = rnd(k, c, r, r, scale=(2.0 / (c * r * r)) ** 0.5)
+        b = rnd(k, scale=0.1)
+        conv = ops.Conv2d(wt, b, stride=stride, pad=pad, act=ops.ACT_RELU if idx == 0 else ops.ACT_NONE, in_hw=(h, w),
+                          has_residual=idx == 1, tile_hint=hint)
+        assert (conv.plan.mi, conv.plan.ni, conv.plan.kw, conv.plan.splits > 1) == (1, 1, 1 << (hint & 15), (hint >> 12) > 0)
+        convs.append(conv)
+        xs.append(torch.tensor(x, device=cuda))
+        r_np = rnd(1, k, conv.plan.P, conv.plan.Q) if idx == 1 else None
+        res.append(None if r_np is None else torch.tensor(r_np, device=cuda))
+        refs.append(orc.conv2d(x, wt, b, stride=stride, pad=pad, act=orc.ACT_RELU if idx == 0 else orc.ACT_NONE, residual=r_np))
+    rc, dims = ops.pair_dims(convs[0], convs[1])
+    assert rc == 0 and dims.grid == convs[0].plan.dims.grid + convs[1].plan.dims.grid and dims.block == convs[0].plan.dims.block
+    alone = [convs[0](xs[0]).clone(), convs[1](xs[1], residual=res[1]).clone()]
+    for _ in range(2):  # the second call finds the split counters as the first left them
+        y1, y2 = ops.conv2d_pair(convs[0], xs[0], convs[1], xs[1], residual2=res[1])
+        torch.cuda.synchronize()
+        assert torch.equal(y1, alone[0]) and torch.equal(y2, alone[1])
+    close(y1, refs[0])
+    close(y2, refs[1])
+
+
+def test_pair_launch_refuses_plans_that_do_not_match(cuda):
+    from paella_amd import ops
+    a = ops.Conv2d(rnd(64, 64, 3, 3), None, pad=1, in_hw=(28, 28), tile_hint=0x113)
+    b = ops.Conv2d(rnd(64, 64, 1, 1), None, in_hw=(28, 28), tile_hint=0x112)      # other wave count
+    c = ops.Conv2d(rnd(64, 64, 3, 3), None, pad=1, in_hw=(28, 28), tile_hint=0x123)  # larger tile
+    d = ops.Conv2d(rnd(64, 3, 3, 3), None, pad=1, in_hw=(28, 28), tile_hint=0x113)   # other reduction order
+    for other in (b, c, d):
+        assert ops.pair_dims(a, other)[0] == -2
+    x = torch.zeros(1, 64, 28, 28, device=cuda)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.conv2d_pair(a, x, b, x)
+
+
 def test_conv2d_rejects_what_it_does_not_implement(cuda):
     from paella_amd import ops
     with pytest.raises(RuntimeError, match="unsupported"):
