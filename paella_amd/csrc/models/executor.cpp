@@ -12,6 +12,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <set>
 #include <string>
 #include <utility>
 #include <vector>
@@ -108,52 +109,89 @@ int log2_ceil(int v) {
     return b;
 }
 
-// Lays the nodes out as launches.  Two consecutive MFMA convs on the smallest tile go out as one launch when
-// neither reads or overwrites what the other writes and at least one of them would leave CUs idle by itself
-// (PAELLA_CONV_PAIRS=0 switches this off).  The one with fewer waves per workgroup is re-planned to the other's
+// Lays the nodes out as launches.  Two MFMA convs on the smallest tile go out as one launch when neither reads or
+// overwrites what the other writes and at least one of them would leave CUs idle by itself (PAELLA_CONV_PAIRS=0
+// switches this off, and the launches are the nodes in graph order).  Partners need not be neighbours in the graph's
+// node list: the nodes are re-issued in an order that keeps every read-after-write, write-after-read and
+// write-after-write pair of the list -- on the arena addresses, so that buffers sharing memory count -- and stays
+// as close to the list as that allows.  The conv with fewer waves per workgroup is re-planned to its partner's
 // count; its packed weights do not depend on that.
 void pair_up(paella_model* m) {
     const Graph& g = m->g;
-    const bool enabled = m->pairing;
+    const int n = (int)g.nodes.size();
     auto overlap = [&](const View& a, const View& b) {
         if (a.buf < 0 || b.buf < 0) return false;
         const size_t a0 = g.buffers[a.buf].offset + a.off, b0 = g.buffers[b.buf].offset + b.off;
         return a0 < b0 + b.numel() && b0 < a0 + a.numel();
     };
-    auto independent = [&](const Node& a, const Node& b) {
-        return !overlap(a.y, b.x) && !overlap(a.y, b.x2) && !overlap(a.y, b.y) && !overlap(b.y, a.x) && !overlap(b.y, a.x2);
+    auto ordered = [&](const Node& a, const Node& b) {  // b must stay behind a
+        return overlap(a.y, b.x) || overlap(a.y, b.x2) || overlap(a.y, b.y) || overlap(b.y, a.x) || overlap(b.y, a.x2);
     };
-    auto small_tile = [](const StagePlan& st) { return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1; };
+    auto pairable = [&](int i) {
+        const StagePlan& st = m->plans[i];
+        return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1;
+    };
+    // Both plans on one wave count; false (and nothing changed) if that is not possible.
+    auto match = [&](int i, int j, paella_launch_dims* dims) {
+        StagePlan a = m->plans[i], b = m->plans[j];
+        if (a.conv.k_order != b.conv.k_order || (a.dims.grid > 256 && b.dims.grid > 256)) return false;
+        const int kw = a.conv.kw > b.conv.kw ? a.conv.kw : b.conv.kw;
+        for (StagePlan* st : {&a, &b}) {
+            if (st->conv.kw == kw) continue;
+            const size_t blob = st->conv.blob_bytes;
+            const int hint = log2_ceil(st->conv.splits) << 12 | 1 << 8 | 1 << 4 | log2_ceil(kw);
+            if (paella_conv2d_plan(&st->node->conv, st->node->x2.buf >= 0, hint, &st->conv) != 0 || st->conv.blob_bytes != blob) return false;
+            st->dims = st->conv.dims;
+        }
+        if (paella_conv2d_pair_dims(&a.conv, &b.conv, dims) != 0) return false;
+        m->plans[i] = a;
+        m->plans[j] = b;
+        return true;
+    };
+
+    std::vector<std::vector<int>> later(n);
+    std::vector<int> waits_for(n, 0);
+    for (int i = 0; i < n; ++i)
+        for (int j = i + 1; j < n; ++j)
+            if (m->pairing ? ordered(g.nodes[i], g.nodes[j]) : j == i + 1) {
+                later[i].push_back(j);
+                ++waits_for[j];
+            }
+    std::set<int> ready;
+    for (int i = 0; i < n; ++i)
+        if (waits_for[i] == 0) ready.insert(i);
+
     m->stages.clear();
     size_t ws_first = 0, ws_second = 0;
-    for (size_t i = 0; i < g.nodes.size(); ++i) {
+    while (!ready.empty()) {
         Launch l;
-        l.first = (int)i;
-        l.dims = m->plans[i].dims;
-        if (enabled && i + 1 < g.nodes.size() && small_tile(m->plans[i]) && small_tile(m->plans[i + 1]) &&
-            m->plans[i].conv.k_order == m->plans[i + 1].conv.k_order && independent(g.nodes[i], g.nodes[i + 1]) &&
-            (m->plans[i].dims.grid <= 256 || m->plans[i + 1].dims.grid <= 256)) {
-            StagePlan a = m->plans[i], b = m->plans[i + 1];
-            const int kw = a.conv.kw > b.conv.kw ? a.conv.kw : b.conv.kw;
-            bool ok = true;
-            for (StagePlan* st : {&a, &b}) {
-                if (st->conv.kw == kw) continue;
-                const int hint = log2_ceil(st->conv.splits) << 12 | 1 << 8 | 1 << 4 | log2_ceil(kw);
-                ok = ok && paella_conv2d_plan(&st->node->conv, st->node->x2.buf >= 0, hint, &st->conv) == 0;
-                st->dims = st->conv.dims;
-            }
-            paella_launch_dims dims{};
-            if (ok && a.conv.blob_bytes == m->plans[i].conv.blob_bytes && b.conv.blob_bytes == m->plans[i + 1].conv.blob_bytes &&
-                paella_conv2d_pair_dims(&a.conv, &b.conv, &dims) == 0) {
-                m->plans[i] = a;
-                m->plans[i + 1] = b;
-                l.second = (int)i + 1;
-                l.dims = dims;
-                if (b.conv.workspace_bytes > ws_second) ws_second = b.conv.workspace_bytes;
-                ++i;
-            }
+        l.first = *ready.begin();
+        if (m->pairing && pairable(l.first)) {
+            for (int j : ready)
+                if (j != l.first && pairable(j) && match(l.first, j, &l.dims)) {
+                    l.second = j;
+                    break;
+                }
+            if (l.second < 0)  // an operator that is no such conv goes first if one is ready: it may release a partner
+                for (int j : ready)
+                    if (!pairable(j)) {
+                        l.first = j;
+                        break;
+                    }
+        }
+        if (l.second < 0) {
+            l.dims = m->plans[l.first].dims;
+        } else if (m->plans[l.second].flops / m->plans[l.second].dims.grid > m->plans[l.first].flops / m->plans[l.first].dims.grid) {
+            std::swap(l.first, l.second);  // the conv whose workgroups run longer goes first: the short ones fill in behind them
+        }
+        for (int done : {l.first, l.second}) {
+            if (done < 0) continue;
+            ready.erase(done);
+            for (int j : later[done])
+                if (--waits_for[j] == 0) ready.insert(j);
         }
         if (g.nodes[l.first].op == Op::Conv && m->plans[l.first].conv.workspace_bytes > ws_first) ws_first = m->plans[l.first].conv.workspace_bytes;
+        if (l.second >= 0 && m->plans[l.second].conv.workspace_bytes > ws_second) ws_second = m->plans[l.second].conv.workspace_bytes;
         m->stages.push_back(l);
     }
     m->ws_second = align256(ws_first);
@@ -370,9 +408,14 @@ int paella_model_stage_work(const paella_model* m, int stage, const char** op, d
     return 0;
 }
 
-int paella_model_stage_operators(const paella_model* m, int stage) {
+int paella_model_stage_nodes(const paella_model* m, int stage, int nodes[2]) {
     if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
-    return m->stages[stage].second >= 0 ? 2 : 1;
+    const Launch& l = m->stages[stage];
+    if (nodes) {
+        nodes[0] = l.first;
+        nodes[1] = l.second;
+    }
+    return l.second >= 0 ? 2 : 1;
 }
 
 int paella_exec_create(const paella_model* m, paella_exec** out) {

@@ -375,7 +375,9 @@ Graph arcfaceresnet100() {
             x = b.conv(y, planes[s], 3, stride, 1, NONE, &shortcut, nullptr, kResGain);
         }
     x = b.scale_shift(x, NONE);
-    x = b.dense(GraphBuilder::reshape(x, 512 * 7 * 7, 1, 1), 512);
+    // 49 residual units on seeded weights leave activations in the hundreds; the embedding layer brings the output back to
+    // the order of one (the trained network ends in a normalisation that does the same)
+    x = b.dense(GraphBuilder::reshape(x, 512 * 7 * 7, 1, 1), 512, NONE, 0.01);
     return b.finish(x);
 }
 

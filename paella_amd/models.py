@@ -65,8 +65,13 @@ class Exec:
         check(self.lib.paella_model_stage_dims(self.model, i, ctypes.byref(d)), "paella_model_stage_dims")
         return d
 
-    def stage_operators(self, i):
-        return self.lib.paella_model_stage_operators(self.model, i)
+    def stage_nodes(self, i):
+        """Indices of the graph nodes that stage i launches (one, or two convs sharing a launch)."""
+        nodes = (ctypes.c_int * 2)()
+        count = self.lib.paella_model_stage_nodes(self.model, i, ctypes.byref(nodes))
+        if count < 1:
+            raise RuntimeError("paella_model_stage_nodes failed: %d" % count)
+        return list(nodes)[:count]
 
     def stage_work(self, i):
         op, f, b = ctypes.c_char_p(), ctypes.c_double(), ctypes.c_double()

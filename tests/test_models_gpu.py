@@ -60,23 +60,23 @@ def test_every_intermediate_of_resnet18_matches(cuda):
         arena_in = ex.lib.paella_exec_input(ex.handle)
         base = arena_in - 4 * 0  # the input is buffer 0 at arena offset 0
         offsets = np.cumsum([0] + [((b["C"] * b["H"] * b["W"] + 63) // 64) * 64 for b in desc["buffers"]])
-        i = 0
+        seen = 0
         for stage in range(ex.num_stages):
             ex.launch_stage(stage)
-            for _ in range(ex.stage_operators(stage)):  # a stage is one operator, or two convs in one launch
+            for i in ex.stage_nodes(stage):  # a stage is one operator, or two convs in one launch
                 node = desc["nodes"][i]
                 v = node["y"]
                 n = v["C"] * v["H"] * v["W"]
                 out = np.empty(n, np.float32)
                 _abi.check(_abi.hip().llis_hip_memcpy(out.ctypes.data, base + 4 * int(offsets[v["buf"]] + v["off"]), out.nbytes, 2))
                 assert_close(out, keep[i].reshape(-1), "%s operator %d (%s)" % (name, i, node["op"]))
-                i += 1
-        assert i == len(desc["nodes"])
+                seen += 1
+        assert seen == len(desc["nodes"])
     finally:
         ex.close()
 
 
-@pytest.mark.parametrize("name,pairs", [("resnet18", 3), ("resnet50", None), ("inception_v3", None), ("googlenet", None), ("mnist", 0)])
+@pytest.mark.parametrize("name,pairs", [("resnet18", 3), ("resnet50", None), ("inception_v3", None), ("googlenet", None), ("densenet121", None), ("squeezenet1_1", None), ("ultraface320", None), ("mnist", 0)])
 def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pairs):
     """Two independent convs sharing a launch (a residual block's first conv and its projection, branches of an
     inception module) against the same model built with one launch per operator.  A paired conv may run with more
@@ -93,7 +93,7 @@ def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pai
             os.environ["PAELLA_CONV_PAIRS"] = setting
             ex = models.Exec(name, seed=9)
             try:
-                stages[setting] = [ex.stage_operators(i) for i in range(ex.num_stages)]
+                stages[setting] = [ex.stage_nodes(i) for i in range(ex.num_stages)]
                 ex.set_input(x)
                 ex.forward()
                 outs[setting] = ex.get_output()
@@ -104,13 +104,27 @@ def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pai
             del os.environ["PAELLA_CONV_PAIRS"]
         else:
             os.environ["PAELLA_CONV_PAIRS"] = before
-    assert stages["0"] == [1] * len(desc["nodes"])
-    assert sum(stages["1"]) == len(desc["nodes"])
-    print("case", name, "pairs", stages["1"].count(2), "of", len(desc["nodes"]), "operators", flush=True)
-    if pairs is None:
-        assert stages["1"].count(2) >= 1
-    else:
-        assert stages["1"].count(2) == pairs
+    assert stages["0"] == [[i] for i in range(len(desc["nodes"]))]
+    assert sorted(i for st in stages["1"] for i in st) == list(range(len(desc["nodes"])))   # every operator exactly once
+    n_pairs = sum(len(st) == 2 for st in stages["1"])
+    print("case", name, "pairs", n_pairs, "of", len(desc["nodes"]), "operators", flush=True)
+    if pairs is not None:
+        assert n_pairs == pairs
+    # Whatever the new order, an operator stays behind every earlier one it shares memory with (one of them writing).
+    stage_of = {i: k for k, st in enumerate(stages["1"]) for i in st}
+
+    def span(v):
+        return None if v["buf"] < 0 else (v["buf"], v["off"], v["off"] + v["C"] * v["H"] * v["W"])
+
+    def hit(a, b):
+        return a is not None and b is not None and a[0] == b[0] and a[1] < b[2] and b[1] < a[2]
+
+    nodes = [(span(n["x"]), span(n["x2"]), span(n["y"])) for n in desc["nodes"]]
+    for j, (xj, x2j, yj) in enumerate(nodes):
+        for i in range(j):
+            xi, x2i, yi = nodes[i]
+            if hit(yi, xj) or hit(yi, x2j) or hit(yi, yj) or hit(yj, xi) or hit(yj, x2i):
+                assert stage_of[i] < stage_of[j], (name, i, j)
     assert_close(outs["1"], outs["0"], name)
 
 

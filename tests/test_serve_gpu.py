@@ -219,6 +219,7 @@ def test_benchmark_mixes_serve_and_every_model_still_answers_correctly(cuda, mix
         for model, job, _ in types:
             desc = models.describe(model)
             x = om.make_input(desc, 41, "uniform" if model == "mnist" else "normal")
+            print("case", mix, model, flush=True)
             out, _ = serve.client_single(srv.name, serve.job_path(job), x, models.io_bytes(model)[1] // 4, n=1)
             close(out, om.run(desc, x, seed=1))
 
