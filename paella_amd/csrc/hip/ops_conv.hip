@@ -548,6 +548,11 @@ int conv_out(int in, int k, int stride, int pad, int dil) { return (in + 2 * pad
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+int env_int(const char* name, int fallback) {
+    const char* v = std::getenv(name);
+    return v && *v ? std::atoi(v) : fallback;
+}
+
 }  // namespace
 
 extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, int tile_hint, paella_conv_plan* plan) {
@@ -591,20 +596,21 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             else if (tiles(1, 2) >= target) { mi = 1; ni = 2; }
             else if (d->K > 32 && tiles(2, 1) >= target && PQ <= 32) { mi = 2; ni = 1; }
             else { mi = 1; ni = 1; }
-            kw = 8;
+            kw = env_int("PAELLA_CONV_KW", 8);
             while (kw > 1 && nchunks / kw < 4) kw >>= 1;
         }
         // Grid-level split of the reduction: layers with few output tiles (small feature maps) would otherwise
         // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU, keep >= 4 chunks per wave.
-        // (Measured alternative: about 18 chunks per wave and half as many workgroups runs 15 to 20 % faster
-        // when many kernels are in flight, but 13 to 27 % slower alone; served throughput was the same within
-        // 2 %, so the choice that is faster alone stays.)
+        // Measured on ResNet-18 with four passes in flight / one pass alone (thousand passes per second), by the cap
+        // on workgroups (PAELLA_CONV_WG_CAP) and the waves per workgroup (PAELLA_CONV_KW): 288 x 8: 15.2 / 6.9;
+        // 288 x 4: 14.5 / 6.1; 144 x 8: 13.7 / 6.1; 144 x 4: 11.9 / 5.1; 576 x 8: 13.8 / 6.0.
         const int n_tiles = tiles(mi, ni);
         int splits = 1;
         if (tile_hint > 0) {
             splits = 1 << ((tile_hint >> 12) & 0xF);
         } else {
-            while (splits < 16 && n_tiles * splits * 2 <= 288 && nchunks / (splits * 2 * kw) >= 4) splits *= 2;
+            const int cap = env_int("PAELLA_CONV_WG_CAP", 288);
+            while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= 4) splits *= 2;
         }
         int chunks_per_split = (nchunks + splits - 1) / splits;
         splits = (nchunks + chunks_per_split - 1) / chunks_per_split;  // no empty split
