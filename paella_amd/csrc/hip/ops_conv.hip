@@ -22,6 +22,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -51,6 +53,13 @@ namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Quotient by a divisor the host knows: floor(a / d) = umulhi(a, mul) + (a & one) with mul = floor(2^32 / d) + 1 and
+// one = 0, exact while a * d < 2^32 (the error term a * (mul * d - 2^32) / (d * 2^32) stays below 1 / d); d = 1 is
+// mul = 0, one = ~0.  A division costs about 25 dependent instructions per wave, and the kernel starts with six.
+struct FastDiv {
+    unsigned mul, one;
+};
+
 struct ConvArgs {
     const float* x;
     const float4* wpk;
@@ -74,7 +83,15 @@ struct ConvArgs {
     float lo, hi;
     uint32_t job_id;
     llis::job::FinishedBlockNotifier* notifier;
+    // divisors: of the work-list position (pixel tiles per slab, or slabs per pixel tile), channel tiles, output width,
+    // chunks per filter tap, filter width; fast_div = 0: operands too large for the shortcut, divide
+    FastDiv div_w, div_tm, div_q, div_cb, div_s;
+    int fast_div;
 };
+
+__device__ __forceinline__ unsigned quot(unsigned a, unsigned d, const FastDiv& f, int fast) {
+    return fast ? __umulhi(a, f.mul) + (a & f.one) : a / d;
+}
 
 __device__ __forceinline__ float apply_act(float v, int act, float slope, float lo, float hi) {
     switch (act) {
@@ -131,15 +148,15 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
         const unsigned q = total >> 3, r = total & 7u;
         const unsigned w = p.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
         if (p.slab_major) {
-            const unsigned slab = w / (unsigned)p.n_tiles_n;
+            const unsigned slab = quot(w, (unsigned)p.n_tiles_n, p.div_w, p.fast_div);
             tile_n = (int)(w - slab * (unsigned)p.n_tiles_n);
-            split = (int)(slab / (unsigned)p.n_tiles_m);
+            split = (int)quot(slab, (unsigned)p.n_tiles_m, p.div_tm, p.fast_div);
             tile_m = (int)(slab - (unsigned)split * (unsigned)p.n_tiles_m);
         } else {
             const unsigned per_n = (unsigned)(p.n_tiles_m * p.splits);
-            tile_n = (int)(w / per_n);
+            tile_n = (int)quot(w, per_n, p.div_w, p.fast_div);
             const unsigned rest = w - (unsigned)tile_n * per_n;
-            split = (int)(rest / (unsigned)p.n_tiles_m);
+            split = (int)quot(rest, (unsigned)p.n_tiles_m, p.div_tm, p.fast_div);
             tile_m = (int)(rest - (unsigned)split * (unsigned)p.n_tiles_m);
         }
     }
@@ -152,7 +169,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int pix = n0 + ni * 32 + j;
-        const int ho = pix / p.Q;
+        const int ho = (int)quot((unsigned)pix, (unsigned)p.Q, p.div_q, p.fast_div);
         const int wo = pix - ho * p.Q;
         hb[ni] = (pix < p.PQ) ? ho * p.sh - p.ph : -0x10000000;
         wb[ni] = wo * p.sw - p.pw;
@@ -183,9 +200,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
     const int kk4hw = kk * 4 * HW4;
     int st_cb = 0, st_r = 0, st_s = 0;
     if (TAP_MAJOR) {
-        const int tap = c_begin / p.CB;
+        const int tap = (int)quot((unsigned)c_begin, (unsigned)p.CB, p.div_cb, p.fast_div);
         st_cb = c_begin - tap * p.CB;
-        st_r = tap / p.S;
+        st_r = (int)quot((unsigned)tap, (unsigned)p.S, p.div_s, p.fast_div);
         st_s = tap - st_r * p.S;
     }
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
@@ -548,6 +565,11 @@ int conv_out(int in, int k, int stride, int pad, int dil) { return (in + 2 * pad
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+FastDiv fast_div(unsigned d) {
+    if (d <= 1) return FastDiv{0u, 0xFFFFFFFFu};
+    return FastDiv{(unsigned)((((uint64_t)1) << 32) / d + 1), 0u};
+}
+
 int env_int(const char* name, int fallback) {
     const char* v = std::getenv(name);
     return v && *v ? std::atoi(v) : fallback;
@@ -710,6 +732,18 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     // Weights outweigh the input: keep the workgroups that read one slab of weights on one XCD.
     a.slab_major = (double)d.K * d.C * d.R * d.S > (double)d.C * d.H * d.W ? 1 : 0;
     if (const char* force = std::getenv("PAELLA_CONV_ORDER")) a.slab_major = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : a.slab_major));
+    // Divisions by multiply-high: every dividend of the kernel is below `most`, every divisor at most `widest`.
+    const unsigned d_w = a.slab_major ? (unsigned)a.n_tiles_n : (unsigned)(a.n_tiles_m * a.splits);
+    const unsigned d_cb = a.CB > 0 ? (unsigned)a.CB : 1u;  // unused when C is no multiple of 8
+    a.div_w = fast_div(d_w);
+    a.div_tm = fast_div((unsigned)a.n_tiles_m);
+    a.div_q = fast_div((unsigned)plan->Q);
+    a.div_cb = fast_div(d_cb);
+    a.div_s = fast_div((unsigned)d.S);
+    const uint64_t total = (uint64_t)a.n_tiles_n * a.n_tiles_m * a.splits;
+    const uint64_t most = std::max<uint64_t>({total, (uint64_t)a.n_tiles_n * 32 * plan->ni, (uint64_t)a.nchunks + a.chunks_per_split});
+    const uint64_t widest = std::max<uint64_t>({d_w, (uint64_t)a.n_tiles_m, (uint64_t)plan->Q, d_cb, (uint64_t)d.S});
+    a.fast_div = (most * widest < ((uint64_t)1 << 32) && !std::getenv("PAELLA_CONV_NO_FAST_DIV")) ? 1 : 0;
     return 0;
 }
 
