@@ -70,6 +70,8 @@ typedef struct paella_conv_plan {
     int splits;                  /* workgroups per output tile that split the reduction further (grid z) */
     int m_pad, k_pad;            /* padded GEMM dims of the packed weight blob */
     int k_order;                 /* reduction order of the blob: 0 = (c, r, s), 1 = (r, s, c) (chosen when C % 8 == 0) */
+    int wg_order;                /* which workgroups share an XCD (and its L2): 1 = readers of the same weights, 0 = neighbouring pixel tiles, 2 = launch order */
+    int fast_div;                /* 1: the kernel divides by multiply-high where its operands allow (0 only for tests of the plain path) */
     size_t blob_bytes;           /* size of the packed weight blob */
     size_t workspace_bytes;      /* per-request scratch for splits > 1 (0 otherwise); must start out zeroed */
     paella_launch_dims dims;

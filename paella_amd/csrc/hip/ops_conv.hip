@@ -644,6 +644,11 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->k_pad = k_pad;
         // Reduction order: (r, s, c) when whole chunks of 8 share a filter tap, else (c, r, s) with the offset table.
         plan->k_order = (d->C % 8 == 0 && !std::getenv("PAELLA_CONV_NO_TAP_MAJOR")) ? 1 : 0;
+        // Which workgroups share an XCD.  Weights outweigh the input: those that read one slab of weights; else neighbouring pixels.
+        plan->wg_order = (double)d->K * d->C * d->R * d->S > (double)d->C * d->H * d->W ? 1 : 0;
+        if (const char* force = std::getenv("PAELLA_CONV_ORDER"))
+            plan->wg_order = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : plan->wg_order));
+        plan->fast_div = std::getenv("PAELLA_CONV_NO_FAST_DIV") ? 0 : 1;
         plan->blob_bytes = (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
         if (plan->blob_bytes >= ((size_t)1 << 31)) return PAELLA_ENOSUP;  // weights are addressed with 32-bit byte offsets
         // Workspace = fixed-size counter area (so that stages of one request, which share the workspace, never
@@ -729,9 +734,7 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     a.notifier = nf;
     a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
     a.n_tiles_m = plan->m_pad / (32 * plan->mi);
-    // Weights outweigh the input: keep the workgroups that read one slab of weights on one XCD.
-    a.slab_major = (double)d.K * d.C * d.R * d.S > (double)d.C * d.H * d.W ? 1 : 0;
-    if (const char* force = std::getenv("PAELLA_CONV_ORDER")) a.slab_major = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : a.slab_major));
+    a.slab_major = plan->wg_order;
     // Divisions by multiply-high: every dividend of the kernel is below `most`, every divisor at most `widest`.
     const unsigned d_w = a.slab_major ? (unsigned)a.n_tiles_n : (unsigned)(a.n_tiles_m * a.splits);
     const unsigned d_cb = a.CB > 0 ? (unsigned)a.CB : 1u;  // unused when C is no multiple of 8
@@ -743,7 +746,7 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     const uint64_t total = (uint64_t)a.n_tiles_n * a.n_tiles_m * a.splits;
     const uint64_t most = std::max<uint64_t>({total, (uint64_t)a.n_tiles_n * 32 * plan->ni, (uint64_t)a.nchunks + a.chunks_per_split});
     const uint64_t widest = std::max<uint64_t>({d_w, (uint64_t)a.n_tiles_m, (uint64_t)plan->Q, d_cb, (uint64_t)d.S});
-    a.fast_div = (most * widest < ((uint64_t)1 << 32) && !std::getenv("PAELLA_CONV_NO_FAST_DIV")) ? 1 : 0;
+    a.fast_div = (plan->fast_div && most * widest < ((uint64_t)1 << 32)) ? 1 : 0;
     return 0;
 }
 

@@ -161,20 +161,17 @@ def test_pair_launch_refuses_plans_that_do_not_match(cuda):
 @pytest.mark.parametrize("shape", [(64, 56, 56, 64, 3, 1, 1), (8, 9, 9, 40, 1, 1, 0), (2048, 1, 1, 1000, 1, 1, 0), (5, 9, 11, 7, 3, 1, 1),
                                    (256, 14, 14, 256, 3, 2, 1), (16, 33, 1, 24, 3, 1, 1)])
 def test_conv2d_index_arithmetic_shortcut_changes_no_bit(cuda, shape):
-    """The kernel divides by multiply-high with constants from the host; PAELLA_CONV_NO_FAST_DIV makes it divide.
+    """The kernel divides by multiply-high with constants from the host; plan.fast_div = 0 makes it divide.
     Divisors of 1 (one output column, 1x1 filters, 8 input channels, a single tile) are the special case of the shortcut."""
-    import os
     from paella_amd import ops
     c, h, w, k, r, stride, pad = shape
     x, wt, b = rnd(1, c, h, w), rnd(k, c, r, r, scale=(2.0 / (c * r * r)) ** 0.5), rnd(k, scale=0.1)
     conv = ops.Conv2d(wt, b, stride=stride, pad=pad, act=ops.ACT_RELU, in_hw=(h, w))
     xd = torch.tensor(x, device=cuda)
     fast = conv(xd).clone()
-    os.environ["PAELLA_CONV_NO_FAST_DIV"] = "1"
-    try:
-        slow = conv(xd).clone()
-    finally:
-        del os.environ["PAELLA_CONV_NO_FAST_DIV"]
+    assert conv.plan.fast_div == 1
+    conv.plan.fast_div = 0
+    slow = conv(xd).clone()
     torch.cuda.synchronize()
     assert torch.equal(fast, slow)
     close(fast, orc.conv2d(x, wt, b, stride=stride, pad=pad, act=orc.ACT_RELU))
