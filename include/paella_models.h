@@ -59,13 +59,13 @@ int paella_model_weight_values(const char* name, uint64_t seed, int tensor, floa
 /* ---- device */
 /* Returns the process-wide instance for (name, seed), building and uploading it on first use. */
 int paella_model_get(const char* name, uint64_t seed, paella_model** out);
-/* A stage is one launch: one operator of the graph, or two convs that do not depend on each other sharing a grid
- * (paella_conv2d_launch_pair).  Stages follow the graph's node order except where a conv is moved next to a
- * partner, which never reorders two nodes of which one reads or overwrites what the other writes.  With
+/* A stage is one launch: one operator of the graph, or up to four convs that do not depend on each other sharing a
+ * grid (paella_conv2d_launch_group).  Stages follow the graph's node order except where a conv is moved next to
+ * partners, which never reorders two nodes of which one reads or overwrites what the other writes.  With
  * PAELLA_CONV_PAIRS=0 in the environment when the model is built, stage i is node i. */
 int paella_model_num_stages(const paella_model* m);
-/* Number of operators of stage i (1, or 2 for a pair) and their node indices (nodes[1] = -1 for a single one). */
-int paella_model_stage_nodes(const paella_model* m, int stage, int nodes[2]);
+/* Number of operators of stage i; their node indices, in launch order, go to nodes[0 .. min(count, capacity) - 1]. */
+int paella_model_stage_nodes(const paella_model* m, int stage, int* nodes, int capacity);
 /* Launch shape of stage i in the scheduler's units (vgprs read from the loaded code object). */
 int paella_model_stage_dims(const paella_model* m, int stage, paella_launch_dims* dims);
 /* Operator name ("conv", "dwconv", "dense", "pool", "gap", "eltwise", "softmax", "lrn") and algorithmic work of stage i

@@ -113,6 +113,11 @@ typedef struct paella_conv_operands {
 } paella_conv_operands;
 
 int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_plan* second, paella_launch_dims* dims);
+/* The same for 2 to PAELLA_CONV_GROUP_MAX convs, one problem's workgroups after the other's in the order given; every
+ * pair of members must meet the conditions above. */
+#define PAELLA_CONV_GROUP_MAX 4
+int paella_conv2d_group_dims(const paella_conv_plan* const* plans, int n, paella_launch_dims* dims);
+int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void* stream, uint32_t job_id, void* notifier);
 int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second,
                               void* stream, uint32_t job_id, void* notifier);
 

@@ -34,7 +34,7 @@ int g_direct_queue_count = 0;
 namespace {
 
 constexpr uint32_t kQueuePackets = 4096;       // ring size (power of two)
-constexpr uint32_t kKernargSlotBytes = 768;    // one slot per packet index: explicit args <= 512 + implicit block 256
+constexpr uint32_t kKernargSlotBytes = 1280;   // one slot per packet index: explicit args <= 1024 + implicit block 256
 constexpr size_t kImplicitBytes = 256;
 
 struct Runtime {

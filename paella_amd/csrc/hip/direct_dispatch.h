@@ -55,7 +55,7 @@ inline void pack_args(char* buf, size_t& offset, const T& first, const Rest&... 
     pack_args(buf, offset, rest...);
 }
 
-constexpr size_t kMaxExplicitArgBytes = 512;  // largest: two conv problems in one launch
+constexpr size_t kMaxExplicitArgBytes = 1024;  // largest: four conv problems in one launch
 
 // Clock bridge for latency probes: the host's reading of the system timestamp, its frequency, and the
 // translation of a device realtime-counter value (what wall_clock64() returns in a kernel) into that domain.

@@ -472,21 +472,25 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MI
     conv_tile<MI, NI, KW, TAP_MAJOR>(p, blockIdx.x);
 }
 
-// Two independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
-// projection beside a residual block's first 3x3, the parallel branches of an inception module) share a grid, the
-// first problem's workgroups followed by the second's.  Both use the smallest tile and the same wave count; the
-// hooks see one kernel of first_grid + second grid workgroups.
-struct ConvPairArgs {
-    ConvArgs first, second;
-    unsigned first_grid;
+// Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
+// projection beside a residual block's first 3x3, the parallel branches of an inception module) share a grid, one
+// problem's workgroups after the other's.  All use the smallest tile and the same wave count; the hooks see one
+// kernel of as many workgroups as the problems have together.  A workgroup finds its problem by its id and reads
+// that problem's arguments (an index into the argument block, the same for the whole workgroup).
+constexpr int kMaxGroup = PAELLA_CONV_GROUP_MAX;
+
+struct ConvGroupArgs {
+    ConvArgs prob[kMaxGroup];
+    unsigned start[kMaxGroup];  // first workgroup id of each problem; 0xFFFFFFFF for unused entries
 };
 
 template <int KW, bool TAP_MAJOR>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_pair_kernel(ConvPairArgs g) {
-    const bool second = blockIdx.x >= g.first_grid;  // the same for the whole workgroup
-    ConvArgs p = g.first;
-    if (second) p = g.second;
-    conv_tile<1, 1, KW, TAP_MAJOR>(p, second ? blockIdx.x - g.first_grid : blockIdx.x);
+__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i)
+        if (blockIdx.x >= g.start[i]) idx = i;
+    conv_tile<1, 1, KW, TAP_MAJOR>(g.prob[idx], blockIdx.x - g.start[idx]);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -755,31 +759,38 @@ int allow_lds(const void* kern, unsigned lds_bytes) {
     return (int)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
 }
 
-typedef void (*ConvPairKernel)(ConvPairArgs);
+typedef void (*ConvGroupKernel)(ConvGroupArgs);
 
-ConvPairKernel pick_pair_kernel(int kw, int k_order) {
+ConvGroupKernel pick_group_kernel(int kw, int k_order) {
     switch (kw) {
-        case 1: return k_order ? conv_mfma_pair_kernel<1, true> : conv_mfma_pair_kernel<1, false>;
-        case 2: return k_order ? conv_mfma_pair_kernel<2, true> : conv_mfma_pair_kernel<2, false>;
-        case 4: return k_order ? conv_mfma_pair_kernel<4, true> : conv_mfma_pair_kernel<4, false>;
-        case 8: return k_order ? conv_mfma_pair_kernel<8, true> : conv_mfma_pair_kernel<8, false>;
+        case 1: return k_order ? conv_mfma_group_kernel<1, true> : conv_mfma_group_kernel<1, false>;
+        case 2: return k_order ? conv_mfma_group_kernel<2, true> : conv_mfma_group_kernel<2, false>;
+        case 4: return k_order ? conv_mfma_group_kernel<4, true> : conv_mfma_group_kernel<4, false>;
+        case 8: return k_order ? conv_mfma_group_kernel<8, true> : conv_mfma_group_kernel<8, false>;
         default: return nullptr;
     }
 }
 
 }  // namespace
 
-extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* a, const paella_conv_plan* b, paella_launch_dims* dims) {
-    if (!a || !b) return PAELLA_EINVAL;
-    if (a->kind != 0 || b->kind != 0 || a->mi != 1 || a->ni != 1 || b->mi != 1 || b->ni != 1 || a->kw != b->kw || a->k_order != b->k_order)
-        return PAELLA_ENOSUP;
+extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, int n, paella_launch_dims* dims) {
+    if (!plans || n < 2 || n > kMaxGroup) return PAELLA_EINVAL;
+    for (int i = 0; i < n; ++i) {
+        if (!plans[i]) return PAELLA_EINVAL;
+        const paella_conv_plan& p = *plans[i];
+        if (p.kind != 0 || p.mi != 1 || p.ni != 1 || p.kw != plans[0]->kw || p.k_order != plans[0]->k_order) return PAELLA_ENOSUP;
+    }
     if (dims) {
-        dims->grid = a->dims.grid + b->dims.grid;
-        dims->block = a->dims.block;
-        dims->lds_bytes = a->dims.lds_bytes > b->dims.lds_bytes ? a->dims.lds_bytes : b->dims.lds_bytes;
-        dims->vgprs = a->dims.vgprs;
+        dims->grid = 0;
+        dims->lds_bytes = 0;
+        for (int i = 0; i < n; ++i) {
+            dims->grid += plans[i]->dims.grid;
+            if (plans[i]->dims.lds_bytes > dims->lds_bytes) dims->lds_bytes = plans[i]->dims.lds_bytes;
+        }
+        dims->block = plans[0]->dims.block;
+        dims->vgprs = plans[0]->dims.vgprs;
         hipFuncAttributes attr;
-        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_pair_kernel(a->kw, a->k_order))) == hipSuccess && attr.numRegs > 0)
+        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_group_kernel(plans[0]->kw, plans[0]->k_order))) == hipSuccess && attr.numRegs > 0)
             dims->vgprs = (unsigned)attr.numRegs;
         else
             (void)hipGetLastError();
@@ -787,24 +798,40 @@ extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* a, const paella_c
     return 0;
 }
 
-extern "C" int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second, void* stream, uint32_t job_id,
-                                         void* notifier) {
-    if (!first || !second) return PAELLA_EINVAL;
+extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void* stream, uint32_t job_id, void* notifier) {
+    if (!members || n < 2 || n > kMaxGroup) return PAELLA_EINVAL;
+    const paella_conv_plan* plans[kMaxGroup];
+    for (int i = 0; i < n; ++i) plans[i] = members[i].plan;
     paella_launch_dims dims;
-    if (int rc = paella_conv2d_pair_dims(first->plan, second->plan, &dims)) return rc;
-    if (first->plan->splits > 1 && second->plan->splits > 1 && first->workspace == second->workspace) return PAELLA_EINVAL;
+    if (int rc = paella_conv2d_group_dims(plans, n, &dims)) return rc;
+    for (int i = 0; i < n; ++i)  // two split reductions must not share their counters and partial tiles
+        for (int j = i + 1; j < n; ++j)
+            if (plans[i]->splits > 1 && plans[j]->splits > 1 && members[i].workspace == members[j].workspace) return PAELLA_EINVAL;
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
-    ConvPairArgs g;
-    if (int rc = fill_args(first->plan, first->x, first->blob_dev, first->bias, first->residual, first->slope, first->y, first->workspace, job_id, nf, g.first))
-        return rc;
-    if (int rc = fill_args(second->plan, second->x, second->blob_dev, second->bias, second->residual, second->slope, second->y, second->workspace, job_id,
-                           nf, g.second))
-        return rc;
-    g.first_grid = first->plan->dims.grid;
-    ConvPairKernel kern = pick_pair_kernel(first->plan->kw, first->plan->k_order);
+    ConvGroupArgs g;
+    unsigned next = 0;
+    for (int i = 0; i < kMaxGroup; ++i) {
+        const paella_conv_operands& m = members[i < n ? i : 0];  // unused entries: a valid copy that no workgroup selects
+        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, g.prob[i])) return rc;
+        g.start[i] = i < n ? next : 0xFFFFFFFFu;
+        if (i < n) next += m.plan->dims.grid;
+    }
+    ConvGroupKernel kern = pick_group_kernel(plans[0]->kw, plans[0]->k_order);
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
     paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
     return (int)hipGetLastError();
+}
+
+extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_plan* second, paella_launch_dims* dims) {
+    const paella_conv_plan* plans[2] = {first, second};
+    return paella_conv2d_group_dims(plans, 2, dims);
+}
+
+extern "C" int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second, void* stream, uint32_t job_id,
+                                         void* notifier) {
+    if (!first || !second) return PAELLA_EINVAL;
+    const paella_conv_operands members[2] = {*first, *second};
+    return paella_conv2d_launch_group(members, 2, stream, job_id, notifier);
 }
 
 extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,

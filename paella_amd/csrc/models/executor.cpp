@@ -6,6 +6,7 @@
 #include "paella_hip.h"
 #include "paella_models.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -33,19 +34,20 @@ struct StagePlan {
     const float* shift = nullptr;
 };
 
-// One launch: an operator, or two convs that do not depend on each other sharing a grid.
+// One launch: an operator, or up to PAELLA_CONV_GROUP_MAX convs that do not depend on each other sharing a grid.
 struct Launch {
-    int first = -1, second = -1;  // node indices; second < 0: a single operator
+    int nodes[PAELLA_CONV_GROUP_MAX] = {-1, -1, -1, -1};  // node indices, in launch order
+    int count = 0;
     paella_launch_dims dims{};
 };
 
 struct paella_model {
     Graph g;
     // Split-reduction scratch of a request (stages of one request never overlap).  Every conv expects arrival
-    // counters that read zero at the head of its workspace and partial tiles behind them, so the second convs of
-    // pairs get an area of their own: a first conv's partial tiles never land on a second conv's counters.
+    // counters that read zero at the head of its workspace and partial tiles behind them, so the second to fourth
+    // convs of a group get areas of their own: no conv's partial tiles land on another's counters.
     size_t workspace_bytes = 0;
-    size_t ws_second = 0;        // byte offset of that area
+    size_t ws_area[PAELLA_CONV_GROUP_MAX] = {0, 0, 0, 0};  // byte offset of the area of the k-th conv of a launch
     uint64_t seed = 0;
     bool pairing = true;
     char* weights_dev = nullptr;
@@ -109,13 +111,13 @@ int log2_ceil(int v) {
     return b;
 }
 
-// Lays the nodes out as launches.  Two MFMA convs on the smallest tile go out as one launch when neither reads or
-// overwrites what the other writes and at least one of them would leave CUs idle by itself (PAELLA_CONV_PAIRS=0
-// switches this off, and the launches are the nodes in graph order).  Partners need not be neighbours in the graph's
-// node list: the nodes are re-issued in an order that keeps every read-after-write, write-after-read and
-// write-after-write pair of the list -- on the arena addresses, so that buffers sharing memory count -- and stays
-// as close to the list as that allows.  The conv with fewer waves per workgroup is re-planned to its partner's
-// count; its packed weights do not depend on that.
+// Lays the nodes out as launches.  MFMA convs on the smallest tile go out together, up to four in one launch, when
+// none reads or overwrites what another writes and the device is not full yet (PAELLA_CONV_PAIRS=0 switches this
+// off, and the launches are the nodes in graph order).  Partners need not be neighbours in the graph's node list: the
+// nodes are re-issued in an order that keeps every read-after-write, write-after-read and write-after-write pair of
+// the list -- on the arena addresses, so that buffers sharing memory count -- and stays as close to the list as that
+// allows.  Convs with fewer waves per workgroup are re-planned to the largest count of their group; their packed
+// weights do not depend on that.
 void pair_up(paella_model* m) {
     const Graph& g = m->g;
     const int n = (int)g.nodes.size();
@@ -131,21 +133,14 @@ void pair_up(paella_model* m) {
         const StagePlan& st = m->plans[i];
         return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1;
     };
-    // Both plans on one wave count; false (and nothing changed) if that is not possible.
-    auto match = [&](int i, int j, paella_launch_dims* dims) {
-        StagePlan a = m->plans[i], b = m->plans[j];
-        if (a.conv.k_order != b.conv.k_order || (a.dims.grid > 256 && b.dims.grid > 256)) return false;
-        const int kw = a.conv.kw > b.conv.kw ? a.conv.kw : b.conv.kw;
-        for (StagePlan* st : {&a, &b}) {
-            if (st->conv.kw == kw) continue;
-            const size_t blob = st->conv.blob_bytes;
-            const int hint = log2_ceil(st->conv.splits) << 12 | 1 << 8 | 1 << 4 | log2_ceil(kw);
-            if (paella_conv2d_plan(&st->node->conv, st->node->x2.buf >= 0, hint, &st->conv) != 0 || st->conv.blob_bytes != blob) return false;
-            st->dims = st->conv.dims;
-        }
-        if (paella_conv2d_pair_dims(&a.conv, &b.conv, dims) != 0) return false;
-        m->plans[i] = a;
-        m->plans[j] = b;
+    // The plan of node i with kw waves per workgroup; false if that is not possible.
+    auto with_waves = [&](int i, int kw, StagePlan* out) {
+        *out = m->plans[i];
+        if (out->conv.kw == kw) return true;
+        const size_t blob = out->conv.blob_bytes;
+        const int hint = log2_ceil(out->conv.splits) << 12 | 1 << 8 | 1 << 4 | log2_ceil(kw);
+        if (paella_conv2d_plan(&out->node->conv, out->node->x2.buf >= 0, hint, &out->conv) != 0 || out->conv.blob_bytes != blob) return false;
+        out->dims = out->conv.dims;
         return true;
     };
 
@@ -157,45 +152,80 @@ void pair_up(paella_model* m) {
                 later[i].push_back(j);
                 ++waits_for[j];
             }
-    std::set<int> ready;
+    std::set<int> ready;  // no two ready nodes are ordered with respect to each other
     for (int i = 0; i < n; ++i)
         if (waits_for[i] == 0) ready.insert(i);
 
     m->stages.clear();
-    size_t ws_first = 0, ws_second = 0;
+    size_t area[PAELLA_CONV_GROUP_MAX] = {0, 0, 0, 0};
     while (!ready.empty()) {
         Launch l;
-        l.first = *ready.begin();
-        if (m->pairing && pairable(l.first)) {
-            for (int j : ready)
-                if (j != l.first && pairable(j) && match(l.first, j, &l.dims)) {
-                    l.second = j;
-                    break;
+        l.nodes[0] = *ready.begin();
+        l.count = 1;
+        if (m->pairing && pairable(l.nodes[0])) {
+            // Candidates: ready convs of the same reduction order, taken while the launch leaves CUs idle or the newcomer is small.
+            unsigned grid = m->plans[l.nodes[0]].dims.grid;
+            int kw = m->plans[l.nodes[0]].conv.kw;
+            for (int j : ready) {
+                if (l.count == PAELLA_CONV_GROUP_MAX) break;
+                if (j == l.nodes[0] || !pairable(j) || m->plans[j].conv.k_order != m->plans[l.nodes[0]].conv.k_order) continue;
+                const unsigned gj = m->plans[j].dims.grid;
+                if ((grid > 256 && gj > 256) || grid + gj > 1024) continue;
+                l.nodes[l.count++] = j;
+                grid += gj;
+                if (m->plans[j].conv.kw > kw) kw = m->plans[j].conv.kw;
+            }
+            if (l.count > 1) {
+                StagePlan re[PAELLA_CONV_GROUP_MAX];
+                const paella_conv_plan* plans[PAELLA_CONV_GROUP_MAX];
+                int kept = 0;
+                for (int k = 0; k < l.count; ++k)
+                    if (with_waves(l.nodes[k], kw, &re[kept])) {
+                        l.nodes[kept] = l.nodes[k];
+                        plans[kept] = &re[kept].conv;
+                        ++kept;
+                    } else if (k == 0) {
+                        kept = 0;
+                        break;
+                    }
+                if (kept > 1 && paella_conv2d_group_dims(plans, kept, &l.dims) == 0) {
+                    for (int k = 0; k < kept; ++k) m->plans[l.nodes[k]] = re[k];
+                    l.count = kept;
+                } else {
+                    l.nodes[0] = *ready.begin();
+                    l.count = 1;
                 }
-            if (l.second < 0)  // an operator that is no such conv goes first if one is ready: it may release a partner
+                for (int k = l.count; k < PAELLA_CONV_GROUP_MAX; ++k) l.nodes[k] = -1;
+            }
+            if (l.count == 1)  // an operator that is no such conv goes first if one is ready: it may release a partner
                 for (int j : ready)
                     if (!pairable(j)) {
-                        l.first = j;
+                        l.nodes[0] = j;
                         break;
                     }
         }
-        if (l.second < 0) {
-            l.dims = m->plans[l.first].dims;
-        } else if (m->plans[l.second].flops / m->plans[l.second].dims.grid > m->plans[l.first].flops / m->plans[l.first].dims.grid) {
-            std::swap(l.first, l.second);  // the conv whose workgroups run longer goes first: the short ones fill in behind them
+        if (l.count == 1) {
+            l.dims = m->plans[l.nodes[0]].dims;
+        } else {
+            // the convs whose workgroups run longer go first: the short ones fill in behind them
+            std::stable_sort(l.nodes, l.nodes + l.count, [&](int a, int b) {
+                return m->plans[a].flops / m->plans[a].dims.grid > m->plans[b].flops / m->plans[b].dims.grid;
+            });
         }
-        for (int done : {l.first, l.second}) {
-            if (done < 0) continue;
+        for (int k = 0; k < l.count; ++k) {
+            const int done = l.nodes[k];
             ready.erase(done);
             for (int j : later[done])
                 if (--waits_for[j] == 0) ready.insert(j);
+            if (g.nodes[done].op == Op::Conv && m->plans[done].conv.workspace_bytes > area[k]) area[k] = m->plans[done].conv.workspace_bytes;
         }
-        if (g.nodes[l.first].op == Op::Conv && m->plans[l.first].conv.workspace_bytes > ws_first) ws_first = m->plans[l.first].conv.workspace_bytes;
-        if (l.second >= 0 && m->plans[l.second].conv.workspace_bytes > ws_second) ws_second = m->plans[l.second].conv.workspace_bytes;
         m->stages.push_back(l);
     }
-    m->ws_second = align256(ws_first);
-    m->workspace_bytes = ws_second ? m->ws_second + ws_second : ws_first;
+    m->workspace_bytes = 0;
+    for (int k = 0; k < PAELLA_CONV_GROUP_MAX; ++k) {
+        m->ws_area[k] = m->workspace_bytes;
+        m->workspace_bytes += align256(area[k]);
+    }
 }
 
 int build(paella_model* m) {
@@ -400,22 +430,22 @@ int paella_model_stage_dims(const paella_model* m, int stage, paella_launch_dims
 int paella_model_stage_work(const paella_model* m, int stage, const char** op, double* flops, double* bytes) {
     if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
     const Launch& l = m->stages[stage];
-    const StagePlan& a = m->plans[l.first];
-    const StagePlan* b = l.second >= 0 ? &m->plans[l.second] : nullptr;
-    if (op) *op = a.op;
-    if (flops) *flops = a.flops + (b ? b->flops : 0);
-    if (bytes) *bytes = a.bytes + (b ? b->bytes : 0);
+    if (op) *op = m->plans[l.nodes[0]].op;
+    double f = 0, b = 0;
+    for (int k = 0; k < l.count; ++k) {
+        f += m->plans[l.nodes[k]].flops;
+        b += m->plans[l.nodes[k]].bytes;
+    }
+    if (flops) *flops = f;
+    if (bytes) *bytes = b;
     return 0;
 }
 
-int paella_model_stage_nodes(const paella_model* m, int stage, int nodes[2]) {
-    if (!m || stage < 0 || (size_t)stage >= m->stages.size()) return PAELLA_EINVAL;
+int paella_model_stage_nodes(const paella_model* m, int stage, int* nodes, int capacity) {
+    if (!m || stage < 0 || (size_t)stage >= m->stages.size() || capacity < 0) return PAELLA_EINVAL;
     const Launch& l = m->stages[stage];
-    if (nodes) {
-        nodes[0] = l.first;
-        nodes[1] = l.second;
-    }
-    return l.second >= 0 ? 2 : 1;
+    for (int k = 0; nodes && k < l.count && k < capacity; ++k) nodes[k] = l.nodes[k];
+    return l.count;
 }
 
 int paella_exec_create(const paella_model* m, paella_exec** out) {
@@ -473,16 +503,18 @@ void* paella_exec_output(paella_exec* e) { return e ? e->ptr(e->m->g.output) : n
 int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier) {
     if (!e || stage < 0 || (size_t)stage >= e->m->stages.size()) return PAELLA_EINVAL;
     const Launch& l = e->m->stages[stage];
-    const StagePlan& st = e->m->plans[l.first];
-    const Node& n = *st.node;
-    if (l.second >= 0) {
-        const StagePlan& st2 = e->m->plans[l.second];
-        const Node& n2 = *st2.node;
-        const paella_conv_operands a{&st.conv, e->ptr(n.x), st.w, st.bias, e->ptr(n.x2), st.slope, e->ptr(n.y), e->workspace};
-        const paella_conv_operands b{&st2.conv, e->ptr(n2.x), st2.w, st2.bias, e->ptr(n2.x2), st2.slope, e->ptr(n2.y),
-                                     e->workspace ? static_cast<char*>(e->workspace) + e->m->ws_second : nullptr};
-        return paella_conv2d_launch_pair(&a, &b, stream, job_id, notifier);
+    if (l.count > 1) {
+        paella_conv_operands members[PAELLA_CONV_GROUP_MAX];
+        for (int k = 0; k < l.count; ++k) {
+            const StagePlan& sk = e->m->plans[l.nodes[k]];
+            const Node& nk = *sk.node;
+            members[k] = paella_conv_operands{&sk.conv, e->ptr(nk.x), sk.w, sk.bias, e->ptr(nk.x2), sk.slope, e->ptr(nk.y),
+                                              e->workspace ? static_cast<char*>(e->workspace) + e->m->ws_area[k] : nullptr};
+        }
+        return paella_conv2d_launch_group(members, l.count, stream, job_id, notifier);
     }
+    const StagePlan& st = e->m->plans[l.nodes[0]];
+    const Node& n = *st.node;
     const float* x = e->ptr(n.x);
     const float* x2 = e->ptr(n.x2);
     float* y = e->ptr(n.y);

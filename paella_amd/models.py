@@ -66,9 +66,9 @@ class Exec:
         return d
 
     def stage_nodes(self, i):
-        """Indices of the graph nodes that stage i launches (one, or two convs sharing a launch)."""
-        nodes = (ctypes.c_int * 2)()
-        count = self.lib.paella_model_stage_nodes(self.model, i, ctypes.byref(nodes))
+        """Indices of the graph nodes that stage i launches (one operator, or several convs sharing a launch)."""
+        nodes = (ctypes.c_int * 8)()
+        count = self.lib.paella_model_stage_nodes(self.model, i, nodes, 8)
         if count < 1:
             raise RuntimeError("paella_model_stage_nodes failed: %d" % count)
         return list(nodes)[:count]

@@ -83,6 +83,18 @@ def conv2d_pair(first, x1, second, x2, residual1=None, residual2=None, stream=No
     return y1, y2
 
 
+def conv2d_group(convs, xs, residuals=None, stream=None, job_id=0, notifier=None):
+    """Up to four independent Conv2d layers as one launch (paella_conv2d_launch_group); returns their outputs."""
+    residuals = residuals or [None] * len(convs)
+    members = (ConvOperands * len(convs))()
+    outs = []
+    for k, (c, x, r) in enumerate(zip(convs, xs, residuals)):
+        members[k], y = c.operands(x, r)
+        outs.append(y)
+    check(convs[0].lib.paella_conv2d_launch_group(members, len(convs), _stream(stream), job_id, notifier), "paella_conv2d_launch_group")
+    return outs
+
+
 def pair_dims(first, second):
     d = LaunchDims()
     rc = first.lib.paella_conv2d_pair_dims(ctypes.byref(first.plan), ctypes.byref(second.plan), ctypes.byref(d))

@@ -78,7 +78,7 @@ def test_every_intermediate_of_resnet18_matches(cuda):
 
 @pytest.mark.parametrize("name,pairs", [("resnet18", 3), ("resnet50", None), ("inception_v3", None), ("googlenet", None), ("densenet121", None), ("squeezenet1_1", None), ("ultraface320", None), ("mnist", 0)])
 def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pairs):
-    """Two independent convs sharing a launch (a residual block's first conv and its projection, branches of an
+    """Independent convs sharing a launch (a residual block's first conv and its projection, up to four branches of an
     inception module) against the same model built with one launch per operator.  A paired conv may run with more
     waves per workgroup than it would alone, which changes its summation order: the outputs agree within the fp32
     tolerance, not bit for bit (two launches with the same plans do: see the operator tests)."""
@@ -106,8 +106,9 @@ def test_paired_convs_change_the_launch_count_and_not_the_output(cuda, name, pai
             os.environ["PAELLA_CONV_PAIRS"] = before
     assert stages["0"] == [[i] for i in range(len(desc["nodes"]))]
     assert sorted(i for st in stages["1"] for i in st) == list(range(len(desc["nodes"])))   # every operator exactly once
-    n_pairs = sum(len(st) == 2 for st in stages["1"])
-    print("case", name, "pairs", n_pairs, "of", len(desc["nodes"]), "operators", flush=True)
+    n_pairs = sum(len(st) >= 2 for st in stages["1"])
+    assert max(len(st) for st in stages["1"]) <= 4
+    print("case", name, len(desc["nodes"]), "operators in", len(stages["1"]), "launches,", n_pairs, "of them shared", flush=True)
     if pairs is not None:
         assert n_pairs == pairs
     # Whatever the new order, an operator stays behind every earlier one it shares memory with (one of them writing).

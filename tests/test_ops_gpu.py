@@ -145,6 +145,28 @@ def test_two_convs_in_one_launch_equal_two_launches_bit_for_bit(cuda, pair):
     close(y2, refs[1])
 
 
+@pytest.mark.parametrize("count", [3, 4])
+def test_group_of_convs_in_one_launch_equals_separate_launches_bit_for_bit(cuda, count):
+    """Branches of an inception module: 1x1, 1x1 ahead of a 5x5, 1x1 ahead of a 3x3, 1x1 behind a pool, one of them split
+    over the reduction; every member on its own workspace."""
+    from paella_amd import ops
+    shapes = [(192, 35, 35, 64, 1, 0, 0x113), (192, 35, 35, 48, 1, 0, 0x1113), (96, 35, 35, 96, 3, 1, 0x113), (192, 35, 35, 32, 1, 0, 0x113)][:count]
+    convs, xs, alone, refs = [], [], [], []
+    for c, h, w, k, r, pad, hint in shapes:
+        x, wt, b = rnd(1, c, h, w), rnd(k, c, r, r, scale=(2.0 / (c * r * r)) ** 0.5), rnd(k, scale=0.1)
+        conv = ops.Conv2d(wt, b, pad=pad, act=ops.ACT_RELU, in_hw=(h, w), tile_hint=hint)
+        convs.append(conv)
+        xs.append(torch.tensor(x, device=cuda))
+        alone.append(conv(xs[-1]).clone())
+        refs.append(orc.conv2d(x, wt, b, pad=pad, act=orc.ACT_RELU))
+    for _ in range(2):
+        outs = ops.conv2d_group(convs, xs)
+        torch.cuda.synchronize()
+        for got, want, ref in zip(outs, alone, refs):
+            assert torch.equal(got, want)
+            close(got, ref)
+
+
 def test_pair_launch_refuses_plans_that_do_not_match(cuda):
     from paella_amd import ops
     a = ops.Conv2d(rnd(64, 64, 3, 3), None, pad=1, in_hw=(28, 28), tile_hint=0x113)
