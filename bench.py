@@ -384,7 +384,7 @@ def main():
     log("[bench] per-launch timing of the forward pass (kernel begin/end timestamps through HIP events), taken before the serving arms")
     achieved = rl["conv_flops"] / (rl["conv_us"] * 1e-6) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-                "traffic": CONV_TRAFFIC_BYTES_PER_LAUNCH.get(args.model), "kernel": "conv_mfma_kernel and conv_mfma_pair_kernel (all %d conv launches of one %s forward pass)" % (rl["conv_launches"], args.model),
+                "traffic": CONV_TRAFFIC_BYTES_PER_LAUNCH.get(args.model), "kernel": "conv_mfma_kernel and conv_mfma_group_kernel (all %d conv launches of one %s forward pass)" % (rl["conv_launches"], args.model),
                 "flops_per_launch_avg": rl["conv_flops"] / rl["conv_launches"], "us_per_launch_avg": rl["conv_us"] / rl["conv_launches"]}
     log("[bench]   conv: %.2f TFLOP/s (%.1f%% of fp32 MFMA peak), forward %.0f us, direct loop %.0f req/s" %
         (achieved, 100 * roofline["frac"], rl["forward_us"], rl["direct_rps"]))
