@@ -480,7 +480,8 @@ def main():
         "config": {"workload": "%s batch 1 fp32 %s, seeded weights, inputs resident in device memory, full3 scheduler, %d streams, "
                                "saturation with %d outstanding requests" % (args.model, in_shape, args.num_streams, args.concurrency),
                    # kernels only: the input is resident and an output of at most 64 KiB is written to host memory by the last kernel
-                   "gmac_per_request": tot["macs"] / 1e9, "stages_per_request": tot["stages"] + (0 if models.io_bytes(args.model)[1] <= 65536 else 1)},
+                   "gmac_per_request": tot["macs"] / 1e9, "operators_per_request": tot["stages"],
+                   "stages_per_request": (len(rl["per_stage_us"]) if rl else tot["stages"]) + (0 if models.io_bytes(args.model)[1] <= 65536 else 1)},
         "pcie_inclusive_requests_per_s": pcie_inclusive,
         # open-loop latency at 80 % of the saturation rate; at saturation every request is submitted at t = 0 and
         # its latency is its position in the queue, so no latency is quoted for the timed arm itself
