@@ -36,7 +36,7 @@ def log(*a):
 # HBM-side bytes per conv launch (mean over the conv launches of one forward pass), from the FETCH_SIZE / WRITE_SIZE
 # counter passes of `bench.py --roofline-only` scaled by the copy-kernel calibration (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0);
 # counters cannot be collected from inside this process, so the figure is carried here and is null for other models.
-CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 7.11e6}  # 17 launches: 20 convs, 3 of them sharing a launch with another
+CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 7.10e6}  # 17 launches: 20 convs, 3 of them sharing a launch with another
 
 
 def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2, unfair=1e6):
