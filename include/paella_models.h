@@ -53,6 +53,10 @@ int paella_model_write_dim(const char* name, const char* path);
 int paella_model_describe(const char* name, char* json, size_t cap, size_t* needed);
 /* Algorithmic totals of one forward pass. */
 int paella_model_totals(const char* name, double* macs, double* params, double* flops, double* bytes, int* stages);
+/* The launches a model is executed as (see paella_model_num_stages below), computed on the host without a device:
+ * for every launch its number of operators followed by their node indices.  Returns the number of ints the list
+ * takes (written up to `capacity`), negative on error. */
+int paella_model_launch_plan(const char* name, int* out, size_t capacity);
 /* Fills out[i] with element i of weight tensor `tensor` of the model under `seed` (host memory). */
 int paella_model_weight_values(const char* name, uint64_t seed, int tensor, float* out, size_t count);
 

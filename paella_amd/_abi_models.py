@@ -14,6 +14,7 @@ MODEL_SYMBOLS = {
     "paella_model_totals": (c_int, [c_char_p, _pd, _pd, _pd, _pd, ctypes.POINTER(c_int)]),
     "paella_model_weight_values": (c_int, [c_char_p, c_u64, c_int, c_void_p, c_size_t]),
     "paella_model_get": (c_int, [c_char_p, c_u64, ctypes.POINTER(c_void_p)]),
+    "paella_model_launch_plan": (c_int, [ctypes.c_char_p, ctypes.POINTER(c_int), ctypes.c_size_t]),
     "paella_model_num_stages": (c_int, [c_void_p]),
     "paella_model_stage_nodes": (c_int, [c_void_p, c_int, ctypes.POINTER(c_int), c_int]),
     "paella_model_stage_dims": (c_int, [c_void_p, c_int, ctypes.POINTER(LaunchDims)]),

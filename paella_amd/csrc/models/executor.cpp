@@ -228,12 +228,12 @@ void pair_up(paella_model* m) {
     }
 }
 
-int build(paella_model* m) {
+// Plans every node and lays out the weight arena (host arithmetic only).
+int plan_nodes(paella_model* m, std::vector<size_t>& tensor_off, std::vector<size_t>& blob_off, size_t& total) {
     const Graph& g = m->g;
-    // Pass 1: plan every node and lay out the weight arena.
-    std::vector<size_t> tensor_off(g.weights.size(), (size_t)-1);
-    std::vector<size_t> blob_off(g.nodes.size(), (size_t)-1);
-    size_t total = 0;
+    tensor_off.assign(g.weights.size(), (size_t)-1);
+    blob_off.assign(g.nodes.size(), (size_t)-1);
+    total = 0;
     m->plans.resize(g.nodes.size());
     for (size_t i = 0; i < g.nodes.size(); ++i) {
         const Node& n = g.nodes[i];
@@ -302,9 +302,17 @@ int build(paella_model* m) {
         }
     }
 
+    return 0;
+}
+
+int build(paella_model* m) {
+    const Graph& g = m->g;
+    std::vector<size_t> tensor_off, blob_off;
+    size_t total = 0;
+    if (int rc = plan_nodes(m, tensor_off, blob_off, total)) return rc;
     pair_up(m);
 
-    // Pass 2: generate, pack, upload.
+    // Generate, pack, upload.
     std::vector<char> host(total, 0);
     std::vector<float> tmp;
     for (size_t t = 0; t < g.weights.size(); ++t) {
@@ -391,6 +399,26 @@ int paella_model_totals(const char* name, double* macs, double* params, double* 
     }
     if (stages) *stages = (int)g->nodes.size();
     return 0;
+}
+
+int paella_model_launch_plan(const char* name, int* out, size_t capacity) {
+    const Graph* g = graph_of(name);
+    if (!g) return PAELLA_EINVAL;
+    paella_model m;
+    m.g = *g;
+    m.pairing = pairing_enabled();
+    std::vector<size_t> tensor_off, blob_off;
+    size_t total = 0;
+    if (int rc = plan_nodes(&m, tensor_off, blob_off, total)) return rc;
+    pair_up(&m);
+    size_t used = 0;
+    for (const Launch& l : m.stages) {
+        if (out && used < capacity) out[used] = l.count;
+        ++used;
+        for (int k = 0; k < l.count; ++k, ++used)
+            if (out && used < capacity) out[used] = l.nodes[k];
+    }
+    return (int)used;
 }
 
 int paella_model_weight_values(const char* name, uint64_t seed, int tensor, float* out, size_t count) {

@@ -29,6 +29,21 @@ def totals(name):
     return {"macs": m.value, "params": p.value, "flops": f.value, "bytes": b.value, "stages": s.value}
 
 
+def launch_plan(name):
+    """The launches of a model as lists of node indices (host arithmetic only, no device needed)."""
+    lib = _abi.ops()
+    need = lib.paella_model_launch_plan(name.encode(), None, 0)
+    if need < 0:
+        raise RuntimeError("paella_model_launch_plan failed: %d" % need)
+    buf = (ctypes.c_int * need)()
+    lib.paella_model_launch_plan(name.encode(), buf, need)
+    out, i = [], 0
+    while i < need:
+        out.append(list(buf[i + 1:i + 1 + buf[i]]))
+        i += 1 + buf[i]
+    return out
+
+
 def io_bytes(name):
     lib = _abi.ops()
     i, o = ctypes.c_size_t(), ctypes.c_size_t()

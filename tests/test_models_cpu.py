@@ -355,3 +355,50 @@ def test_io_shapes_match_the_reference_dim_sidecars(tmp_path):
         cut = vals.index(-1)
         assert vals[:cut] == want_in
         assert int(np.prod(vals[cut + 1:])) == int(np.prod(dims["output"])) and vals[cut + 1:cut + 3] == dims["output"][:2]
+
+
+ZOO = ["mnist", "resnet18", "resnet34", "resnet50", "mobilenetv2", "inception_v3", "squeezenet1_1", "googlenet", "densenet121",
+       "ultraface320", "arcfaceresnet100"]
+
+
+@pytest.mark.parametrize("name", ZOO)
+def test_launch_plan_keeps_every_dependence_of_the_graph(name):
+    """The executor launches independent convs together and re-issues nodes to bring partners side by side.  Whatever
+    the order, every operator appears exactly once, a launch holds at most four of them and only convs when it holds
+    several, and an operator stays behind every earlier one it shares memory with when one of the two writes it."""
+    import os
+    from paella_amd import models
+    desc = models.describe(name)
+    nodes = desc["nodes"]
+    before = os.environ.get("PAELLA_CONV_PAIRS")
+    try:
+        os.environ["PAELLA_CONV_PAIRS"] = "0"
+        assert models.launch_plan(name) == [[i] for i in range(len(nodes))]
+        os.environ["PAELLA_CONV_PAIRS"] = "1"
+        plan = models.launch_plan(name)
+    finally:
+        if before is None:
+            del os.environ["PAELLA_CONV_PAIRS"]
+        else:
+            os.environ["PAELLA_CONV_PAIRS"] = before
+    assert sorted(i for launch in plan for i in launch) == list(range(len(nodes)))
+    assert all(1 <= len(launch) <= 4 for launch in plan)
+    assert all(nodes[i]["op"] == "conv" and nodes[i]["groups"] == 1 for launch in plan if len(launch) > 1 for i in launch)
+    stage_of = {i: k for k, launch in enumerate(plan) for i in launch}
+
+    def span(v):
+        return None if v["buf"] < 0 else (v["buf"], v["off"], v["off"] + v["C"] * v["H"] * v["W"])
+
+    def hit(a, b):
+        return a is not None and b is not None and a[0] == b[0] and a[1] < b[2] and b[1] < a[2]
+
+    spans = [(span(n["x"]), span(n["x2"]), span(n["y"])) for n in nodes]
+    for j, (xj, x2j, yj) in enumerate(spans):
+        for i in range(j):
+            xi, x2i, yi = spans[i]
+            if hit(yi, xj) or hit(yi, x2j) or hit(yi, yj) or hit(yj, xi) or hit(yj, x2i):
+                assert stage_of[i] < stage_of[j], (name, i, j)
+    if name == "resnet18":
+        assert [launch for launch in plan if len(launch) > 1] == [[7, 6], [12, 11], [17, 16]]  # first 3x3 of the block, then its projection
+    if name in ("inception_v3", "googlenet"):
+        assert max(len(launch) for launch in plan) >= 3 and len(plan) < 0.7 * len(nodes)
