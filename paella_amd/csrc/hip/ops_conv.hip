@@ -624,6 +624,9 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             if (tiles(1, 1) <= 2048) { mi = 1; ni = 1; }
             else if (tiles(1, 2) <= 2048 || d->K <= 32) { mi = 1; ni = 2; }
             else { mi = 2; ni = 2; }
+            // The same holds with four passes in flight, where throughput rather than latency might have favoured operand
+            // reuse (ResNet-18, thousand passes per second, four queues / one): 32 x 32 everywhere 15.8 / 7.0; 64 x 32 where
+            // K is a multiple of 64: 12.1 / 4.9, only from K = 256: 13.2 / 5.6; 32 x 64 on the 56 x 56 layers: 14.4 / 6.4.
             // (at most 4 where the reduction goes through the offset table -- stems: 7.8 against 7.9 us, 4.4 against 4.7)
             const int kw_max = d->C % 8 == 0 ? env_int("PAELLA_CONV_KW", 8) : 4;
             kw = 2;

@@ -66,6 +66,62 @@ __global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x,
     paella::hook_exit(notifier, job_id);
 }
 
+// Long rows (I >= kDenseLongRow, a multiple of 4): with one wave per row a layer of few, long rows (an embedding
+// head: 512 rows of 100 KB) occupies half the SIMDs with one load in flight each.  Here a workgroup of eight
+// waves owns two rows; each wave takes an eighth of both rows, keeps eight weight loads in flight per lane and
+// uses every x value for both rows; the partial sums meet in LDS and are added in wave order (deterministic).
+constexpr int kDenseLongRow = 8192;
+
+__global__ __launch_bounds__(512) void dense_long_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                         const float* __restrict__ bias, float* __restrict__ y, int I, int O,
+                                                         int act, uint32_t job_id, Notifier* notifier) {
+    paella::hook_entry(notifier, job_id);
+    __shared__ float part[2][8];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int o0 = blockIdx.x * 2;
+    const int o1 = min(o0 + 1, O - 1);  // an odd O: the last workgroup reads its only row twice and stores it once
+    const int I4 = I >> 2;
+    const int per = (I4 + 7) >> 3;
+    const int begin = wave * per;
+    const int end = min(I4, begin + per);
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const float4* wa = reinterpret_cast<const float4*>(w + (size_t)o0 * I);
+    const float4* wb = reinterpret_cast<const float4*>(w + (size_t)o1 * I);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f, b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+    auto dot = [](const float4& p, const float4& q) { return p.x * q.x + p.y * q.y + p.z * q.z + p.w * q.w; };
+    int i = begin + lane;
+    for (; i + 192 < end; i += 256) {
+        const float4 p0 = wa[i], p1 = wa[i + 64], p2 = wa[i + 128], p3 = wa[i + 192];
+        const float4 q0 = wb[i], q1 = wb[i + 64], q2 = wb[i + 128], q3 = wb[i + 192];
+        const float4 v0 = x4[i], v1 = x4[i + 64], v2 = x4[i + 128], v3 = x4[i + 192];
+        a0 += dot(p0, v0); a1 += dot(p1, v1); a2 += dot(p2, v2); a3 += dot(p3, v3);
+        b0 += dot(q0, v0); b1 += dot(q1, v1); b2 += dot(q2, v2); b3 += dot(q3, v3);
+    }
+    for (; i < end; i += 64) {
+        const float4 v = x4[i];
+        a0 += dot(wa[i], v);
+        b0 += dot(wb[i], v);
+    }
+    const float sa = wave_sum((a0 + a1) + (a2 + a3));
+    const float sb = wave_sum((b0 + b1) + (b2 + b3));
+    if (lane == 0) {
+        part[0][wave] = sa;
+        part[1][wave] = sb;
+    }
+    __syncthreads();
+    if (threadIdx.x < 2) {
+        const int o = o0 + (int)threadIdx.x;
+        if (o < O) {
+            float v = 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v += part[threadIdx.x][k];
+            store_out(y + o, act_apply(v + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f));
+        }
+    }
+    paella::hook_exit(notifier, job_id);
+}
+
 // ------------------------------------------------------------------------------------------ pooling
 struct PoolArgs {
     const float* x;
@@ -274,16 +330,23 @@ int paella_pool_out(int in, int k, int stride, int pad, int ceil_mode) {
     return out;
 }
 
+static bool dense_long(int I) { return I >= kDenseLongRow && (I & 3) == 0; }
+
 int paella_dense_dims(int I, int O, paella_launch_dims* dims) {
     if (I <= 0 || O <= 0 || !dims) return PAELLA_EINVAL;
-    set_dims(dims, blocks_for(O, 4), 256, 0, 32);
+    if (dense_long(I)) set_dims(dims, blocks_for(O, 2), 512, 64, 48);
+    else set_dims(dims, blocks_for(O, 4), 256, 0, 32);
     return 0;
 }
 
 int paella_dense_launch(const float* x, const float* w, const float* bias, float* y, int I, int O, int act, void* stream,
                         uint32_t job_id, void* notifier) {
     if (!x || !w || !y || I <= 0 || O <= 0 || act < 0 || act > PAELLA_ACT_RELU6) return PAELLA_EINVAL;
-    paella::launch(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
+    if (dense_long(I))
+        paella::launch(dense_long_kernel, dim3(blocks_for(O, 2)), dim3(512), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
+                       (Notifier*)notifier);
+    else
+        paella::launch(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
                        (Notifier*)notifier);
     return (int)hipGetLastError();
 }

@@ -218,7 +218,8 @@ def test_depthwise_conv_parity(cuda, c, h, w, r, stride, pad):
     close(conv(torch.tensor(x, device=cuda)), ref)
 
 
-@pytest.mark.parametrize("i,o", [(256, 10), (512, 1000), (2048, 1000), (1280, 1000), (25088, 512), (37, 11)])
+@pytest.mark.parametrize("i,o", [(256, 10), (512, 1000), (2048, 1000), (1280, 1000), (25088, 512), (37, 11), (25088, 511), (8192, 3), (8196, 5), (9001, 4),
+                                 (16388, 1)])
 def test_dense_parity(cuda, i, o):
     from paella_amd import ops
     x, w, b = rnd(1, i), rnd(o, i, scale=i ** -0.5), rnd(o)
