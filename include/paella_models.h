@@ -63,8 +63,10 @@ int paella_model_weight_values(const char* name, uint64_t seed, int tensor, floa
 /* ---- device */
 /* Returns the process-wide instance for (name, seed), building and uploading it on first use. */
 int paella_model_get(const char* name, uint64_t seed, paella_model** out);
-/* A stage is one launch: one operator of the graph, or up to four convs that do not depend on each other sharing a
- * grid (paella_conv2d_launch_group).  Stages follow the graph's node order except where a conv is moved next to
+/* A stage is one launch: one operator of the graph, up to four convs that do not depend on each other sharing a
+ * grid (paella_conv2d_launch_group), or a per-channel scale-shift operator followed by the conv that applies it to
+ * its own input (paella_conv2d_launch_transformed; when several convs read the scale-shift result, it is listed with
+ * the first of them and the others apply it as well; its own output is never written).  Stages follow the graph's node order except where a conv is moved next to
  * partners, which never reorders two nodes of which one reads or overwrites what the other writes.  With
  * PAELLA_CONV_PAIRS=0 in the environment when the model is built, stage i is node i. */
 int paella_model_num_stages(const paella_model* m);

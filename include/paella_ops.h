@@ -93,6 +93,20 @@ int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const voi
                          const float* residual, const float* slope, float* y, void* workspace,
                          void* stream, uint32_t job_id, void* notifier);
 
+/* The same conv on a transformed input: x' = in_act(x * in_scale[c] + in_shift[c]) per input channel c, with the
+ * zero padding applied AFTER the transform (a padding tap contributes 0, not in_act(in_shift[c])); in_act is
+ * PAELLA_ACT_NONE or PAELLA_ACT_RELU.  This is a batch-norm (+ ReLU) stage that stands in front of a conv and cannot
+ * be folded into the producer's weights -- pre-activation dense layers, the leading norm of an ArcFace unit -- run
+ * inside the conv's operand fetch instead of as a kernel of its own.  The reference's generated code gets the same
+ * effect from TVM's operator fusion (the kernels behind reference jobs/tvm_arcfaceresnet100/tvm_arcfaceresnet100.cpp:41 and
+ * jobs/tvm_densenet121/tvm_densenet121.cpp:41).  Only plans for which paella_conv2d_plan_takes_input_transform() returns 1
+ * (MFMA plan, mi == ni == 1, C a multiple of 8); PAELLA_ENOSUP otherwise. */
+int paella_conv2d_plan_takes_input_transform(const paella_conv_plan* plan);
+int paella_conv2d_launch_transformed(const paella_conv_plan* plan, const float* x, const float* in_scale, const float* in_shift,
+                                     int in_act, const void* blob_dev, const float* bias, const float* residual,
+                                     const float* slope, float* y, void* workspace, void* stream, uint32_t job_id,
+                                     void* notifier);
+
 /* Two convs that do not depend on each other as ONE launch: the first problem's workgroups followed by the
  * second's, so that layers whose own grids are far below the 256 CUs (the 1x1 projection beside a residual block's
  * first 3x3 conv, parallel branches of an inception module) fill the device together and cost one dispatch.  No

@@ -107,6 +107,16 @@ template <int MI, int NI>
 struct Frag {
     float4 a[MI];
     float b[NI][4];
+    float4 sc, sh;  // only with a fused input transform: scale and shift of the lane's four channels (zero for a padding tap)
+};
+
+// Per-channel transform of the conv's input, applied to the im2col operand on its way into the matrix pipe:
+// x' = max(x * scale[c] + shift[c], lo) inside the image, 0 in the padding -- a batch-norm (lo = -inf) or batch-norm + ReLU
+// (lo = 0) stage that would otherwise run as a kernel of its own in front of the conv.
+struct PreOp {
+    const float* scale;
+    const float* shift;
+    float lo;
 };
 
 // Build-time diagnostic: -DPAELLA_CONV_ABLATE=<bits> removes parts of the kernel to see what bounds it
@@ -122,8 +132,9 @@ struct Frag {
 #endif
 
 // One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
-template <int MI, int NI, int KW, bool TAP_MAJOR>
-__device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid) {
+template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
+__device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
+    static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
     CONV_TL(0);
     if (PAELLA_CONV_ABLATE & 16) return;
     paella::hook_entry(p.notifier, p.job_id);
@@ -198,6 +209,11 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
     // with consecutive chunk indices): channel block within the tap, filter row, filter column.
     const int HW4 = p.H * p.W * 4;
     const int kk4hw = kk * 4 * HW4;
+    __amdgpu_buffer_rsrc_t sres, hres;
+    if (PRE) {
+        sres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, (unsigned)(p.CB * 32), 0x00027000);
+        hres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, (unsigned)(p.CB * 32), 0x00027000);
+    }
     int st_cb = 0, st_r = 0, st_s = 0;
     if (TAP_MAJOR) {
         const int tap = (int)quot((unsigned)c_begin, (unsigned)p.CB, p.div_cb, p.fast_div);
@@ -226,6 +242,11 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
                 for (int t = 0; t < 4; ++t)  // the channel step rides in the scalar offset, which is not range-checked:
                                              // an out-of-range voff stays out of range, a valid one stays valid
                     f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, voff, t * HW4, 0));
+                if (PRE) {  // a tap outside the image gets scale = shift = 0, so it stays the zero the padding asks for
+                    const int soff = ok ? (st_cb * 8 + kk * 4) * 4 : -1;
+                    f.sc = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(sres, soff, 0, 0));
+                    f.sh = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(hres, soff, 0, 0));
+                }
             }
             if (++st_cb == p.CB) {
                 st_cb = 0;
@@ -319,8 +340,14 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
                 const float av = t == 0 ? f.a[mi].x : t == 1 ? f.a[mi].y : t == 2 ? f.a[mi].z : f.a[mi].w;
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
-                    if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * f.b[ni][t];
-                    else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, f.b[ni][t], acc[mi][ni], 0, 0, 0);
+                    float bv = f.b[ni][t];
+                    if (PRE) {
+                        const float sc = t == 0 ? f.sc.x : t == 1 ? f.sc.y : t == 2 ? f.sc.z : f.sc.w;
+                        const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
+                        bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
+                    }
+                    if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * bv;
+                    else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
                 }
             }
         }
@@ -470,6 +497,17 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid)
 template <int MI, int NI, int KW, bool TAP_MAJOR>
 __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
     conv_tile<MI, NI, KW, TAP_MAJOR>(p, blockIdx.x);
+}
+
+// A conv that applies a per-channel transform to its input on the way (smallest tile, tap-major order).
+struct ConvPreArgs {
+    ConvArgs conv;
+    PreOp pre;
+};
+
+template <int KW>
+__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_pre_kernel(ConvPreArgs a) {
+    conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
 }
 
 // Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
@@ -868,6 +906,43 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.notifier = nf;
     dim3 grid((PQ + 255) / 256, d.C);
     paella::launch(dwconv_kernel, grid, dim3(256), 0, st, a);
+    return (int)hipGetLastError();
+}
+
+typedef void (*ConvPreKernel)(ConvPreArgs);
+
+static ConvPreKernel pick_pre_kernel(int kw) {
+    switch (kw) {
+        case 1: return conv_mfma_pre_kernel<1>;
+        case 2: return conv_mfma_pre_kernel<2>;
+        case 4: return conv_mfma_pre_kernel<4>;
+        case 8: return conv_mfma_pre_kernel<8>;
+        default: return nullptr;
+    }
+}
+
+extern "C" int paella_conv2d_plan_takes_input_transform(const paella_conv_plan* plan) {
+    return plan && plan->kind == 0 && plan->mi == 1 && plan->ni == 1 && plan->k_order == 1 ? 1 : 0;
+}
+
+extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, const float* x, const float* in_scale, const float* in_shift,
+                                                int in_act, const void* blob_dev, const float* bias, const float* residual,
+                                                const float* slope, float* y, void* workspace, void* stream, uint32_t job_id,
+                                                void* notifier) {
+    if (!plan || !x || !in_scale || !in_shift || !blob_dev || !y) return PAELLA_EINVAL;
+    if (in_act != PAELLA_ACT_NONE && in_act != PAELLA_ACT_RELU) return PAELLA_EINVAL;
+    if (!paella_conv2d_plan_takes_input_transform(plan)) return PAELLA_ENOSUP;
+    ConvPreKernel kern = pick_pre_kernel(plan->kw);
+    if (!kern) return PAELLA_EINVAL;
+    ConvPreArgs a;
+    if (int rc = fill_args(plan, x, blob_dev, bias, residual, slope, y, workspace, job_id,
+                           reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier), a.conv))
+        return rc;
+    a.pre.scale = in_scale;
+    a.pre.shift = in_shift;
+    a.pre.lo = in_act == PAELLA_ACT_RELU ? 0.f : -__builtin_inff();
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
+    paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();
 }
 

@@ -38,6 +38,7 @@ struct StagePlan {
 struct Launch {
     int nodes[PAELLA_CONV_GROUP_MAX] = {-1, -1, -1, -1};  // node indices, in launch order
     int count = 0;
+    int pre = -1;  // count == 1: the scale-shift node whose work the conv nodes[0] does on its input, if any
     paella_launch_dims dims{};
 };
 
@@ -52,6 +53,8 @@ struct paella_model {
     bool pairing = true;
     char* weights_dev = nullptr;
     std::vector<StagePlan> plans;   // one per node
+    std::vector<int> absorbed_by;   // per node: the conv that applies this scale-shift node to its own input, or -1
+    std::vector<int> pre_of;        // per node: the scale-shift node this conv applies to its input, or -1
     std::vector<Launch> stages;     // in execution order
 };
 
@@ -118,6 +121,48 @@ int log2_ceil(int v) {
 // the list -- on the arena addresses, so that buffers sharing memory count -- and stays as close to the list as that
 // allows.  Convs with fewer waves per workgroup are re-planned to the largest count of their group; their packed
 // weights do not depend on that.
+// A per-channel scale-shift stage (batch-norm, with or without ReLU) that feeds nothing but convs able to apply it
+// to their own input is not launched: each of those convs reads the stage's input and transforms it while fetching
+// operands (paella_conv2d_launch_transformed).  Conditions, on arena addresses so that buffers sharing memory count:
+// every reader of the stage's output, up to the node that overwrites it, is such a conv and reads exactly that view;
+// the output is not the model's; and nothing between the stage and its last reader overwrites the stage's input.
+void absorb_scale_shifts(paella_model* m) {
+    const Graph& g = m->g;
+    const int n = (int)g.nodes.size();
+    m->absorbed_by.assign(n, -1);
+    m->pre_of.assign(n, -1);
+    if (!m->pairing) return;
+    auto overlap = [&](const View& a, const View& b) {
+        if (a.buf < 0 || b.buf < 0) return false;
+        const size_t a0 = g.buffers[a.buf].offset + a.off, b0 = g.buffers[b.buf].offset + b.off;
+        return a0 < b0 + b.numel() && b0 < a0 + a.numel();
+    };
+    for (int e = 0; e < n; ++e) {
+        const Node& el = g.nodes[e];
+        if (el.op != Op::Eltwise || el.x2.buf >= 0 || el.scale < 0 || el.shift < 0 || el.slope >= 0) continue;
+        if (el.act != PAELLA_ACT_NONE && el.act != PAELLA_ACT_RELU) continue;
+        if (overlap(el.y, g.output) || overlap(el.y, el.x)) continue;
+        std::vector<int> readers;
+        bool ok = true;
+        for (int j = e + 1; j < n && ok; ++j) {
+            const Node& c = g.nodes[j];
+            if (overlap(c.x, el.y) || overlap(c.x2, el.y)) {
+                const bool same_view = c.x.buf == el.y.buf && c.x.off == el.y.off && c.x.C == el.y.C && c.x.H == el.y.H && c.x.W == el.y.W;
+                ok = c.op == Op::Conv && same_view && !overlap(c.x2, el.y) && m->pre_of[j] < 0 &&
+                     paella_conv2d_plan_takes_input_transform(&m->plans[j].conv) == 1;
+                if (ok) readers.push_back(j);
+            }
+            if (overlap(c.y, el.y)) break;  // the output's memory starts a new life here
+        }
+        if (!ok || readers.empty()) continue;
+        for (int k = e + 1; k < readers.back() && ok; ++k)
+            if (overlap(g.nodes[k].y, el.x)) ok = false;
+        if (!ok) continue;
+        m->absorbed_by[e] = readers.front();
+        for (int j : readers) m->pre_of[j] = e;
+    }
+}
+
 void pair_up(paella_model* m) {
     const Graph& g = m->g;
     const int n = (int)g.nodes.size();
@@ -126,12 +171,18 @@ void pair_up(paella_model* m) {
         const size_t a0 = g.buffers[a.buf].offset + a.off, b0 = g.buffers[b.buf].offset + b.off;
         return a0 < b0 + b.numel() && b0 < a0 + a.numel();
     };
-    auto ordered = [&](const Node& a, const Node& b) {  // b must stay behind a
-        return overlap(a.y, b.x) || overlap(a.y, b.x2) || overlap(a.y, b.y) || overlap(b.y, a.x) || overlap(b.y, a.x2);
+    // What a node reads and writes once absorbed scale-shift stages are gone: the stage itself nothing, the conv
+    // that does its work the stage's input.
+    const View none;
+    auto in1 = [&](int i) -> const View& { return m->absorbed_by[i] >= 0 ? none : m->pre_of[i] >= 0 ? g.nodes[m->pre_of[i]].x : g.nodes[i].x; };
+    auto in2 = [&](int i) -> const View& { return m->absorbed_by[i] >= 0 ? none : g.nodes[i].x2; };
+    auto out = [&](int i) -> const View& { return m->absorbed_by[i] >= 0 ? none : g.nodes[i].y; };
+    auto ordered = [&](int a, int b) {  // b must stay behind a
+        return overlap(out(a), in1(b)) || overlap(out(a), in2(b)) || overlap(out(a), out(b)) || overlap(out(b), in1(a)) || overlap(out(b), in2(a));
     };
     auto pairable = [&](int i) {
         const StagePlan& st = m->plans[i];
-        return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1;
+        return st.node->op == Op::Conv && st.conv.kind == 0 && st.conv.mi == 1 && st.conv.ni == 1 && m->pre_of[i] < 0;
     };
     // The plan of node i with kw waves per workgroup; false if that is not possible.
     auto with_waves = [&](int i, int kw, StagePlan* out) {
@@ -148,13 +199,13 @@ void pair_up(paella_model* m) {
     std::vector<int> waits_for(n, 0);
     for (int i = 0; i < n; ++i)
         for (int j = i + 1; j < n; ++j)
-            if (m->pairing ? ordered(g.nodes[i], g.nodes[j]) : j == i + 1) {
+            if (m->pairing ? ordered(i, j) : j == i + 1) {
                 later[i].push_back(j);
                 ++waits_for[j];
             }
     std::set<int> ready;  // no two ready nodes are ordered with respect to each other
     for (int i = 0; i < n; ++i)
-        if (waits_for[i] == 0) ready.insert(i);
+        if (waits_for[i] == 0 && m->absorbed_by[i] < 0) ready.insert(i);  // an absorbed stage goes out with its first reader
 
     m->stages.clear();
     size_t area[PAELLA_CONV_GROUP_MAX] = {0, 0, 0, 0};
@@ -206,6 +257,8 @@ void pair_up(paella_model* m) {
         }
         if (l.count == 1) {
             l.dims = m->plans[l.nodes[0]].dims;
+            const int pre = m->pre_of[l.nodes[0]];
+            if (pre >= 0 && m->absorbed_by[pre] == l.nodes[0]) l.pre = pre;
         } else {
             // the convs whose workgroups run longer go first: the short ones fill in behind them
             std::stable_sort(l.nodes, l.nodes + l.count, [&](int a, int b) {
@@ -310,6 +363,7 @@ int build(paella_model* m) {
     std::vector<size_t> tensor_off, blob_off;
     size_t total = 0;
     if (int rc = plan_nodes(m, tensor_off, blob_off, total)) return rc;
+    absorb_scale_shifts(m);
     pair_up(m);
 
     // Generate, pack, upload.
@@ -410,11 +464,16 @@ int paella_model_launch_plan(const char* name, int* out, size_t capacity) {
     std::vector<size_t> tensor_off, blob_off;
     size_t total = 0;
     if (int rc = plan_nodes(&m, tensor_off, blob_off, total)) return rc;
+    absorb_scale_shifts(&m);
     pair_up(&m);
     size_t used = 0;
     for (const Launch& l : m.stages) {
-        if (out && used < capacity) out[used] = l.count;
+        if (out && used < capacity) out[used] = l.count + (l.pre >= 0 ? 1 : 0);
         ++used;
+        if (l.pre >= 0) {
+            if (out && used < capacity) out[used] = l.pre;
+            ++used;
+        }
         for (int k = 0; k < l.count; ++k, ++used)
             if (out && used < capacity) out[used] = l.nodes[k];
     }
@@ -472,8 +531,14 @@ int paella_model_stage_work(const paella_model* m, int stage, const char** op, d
 int paella_model_stage_nodes(const paella_model* m, int stage, int* nodes, int capacity) {
     if (!m || stage < 0 || (size_t)stage >= m->stages.size() || capacity < 0) return PAELLA_EINVAL;
     const Launch& l = m->stages[stage];
-    for (int k = 0; nodes && k < l.count && k < capacity; ++k) nodes[k] = l.nodes[k];
-    return l.count;
+    int count = 0;
+    if (l.pre >= 0) {
+        if (nodes && count < capacity) nodes[count] = l.pre;
+        ++count;
+    }
+    for (int k = 0; k < l.count; ++k, ++count)
+        if (nodes && count < capacity) nodes[count] = l.nodes[k];
+    return count;
 }
 
 int paella_exec_create(const paella_model* m, paella_exec** out) {
@@ -548,6 +613,11 @@ int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t j
     float* y = e->ptr(n.y);
     switch (n.op) {
         case Op::Conv:
+            if (const int pre = e->m->pre_of[l.nodes[0]]; pre >= 0) {
+                const StagePlan& sp = e->m->plans[pre];
+                return paella_conv2d_launch_transformed(&st.conv, e->ptr(sp.node->x), sp.scale, sp.shift, sp.node->act, st.w, st.bias, x2,
+                                                        st.slope, y, e->workspace, stream, job_id, notifier);
+            }
             return paella_conv2d_launch(&st.conv, x, st.w, st.bias, x2, st.slope, y, e->workspace, stream, job_id, notifier);
         case Op::Dense:
             return paella_dense_launch(x, reinterpret_cast<const float*>(st.w), st.bias, y, n.dense_in, n.dense_out, n.act, stream, job_id, notifier);

@@ -54,10 +54,23 @@ class Conv2d:
         self.workspace = torch.zeros(max(self.plan.workspace_bytes, 4) // 4, dtype=torch.int32, device=device) if self.plan.workspace_bytes else None
         self.lib = lib
 
-    def __call__(self, x, residual=None, out=None, stream=None, job_id=0, notifier=None):
+    def takes_input_transform(self):
+        return bool(self.lib.paella_conv2d_plan_takes_input_transform(ctypes.byref(self.plan)))
+
+    def __call__(self, x, residual=None, out=None, stream=None, job_id=0, notifier=None, in_scale=None, in_shift=None, in_act=ACT_NONE):
+        """in_scale / in_shift (per input channel, device tensors): the conv reads in_act(x * in_scale + in_shift), padded
+        with zeros after that transform."""
         p = self.plan
         assert x.shape == (1, p.d.C, p.d.H, p.d.W), (tuple(x.shape), p.d.C, p.d.H, p.d.W)
         y = out if out is not None else torch.empty((1, p.d.K, p.P, p.Q), device=x.device, dtype=torch.float32)
+        if in_scale is not None:
+            assert in_scale.numel() == p.d.C and in_shift.numel() == p.d.C
+            check(self.lib.paella_conv2d_launch_transformed(ctypes.byref(p), _ptr(x), _ptr(in_scale), _ptr(in_shift), in_act,
+                                                            ctypes.c_void_p(self.blob.data_ptr()), _ptr(self.bias), _ptr(residual),
+                                                            _ptr(self.slope), _ptr(y),
+                                                            ctypes.c_void_p(self.workspace.data_ptr()) if self.workspace is not None else None,
+                                                            _stream(stream), job_id, notifier), "paella_conv2d_launch_transformed")
+            return y
         check(self.lib.paella_conv2d_launch(ctypes.byref(p), _ptr(x), ctypes.c_void_p(self.blob.data_ptr()),
                                             _ptr(self.bias), _ptr(residual), _ptr(self.slope), _ptr(y),
                                             ctypes.c_void_p(self.workspace.data_ptr()) if self.workspace is not None else None,

@@ -383,8 +383,16 @@ def test_launch_plan_keeps_every_dependence_of_the_graph(name):
             os.environ["PAELLA_CONV_PAIRS"] = before
     assert sorted(i for launch in plan for i in launch) == list(range(len(nodes)))
     assert all(1 <= len(launch) <= 4 for launch in plan)
-    assert all(nodes[i]["op"] == "conv" and nodes[i]["groups"] == 1 for launch in plan if len(launch) > 1 for i in launch)
+    # a scale-shift operator may lead the conv that applies it to its own input; apart from that, shared launches hold convs only
+    absorbed = {launch[0]: launch[1] for launch in plan if len(launch) == 2 and nodes[launch[0]]["op"] == "eltwise"}
+    for e, c in absorbed.items():
+        assert nodes[c]["op"] == "conv" and nodes[c]["groups"] == 1 and nodes[c]["x"] == nodes[e]["y"] and nodes[e]["x2"]["buf"] < 0
+        assert nodes[e]["act"] in (0, 1), nodes[e]
+    assert all(nodes[i]["op"] == "conv" and nodes[i]["groups"] == 1 for launch in plan if len(launch) > 1 and launch[0] not in absorbed
+               for i in launch)
     stage_of = {i: k for k, launch in enumerate(plan) for i in launch}
+    # An absorbed operator's output is never written: its readers read its input instead, at their own position.
+    readers = {e: [j for j in range(e + 1, len(nodes)) if nodes[j]["x"] == nodes[e]["y"]] for e in absorbed}
 
     def span(v):
         return None if v["buf"] < 0 else (v["buf"], v["off"], v["off"] + v["C"] * v["H"] * v["W"])
@@ -393,11 +401,23 @@ def test_launch_plan_keeps_every_dependence_of_the_graph(name):
         return a is not None and b is not None and a[0] == b[0] and a[1] < b[2] and b[1] < a[2]
 
     spans = [(span(n["x"]), span(n["x2"]), span(n["y"])) for n in nodes]
+    for e, c in absorbed.items():
+        # the absorbed operator itself touches nothing; every conv that read its output reads its input
+        first = [j for j in range(e + 1, len(nodes)) if hit(spans[j][2], spans[e][2])]
+        live = [j for j in readers[e] if not first or j <= first[0]]
+        assert live and live[0] == c
+        for j in range(e + 1, (first[0] + 1) if first else len(nodes)):   # nobody else reads the output that is never written
+            assert j in live or not (hit(spans[j][0], spans[e][2]) or hit(spans[j][1], spans[e][2])), (name, e, j)
+        for j in live:
+            spans[j] = (spans[e][0], spans[j][1], spans[j][2])
+        spans[e] = (None, None, None)
     for j, (xj, x2j, yj) in enumerate(spans):
         for i in range(j):
             xi, x2i, yi = spans[i]
             if hit(yi, xj) or hit(yi, x2j) or hit(yi, yj) or hit(yj, xi) or hit(yj, x2i):
                 assert stage_of[i] < stage_of[j], (name, i, j)
+    if name in ("densenet121", "arcfaceresnet100"):
+        assert len(absorbed) >= 49 and sum(n["op"] == "eltwise" for n in nodes) - len(absorbed) == 1
     if name == "resnet18":
         assert [launch for launch in plan if len(launch) > 1] == [[7, 6], [12, 11], [17, 16]]  # first 3x3 of the block, then its projection
     if name in ("inception_v3", "googlenet"):

@@ -82,6 +82,62 @@ def test_conv2d_every_tile_variant(cuda, mi, ni, kwlog):
     close(got, ref)
 
 
+# C, H, W, K, R, S, stride, pad, input activation, waves (log2; -1: the library's choice), residual
+TRANSFORMED = [
+    (64, 56, 56, 128, 1, 1, 1, 0, orc.ACT_RELU, -1, False),    # DenseNet bottleneck: norm + ReLU in front of a 1x1
+    (352, 14, 14, 128, 1, 1, 1, 0, orc.ACT_RELU, -1, False),
+    (64, 28, 28, 64, 3, 3, 1, 1, orc.ACT_NONE, -1, False),     # ArcFace unit: norm in front of a zero-padded 3x3
+    (128, 14, 14, 128, 3, 3, 2, 1, orc.ACT_NONE, -1, True),
+    (512, 7, 7, 512, 3, 3, 1, 1, orc.ACT_NONE, -1, False),     # split reduction
+    (40, 19, 23, 72, 3, 3, 1, 2, orc.ACT_RELU, 0, True),       # padding wider than the filter's reach; every wave count
+    (40, 19, 23, 72, 3, 3, 1, 2, orc.ACT_RELU, 1, True),
+    (40, 19, 23, 72, 3, 3, 1, 2, orc.ACT_NONE, 2, False),
+    (40, 19, 23, 72, 5, 3, 2, (2, 1), orc.ACT_RELU, 3, True),
+]
+
+
+@pytest.mark.parametrize("case", TRANSFORMED)
+def test_conv2d_on_transformed_input(cuda, case):
+    """conv(act(x * scale + shift)) in one launch against the oracle's scale-shift followed by its conv.  The shifts are
+    large and of both signs, so a padding tap that wrongly carried act(shift) instead of 0 would show at every border."""
+    from paella_amd import ops
+    c, h, w, k, r, s, stride, pad, in_act, kwlog, with_res = case
+    x = rnd(1, c, h, w)
+    wt, b = rnd(k, c, r, s, scale=(2.0 / (c * r * s)) ** 0.5), rnd(k, scale=0.1)
+    scale, shift = rnd(c) + 1.5, rnd(c, scale=2.0)
+    mid = orc.scale_shift(x, scale, shift, act=in_act)
+    conv = ops.Conv2d(wt, b, stride=stride, pad=pad, act=ops.ACT_RELU, in_hw=(h, w), has_residual=with_res,
+                      tile_hint=0 if kwlog < 0 else (1 << 8) | (1 << 4) | kwlog)
+    assert conv.takes_input_transform()
+    res = rnd(1, k, conv.plan.P, conv.plan.Q) if with_res else None
+    ref = orc.conv2d(mid, wt, b, stride=stride, pad=pad, act=orc.ACT_RELU, residual=res)
+    dev = lambda a: None if a is None else torch.tensor(a, device=cuda)
+    got = conv(dev(x), residual=dev(res), in_scale=dev(scale), in_shift=dev(shift), in_act=in_act)
+    torch.cuda.synchronize()
+    close(got, ref)
+    # and the two-launch form gives the same within the tolerance (the fused form rounds x * scale + shift once, as a
+    # fused multiply-add)
+    two = conv(ops.eltwise(dev(x), scale=dev(scale), shift=dev(shift), act=in_act), residual=dev(res))
+    torch.cuda.synchronize()
+    close(two, ref)
+
+
+def test_conv2d_input_transform_is_refused_where_not_built(cuda):
+    from paella_amd import ops
+    x = torch.zeros((1, 5, 9, 11), device=cuda)
+    conv = ops.Conv2d(rnd(7, 5, 3, 3), None, pad=1, in_hw=(9, 11))      # C is no multiple of 8: offset-table order
+    assert not conv.takes_input_transform()
+    ones = torch.ones(5, device=cuda)
+    with pytest.raises(RuntimeError):
+        conv(x, in_scale=ones, in_shift=ones)
+    big = ops.Conv2d(rnd(72, 40, 3, 3), None, pad=1, in_hw=(19, 23), tile_hint=(2 << 8) | (1 << 4) | 2)   # 64 x 32 tile
+    assert not big.takes_input_transform()
+    conv8 = ops.Conv2d(rnd(8, 8, 3, 3), None, pad=1, in_hw=(9, 11))
+    ones8 = torch.ones(8, device=cuda)
+    with pytest.raises(RuntimeError):
+        conv8(torch.zeros((1, 8, 9, 11), device=cuda), in_scale=ones8, in_shift=ones8, in_act=ops.ACT_RELU6)
+
+
 @pytest.mark.parametrize("act", [orc.ACT_NONE, orc.ACT_RELU6, orc.ACT_CLIP])
 def test_conv2d_epilogues_and_channel_slice_output(cuda, act):
     """Output written into channels [8, 8+24) of a 40-channel concat buffer; the rest must stay untouched."""
