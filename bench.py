@@ -315,27 +315,43 @@ def main():
 
     # The two-tenant mix of the target statement: small CNN : Inception-v3 (299x299) = 9 : 1, full3 against plain
     # multi-stream serving (fifo), first at saturation, then open-loop Poisson at fractions of the lower of the two.
-    mix = None
-    if not args.no_arms and not args.no_mix:
-        mix_jobs = [(serve.job_path("tvm_mnist"), 0.9, args.concurrency), (serve.job_path("tvm_inception_v3"), 0.1, args.concurrency)]
-        n_mix = 3000
+    def mix_arm(workload, tenants, fracs, n_mix=3000):
+        """tenants: (label, job adapter, share).  Saturation, then open-loop Poisson at fractions of the lower saturation rate."""
+        mix_jobs = [(serve.job_path(adapter), share, args.concurrency) for _, adapter, share in tenants]
+        arms2 = [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]
         sat = {}
-        for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+        for label, sched, streams in arms2:
             r = serve_arm(serve, sched, streams, mix_jobs, args.concurrency, n_mix, 300, extra_kernels=args.extra_kernels)
             sat[label] = r["throughput_rps"]
-        mix = {"workload": "small CNN : Inception-v3 = 9 : 1, inputs resident", "saturation_rps": sat, "poisson": []}
-        log("[bench]   mix saturation: full3 %.0f req/s, fifo %.0f req/s" % (sat["full3"], sat["fifo_multi_stream"]))
-        for frac in (0.5, 0.8):
+        res = {"workload": workload, "saturation_rps": sat, "poisson": []}
+        log("[bench]   %s, saturation: full3 %.0f req/s, fifo %.0f req/s" % (workload, sat["full3"], sat["fifo_multi_stream"]))
+        for frac in fracs:
             rate = frac * min(sat.values())
             point = {"offered_rps": rate}
-            for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+            for label, sched, streams in arms2:
                 r = serve_arm(serve, sched, streams, mix_jobs, args.concurrency, n_mix, 300, iat_us=1e6 / rate, extra_kernels=args.extra_kernels)
-                point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"],
-                                "small_cnn_p99_us": r["per_type"][0]["p99"], "inception_v3_p99_us": r["per_type"][1]["p99"]}
-            mix["poisson"].append(point)
-            log("[bench]   mix poisson %.0f req/s: p99 small CNN / Inception: full3 %.0f / %.0f us, fifo %.0f / %.0f us" %
-                (rate, point["full3"]["small_cnn_p99_us"], point["full3"]["inception_v3_p99_us"],
-                 point["fifo_multi_stream"]["small_cnn_p99_us"], point["fifo_multi_stream"]["inception_v3_p99_us"]))
+                point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"]}
+                for k, (tenant, _, _) in enumerate(tenants):
+                    point[label][tenant + "_p99_us"] = r["per_type"][k]["p99"]
+            res["poisson"].append(point)
+            log("[bench]   %s, poisson %.0f req/s: p99 full3 %.0f us, fifo %.0f us; per tenant full3 %s | fifo %s" %
+                (workload, rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"],
+                 " ".join("%.0f" % point["full3"][t + "_p99_us"] for t, _, _ in tenants),
+                 " ".join("%.0f" % point["fifo_multi_stream"][t + "_p99_us"] for t, _, _ in tenants)))
+        return res
+
+    # The two-tenant mix of the target statement: small CNN : Inception-v3 (299x299) = 9 : 1, full3 against plain
+    # multi-stream serving (fifo), first at saturation, then open-loop Poisson at fractions of the lower of the two.
+    # Then the other two mixes of the benchmark configurations, the same way at one load point.
+    mix, other_mixes = None, []
+    if not args.no_arms and not args.no_mix:
+        mix = mix_arm("small CNN : Inception-v3 = 9 : 1, inputs resident",
+                      [("small_cnn", "tvm_mnist", 0.9), ("inception_v3", "tvm_inception_v3", 0.1)], (0.5, 0.8))
+        other_mixes.append(mix_arm("MobileNetV2 : ResNet-50 = 1 : 1, inputs resident",
+                                   [("mobilenetv2", "tvm_mobilenet", 0.5), ("resnet50", "tvm_resnet50", 0.5)], (0.8,)))
+        eight = ["densenet121", "googlenet", "squeezenet1_1", "resnet34", "ultraface320", "arcfaceresnet100", "mobilenet", "mnist"]
+        other_mixes.append(mix_arm("eight models, uniform choice, inputs resident",
+                                   [(m, "tvm_" + m, 0.125) for m in eight], (0.8,), n_mix=2000))
 
     # One client, one request at a time, small CNN, 10 000 requests, input and output crossing PCIe: the latency
     # floor of the full path (its 5 kernels are small enough to be issued as one scheduler stage).
@@ -493,6 +509,7 @@ def main():
         "arms": arms,
         "poisson_sweep": sweep,
         "two_tenant_mix": mix,
+        "other_mixes": other_mixes,
         "small_cnn_closed_loop": closed_loop,
         "fairness_sweep": fairness_sweep,
         "direct_single_stream_rps": rl["direct_rps"],
