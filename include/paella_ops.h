@@ -157,6 +157,15 @@ int paella_pool2d_dims(const paella_pool_desc* d, paella_launch_dims* dims);
 int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y,
                          void* stream, uint32_t job_id, void* notifier);
 
+/* Up to three such convs (tap-major plans: C a multiple of 8) and one pooling operator in ONE launch: the conv
+ * problems' workgroups followed by the pool's, one output element per thread.  An inception module starts with
+ * three 1x1 convs and a 3x3 pool that all read the module's input; alone the pool is a launch shorter than the cost of
+ * launching it.  No counterpart in the reference (one kernel per fused operator).  The pool must not read or
+ * overwrite what a member writes, nor write what a member reads.  Results are bit-identical to separate launches. */
+int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plans, int n, const paella_pool_desc* pool, paella_launch_dims* dims);
+int paella_conv2d_launch_group_pool(const paella_conv_operands* members, int n, const paella_pool_desc* pool, const float* pool_x,
+                                    float* pool_y, void* stream, uint32_t job_id, void* notifier);
+
 /* y[c] = mean over HW of x[c][:] */
 int paella_global_avgpool_dims(int C, int HW, paella_launch_dims* dims);
 int paella_global_avgpool_launch(const float* x, float* y, int C, int HW,

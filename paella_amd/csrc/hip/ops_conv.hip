@@ -33,6 +33,7 @@
 
 #include "launch.h"
 #include "out_store.h"
+#include "pool_body.h"
 
 // Build-time diagnostic (never defined in the shipped library): thread 0 of every workgroup records the
 // 100 MHz wall clock at a few points of the kernel.
@@ -531,6 +532,33 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_
     conv_tile<1, 1, KW, TAP_MAJOR>(g.prob[idx], blockIdx.x - g.start[idx]);
 }
 
+// Up to three such convs and one pooling operator in one launch: an inception module starts with three 1x1 convs and
+// a 3x3 pool that all read the module's input.  The pool's workgroups come last (they are the shortest), each thread
+// one output element as in the pooling kernel, with this kernel's workgroup size.
+constexpr int kMaxGroupWithPool = 3;
+
+struct ConvGroupPoolArgs {
+    ConvArgs prob[kMaxGroupWithPool];
+    unsigned start[kMaxGroupWithPool];  // first workgroup id of each conv; 0xFFFFFFFF for unused entries
+    unsigned pool_start;                // first workgroup id of the pool
+    paella::PoolArgs pool;
+};
+
+template <int KW>
+__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_group_pool_kernel(ConvGroupPoolArgs g) {
+    if (blockIdx.x >= g.pool_start) {
+        paella::hook_entry(g.pool.notifier, g.pool.job_id);
+        paella::pool_element(g.pool, (int)((blockIdx.x - g.pool_start) * (64 * KW) + threadIdx.x));
+        paella::hook_exit(g.pool.notifier, g.pool.job_id);
+        return;
+    }
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGroupWithPool; ++i)
+        if (blockIdx.x >= g.start[i]) idx = i;
+    conv_tile<1, 1, KW, true>(g.prob[idx], blockIdx.x - g.start[idx]);
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Depthwise conv (groups == C == K): HBM-bound, one thread per output pixel, taps from L1/L2.
 
@@ -862,6 +890,77 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
         if (i < n) next += m.plan->dims.grid;
     }
     ConvGroupKernel kern = pick_group_kernel(plans[0]->kw, plans[0]->k_order);
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
+    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
+    return (int)hipGetLastError();
+}
+
+namespace {
+
+typedef void (*ConvGroupPoolKernel)(ConvGroupPoolArgs);
+
+ConvGroupPoolKernel pick_group_pool_kernel(int kw) {
+    switch (kw) {
+        case 1: return conv_mfma_group_pool_kernel<1>;
+        case 2: return conv_mfma_group_pool_kernel<2>;
+        case 4: return conv_mfma_group_pool_kernel<4>;
+        case 8: return conv_mfma_group_pool_kernel<8>;
+        default: return nullptr;
+    }
+}
+
+}  // namespace
+
+extern "C" int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plans, int n, const paella_pool_desc* pool, paella_launch_dims* dims) {
+    if (!plans || n < 1 || n > kMaxGroupWithPool || !pool) return PAELLA_EINVAL;
+    for (int i = 0; i < n; ++i) {
+        if (!plans[i]) return PAELLA_EINVAL;
+        const paella_conv_plan& p = *plans[i];
+        if (p.kind != 0 || p.mi != 1 || p.ni != 1 || p.kw != plans[0]->kw || p.k_order != 1) return PAELLA_ENOSUP;
+    }
+    paella::PoolArgs pa;
+    if (!paella::pool_fill_args(pool, nullptr, nullptr, 0, nullptr, &pa)) return PAELLA_EINVAL;
+    if (dims) {
+        dims->grid = 0;
+        dims->lds_bytes = 0;
+        for (int i = 0; i < n; ++i) {
+            dims->grid += plans[i]->dims.grid;
+            if (plans[i]->dims.lds_bytes > dims->lds_bytes) dims->lds_bytes = plans[i]->dims.lds_bytes;
+        }
+        dims->block = plans[0]->dims.block;
+        dims->grid += (unsigned)(((size_t)pa.C * pa.P * pa.Q + dims->block - 1) / dims->block);
+        dims->vgprs = plans[0]->dims.vgprs;
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_group_pool_kernel(plans[0]->kw))) == hipSuccess && attr.numRegs > 0)
+            dims->vgprs = (unsigned)attr.numRegs;
+        else
+            (void)hipGetLastError();
+    }
+    return 0;
+}
+
+extern "C" int paella_conv2d_launch_group_pool(const paella_conv_operands* members, int n, const paella_pool_desc* pool, const float* pool_x,
+                                               float* pool_y, void* stream, uint32_t job_id, void* notifier) {
+    if (!members || n < 1 || n > kMaxGroupWithPool || !pool || !pool_x || !pool_y) return PAELLA_EINVAL;
+    const paella_conv_plan* plans[kMaxGroupWithPool];
+    for (int i = 0; i < n; ++i) plans[i] = members[i].plan;
+    paella_launch_dims dims;
+    if (int rc = paella_conv2d_group_pool_dims(plans, n, pool, &dims)) return rc;
+    for (int i = 0; i < n; ++i)
+        for (int j = i + 1; j < n; ++j)
+            if (plans[i]->splits > 1 && plans[j]->splits > 1 && members[i].workspace == members[j].workspace) return PAELLA_EINVAL;
+    auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
+    ConvGroupPoolArgs g;
+    unsigned next = 0;
+    for (int i = 0; i < kMaxGroupWithPool; ++i) {
+        const paella_conv_operands& m = members[i < n ? i : 0];  // unused entries: a valid copy that no workgroup selects
+        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, g.prob[i])) return rc;
+        g.start[i] = i < n ? next : 0xFFFFFFFFu;
+        if (i < n) next += m.plan->dims.grid;
+    }
+    g.pool_start = next;
+    if (!paella::pool_fill_args(pool, pool_x, pool_y, job_id, notifier, &g.pool)) return PAELLA_EINVAL;
+    ConvGroupPoolKernel kern = pick_group_pool_kernel(plans[0]->kw);
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
     paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
     return (int)hipGetLastError();

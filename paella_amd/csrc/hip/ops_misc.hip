@@ -12,6 +12,7 @@
 
 #include "launch.h"
 #include "out_store.h"
+#include "pool_body.h"
 
 namespace {
 
@@ -123,60 +124,11 @@ __global__ __launch_bounds__(512) void dense_long_kernel(const float* __restrict
 }
 
 // ------------------------------------------------------------------------------------------ pooling
-struct PoolArgs {
-    const float* x;
-    float* y;
-    int C, H, W, P, Q, R, S, sh, sw, ph, pw;
-    int is_avg, count_include_pad;
-    uint32_t job_id;
-    Notifier* notifier;
-};
+using paella::PoolArgs;
 
 __global__ __launch_bounds__(256) void pool_kernel(PoolArgs p) {
     paella::hook_entry(p.notifier, p.job_id);
-    const int PQ = p.P * p.Q;
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx < p.C * PQ) {
-        const int c = idx / PQ;
-        const int pix = idx - c * PQ;
-        const int po = pix / p.Q;
-        const int qo = pix - po * p.Q;
-        const float* xc = p.x + (size_t)c * p.H * p.W;
-        const int h0 = po * p.sh - p.ph, w0 = qo * p.sw - p.pw;
-        if (p.is_avg) {
-            float acc = 0.f;
-            int valid = 0;
-            for (int r = 0; r < p.R; ++r) {
-                const int h = h0 + r;
-                if ((unsigned)h >= (unsigned)p.H) continue;
-                for (int s = 0; s < p.S; ++s) {
-                    const int w = w0 + s;
-                    if ((unsigned)w >= (unsigned)p.W) continue;
-                    acc += xc[(size_t)h * p.W + w];
-                    ++valid;
-                }
-            }
-            int div = valid;
-            if (p.count_include_pad) {
-                // window clipped to the padded extent [-pad, in + pad)
-                const int he = min(h0 + p.R, p.H + p.ph), we = min(w0 + p.S, p.W + p.pw);
-                div = (he - h0) * (we - w0);
-            }
-            store_out(p.y + idx, div ? acc / (float)div : 0.f);
-        } else {
-            float m = -FLT_MAX;
-            for (int r = 0; r < p.R; ++r) {
-                const int h = h0 + r;
-                if ((unsigned)h >= (unsigned)p.H) continue;
-                for (int s = 0; s < p.S; ++s) {
-                    const int w = w0 + s;
-                    if ((unsigned)w >= (unsigned)p.W) continue;
-                    m = fmaxf(m, xc[(size_t)h * p.W + w]);
-                }
-            }
-            store_out(p.y + idx, m);
-        }
-    }
+    paella::pool_element(p, (int)(blockIdx.x * 256 + threadIdx.x));
     paella::hook_exit(p.notifier, p.job_id);
 }
 
@@ -369,15 +321,9 @@ int paella_pool2d_dims(const paella_pool_desc* d, paella_launch_dims* dims) {
 }
 
 int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y, void* stream, uint32_t job_id, void* notifier) {
-    int P, Q;
-    if (int rc = pool_check(d, &P, &Q)) return rc;
-    if (!x || !y) return PAELLA_EINVAL;
     PoolArgs a;
-    a.x = x; a.y = y;
-    a.C = d->C; a.H = d->H; a.W = d->W; a.P = P; a.Q = Q; a.R = d->R; a.S = d->S;
-    a.sh = d->stride_h; a.sw = d->stride_w; a.ph = d->pad_h; a.pw = d->pad_w;
-    a.is_avg = d->is_avg; a.count_include_pad = d->count_include_pad;
-    a.job_id = job_id; a.notifier = (Notifier*)notifier;
+    if (!x || !y || !paella::pool_fill_args(d, x, y, job_id, notifier, &a)) return PAELLA_EINVAL;
+    const int P = a.P, Q = a.Q;
     paella::launch(pool_kernel, dim3(blocks_for((size_t)d->C * P * Q, 256)), dim3(256), 0, (hipStream_t)stream, a);
     return (int)hipGetLastError();
 }

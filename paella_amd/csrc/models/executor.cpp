@@ -39,6 +39,7 @@ struct Launch {
     int nodes[PAELLA_CONV_GROUP_MAX] = {-1, -1, -1, -1};  // node indices, in launch order
     int count = 0;
     int pre = -1;  // count == 1: the scale-shift node whose work the conv nodes[0] does on its input, if any
+    int pool = -1;  // a pooling node that shares the launch with the convs (at most three then), or -1
     paella_launch_dims dims{};
 };
 
@@ -248,7 +249,22 @@ void pair_up(paella_model* m) {
                 }
                 for (int k = l.count; k < PAELLA_CONV_GROUP_MAX; ++k) l.nodes[k] = -1;
             }
-            if (l.count == 1)  // an operator that is no such conv goes first if one is ready: it may release a partner
+            // A ready pooling operator rides along with up to three tap-major convs (an inception module's 3x3 pool beside
+            // its 1x1 convs): on its own it is a launch shorter than the cost of launching it.
+            if (l.count <= 3 && m->plans[l.nodes[0]].conv.k_order == 1) {
+                const paella_conv_plan* plans[PAELLA_CONV_GROUP_MAX];
+                for (int k = 0; k < l.count; ++k) plans[k] = &m->plans[l.nodes[k]].conv;
+                for (int j : ready) {
+                    if (g.nodes[j].op != Op::Pool) continue;
+                    paella_launch_dims with_pool;
+                    if (paella_conv2d_group_pool_dims(plans, l.count, &g.nodes[j].pool, &with_pool) == 0 && with_pool.grid <= 2048) {
+                        l.pool = j;
+                        l.dims = with_pool;
+                    }
+                    break;
+                }
+            }
+            if (l.count == 1 && l.pool < 0)  // an operator that is no such conv goes first if one is ready: it may release a partner
                 for (int j : ready)
                     if (!pairable(j)) {
                         l.nodes[0] = j;
@@ -256,7 +272,7 @@ void pair_up(paella_model* m) {
                     }
         }
         if (l.count == 1) {
-            l.dims = m->plans[l.nodes[0]].dims;
+            if (l.pool < 0) l.dims = m->plans[l.nodes[0]].dims;
             const int pre = m->pre_of[l.nodes[0]];
             if (pre >= 0 && m->absorbed_by[pre] == l.nodes[0]) l.pre = pre;
         } else {
@@ -271,6 +287,11 @@ void pair_up(paella_model* m) {
             for (int j : later[done])
                 if (--waits_for[j] == 0) ready.insert(j);
             if (g.nodes[done].op == Op::Conv && m->plans[done].conv.workspace_bytes > area[k]) area[k] = m->plans[done].conv.workspace_bytes;
+        }
+        if (l.pool >= 0) {
+            ready.erase(l.pool);
+            for (int j : later[l.pool])
+                if (--waits_for[j] == 0) ready.insert(j);
         }
         m->stages.push_back(l);
     }
@@ -468,7 +489,7 @@ int paella_model_launch_plan(const char* name, int* out, size_t capacity) {
     pair_up(&m);
     size_t used = 0;
     for (const Launch& l : m.stages) {
-        if (out && used < capacity) out[used] = l.count + (l.pre >= 0 ? 1 : 0);
+        if (out && used < capacity) out[used] = l.count + (l.pre >= 0 ? 1 : 0) + (l.pool >= 0 ? 1 : 0);
         ++used;
         if (l.pre >= 0) {
             if (out && used < capacity) out[used] = l.pre;
@@ -476,6 +497,10 @@ int paella_model_launch_plan(const char* name, int* out, size_t capacity) {
         }
         for (int k = 0; k < l.count; ++k, ++used)
             if (out && used < capacity) out[used] = l.nodes[k];
+        if (l.pool >= 0) {
+            if (out && used < capacity) out[used] = l.pool;
+            ++used;
+        }
     }
     return (int)used;
 }
@@ -523,6 +548,7 @@ int paella_model_stage_work(const paella_model* m, int stage, const char** op, d
         f += m->plans[l.nodes[k]].flops;
         b += m->plans[l.nodes[k]].bytes;
     }
+    if (l.pool >= 0) b += m->plans[l.pool].bytes;
     if (flops) *flops = f;
     if (bytes) *bytes = b;
     return 0;
@@ -538,6 +564,10 @@ int paella_model_stage_nodes(const paella_model* m, int stage, int* nodes, int c
     }
     for (int k = 0; k < l.count; ++k, ++count)
         if (nodes && count < capacity) nodes[count] = l.nodes[k];
+    if (l.pool >= 0) {
+        if (nodes && count < capacity) nodes[count] = l.pool;
+        ++count;
+    }
     return count;
 }
 
@@ -596,13 +626,17 @@ void* paella_exec_output(paella_exec* e) { return e ? e->ptr(e->m->g.output) : n
 int paella_exec_launch_stage(paella_exec* e, int stage, void* stream, uint32_t job_id, void* notifier) {
     if (!e || stage < 0 || (size_t)stage >= e->m->stages.size()) return PAELLA_EINVAL;
     const Launch& l = e->m->stages[stage];
-    if (l.count > 1) {
+    if (l.count > 1 || l.pool >= 0) {
         paella_conv_operands members[PAELLA_CONV_GROUP_MAX];
         for (int k = 0; k < l.count; ++k) {
             const StagePlan& sk = e->m->plans[l.nodes[k]];
             const Node& nk = *sk.node;
             members[k] = paella_conv_operands{&sk.conv, e->ptr(nk.x), sk.w, sk.bias, e->ptr(nk.x2), sk.slope, e->ptr(nk.y),
                                               e->workspace ? static_cast<char*>(e->workspace) + e->m->ws_area[k] : nullptr};
+        }
+        if (l.pool >= 0) {
+            const Node& pn = e->m->g.nodes[l.pool];
+            return paella_conv2d_launch_group_pool(members, l.count, &pn.pool, e->ptr(pn.x), e->ptr(pn.y), stream, job_id, notifier);
         }
         return paella_conv2d_launch_group(members, l.count, stream, job_id, notifier);
     }

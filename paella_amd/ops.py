@@ -108,6 +108,30 @@ def conv2d_group(convs, xs, residuals=None, stream=None, job_id=0, notifier=None
     return outs
 
 
+def conv2d_group_pool(convs, xs, pool_x, k, stride, pad=0, ceil_mode=False, is_avg=False, count_include_pad=True, residuals=None,
+                      stream=None, job_id=0, notifier=None):
+    """Up to three independent Conv2d layers and one pooling operator as one launch (paella_conv2d_launch_group_pool);
+    returns the convs' outputs and the pool's."""
+    residuals = residuals or [None] * len(convs)
+    members = (ConvOperands * len(convs))()
+    outs = []
+    for i, (c, x, r) in enumerate(zip(convs, xs, residuals)):
+        members[i], y = c.operands(x, r)
+        outs.append(y)
+    lib = convs[0].lib
+    _, c, h, w = pool_x.shape
+    r, s = _pair(k)
+    sh, sw = _pair(stride)
+    ph, pw = _pair(pad)
+    d = PoolDesc(c, h, w, r, s, sh, sw, ph, pw, int(ceil_mode), int(is_avg), int(count_include_pad))
+    p = lib.paella_pool_out(h, r, sh, ph, int(ceil_mode))
+    q = lib.paella_pool_out(w, s, sw, pw, int(ceil_mode))
+    pool_y = torch.empty((1, c, p, q), device=pool_x.device, dtype=torch.float32)
+    check(lib.paella_conv2d_launch_group_pool(members, len(convs), ctypes.byref(d), _ptr(pool_x), _ptr(pool_y), _stream(stream), job_id,
+                                              notifier), "paella_conv2d_launch_group_pool")
+    return outs, pool_y
+
+
 def pair_dims(first, second):
     d = LaunchDims()
     rc = first.lib.paella_conv2d_pair_dims(ctypes.byref(first.plan), ctypes.byref(second.plan), ctypes.byref(d))

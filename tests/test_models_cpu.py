@@ -388,8 +388,11 @@ def test_launch_plan_keeps_every_dependence_of_the_graph(name):
     for e, c in absorbed.items():
         assert nodes[c]["op"] == "conv" and nodes[c]["groups"] == 1 and nodes[c]["x"] == nodes[e]["y"] and nodes[e]["x2"]["buf"] < 0
         assert nodes[e]["act"] in (0, 1), nodes[e]
+    # ... and one pooling operator may ride at the end of a launch of at most three convs
+    riding = [launch for launch in plan if len(launch) > 1 and nodes[launch[-1]]["op"] == "pool"]
+    assert all(len(launch) <= 4 for launch in riding)
     assert all(nodes[i]["op"] == "conv" and nodes[i]["groups"] == 1 for launch in plan if len(launch) > 1 and launch[0] not in absorbed
-               for i in launch)
+               for i in (launch[:-1] if launch in riding else launch))
     stage_of = {i: k for k, launch in enumerate(plan) for i in launch}
     # An absorbed operator's output is never written: its readers read its input instead, at their own position.
     readers = {e: [j for j in range(e + 1, len(nodes)) if nodes[j]["x"] == nodes[e]["y"]] for e in absorbed}
@@ -421,4 +424,5 @@ def test_launch_plan_keeps_every_dependence_of_the_graph(name):
     if name == "resnet18":
         assert [launch for launch in plan if len(launch) > 1] == [[7, 6], [12, 11], [17, 16]]  # first 3x3 of the block, then its projection
     if name in ("inception_v3", "googlenet"):
-        assert max(len(launch) for launch in plan) >= 3 and len(plan) < 0.7 * len(nodes)
+        assert max(len(launch) for launch in plan) >= 3 and len(plan) < 0.5 * len(nodes)
+        assert len(riding) >= 9   # the 3x3 pool of every inception module goes out with the module's first convs

@@ -122,6 +122,47 @@ def test_conv2d_on_transformed_input(cuda, case):
     close(two, ref)
 
 
+@pytest.mark.parametrize("n_convs,avg,kwlogs", [(3, False, (3, 3, 3)), (3, True, (2, 2, 2)), (1, False, (3,)), (2, True, (1, 1)), (1, True, (0,))])
+def test_convs_and_a_pool_in_one_launch_change_no_bit(cuda, n_convs, avg, kwlogs):
+    """An inception module's first launch: 1x1 convs and the 3x3 stride-1 pool, all reading the module's input, against the
+    same operators launched one by one (and against the oracle)."""
+    from paella_amd import ops
+    c, h, w = 192, 35, 35
+    x = rnd(1, c, h, w)
+    ks = [64, 48, 96][:n_convs]
+    convs, refs = [], []
+    for k, kwlog in zip(ks, kwlogs):
+        wt, b = rnd(k, c, 1, 1, scale=(2.0 / c) ** 0.5), rnd(k, scale=0.1)
+        convs.append(ops.Conv2d(wt, b, act=ops.ACT_RELU, in_hw=(h, w), tile_hint=(1 << 8) | (1 << 4) | kwlog))
+        refs.append(orc.conv2d(x, wt, b, act=orc.ACT_RELU))
+    xd = torch.tensor(x, device=cuda)
+    alone = [conv(xd) for conv in convs]
+    pool_alone = ops.pool2d(xd, 3, 1, pad=1, is_avg=avg, count_include_pad=False)
+    outs, pool_y = ops.conv2d_group_pool(convs, [xd] * n_convs, xd, 3, 1, pad=1, is_avg=avg, count_include_pad=False)
+    torch.cuda.synchronize()
+    for got, one, ref in zip(outs, alone, refs):
+        assert torch.equal(got, one)
+        close(got, ref)
+    assert torch.equal(pool_y, pool_alone)
+    pool_ref = orc.avgpool2d(x, 3, 1, pad=1, count_include_pad=False) if avg else orc.maxpool2d(x, 3, 1, pad=1)
+    close(pool_y, pool_ref)
+
+
+def test_convs_and_a_pool_in_one_launch_refuses_other_plans(cuda):
+    from paella_amd import ops
+    xd = torch.zeros((1, 5, 9, 11), device=cuda)
+    table_order = ops.Conv2d(rnd(7, 5, 1, 1), None, in_hw=(9, 11))     # C is no multiple of 8
+    with pytest.raises(RuntimeError):
+        ops.conv2d_group_pool([table_order], [xd], xd, 3, 1, pad=1)
+    x8 = torch.zeros((1, 8, 9, 11), device=cuda)
+    a = ops.Conv2d(rnd(8, 8, 1, 1), None, in_hw=(9, 11), tile_hint=(1 << 8) | (1 << 4) | 1)
+    b = ops.Conv2d(rnd(8, 8, 1, 1), None, in_hw=(9, 11), tile_hint=(1 << 8) | (1 << 4) | 2)   # another wave count
+    with pytest.raises(RuntimeError):
+        ops.conv2d_group_pool([a, b], [x8, x8], x8, 3, 1, pad=1)
+    with pytest.raises(RuntimeError):
+        ops.conv2d_group_pool([a, a, a, a], [x8] * 4, x8, 3, 1, pad=1)   # at most three convs beside a pool
+
+
 def test_conv2d_input_transform_is_refused_where_not_built(cuda):
     from paella_amd import ops
     x = torch.zeros((1, 5, 9, 11), device=cuda)
