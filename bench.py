@@ -240,6 +240,9 @@ def main():
                     help="also sweep full3's deficit threshold over a ResNet-18 : Inception-v3 = 0.952 : 0.048 mix and report Jain's index")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel over a 64 MiB buffer five times (reference point for memory-traffic counters)")
+    ap.add_argument("--zoo-ops", nargs="?", const="all", default=None, metavar="MODELS",
+                    help="only this: per operator family of every zoo model (or of the comma-separated ones), launches, time and rates "
+                         "of one forward pass, one launch at a time")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the isolated per-launch timing of one forward pass (the leg roofline.achieved comes from); value is null")
     args = ap.parse_args()
@@ -261,6 +264,25 @@ def main():
             _abi.check(_abi.ops().paella_copy_launch(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(y.data_ptr()), n, None, 0, None), "copy")
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"launches": 5, "kib_read_per_launch": n * 4 / 1024, "kib_written_per_launch": n * 4 / 1024}}), flush=True)
+        return
+    if args.zoo_ops:
+        # Isolated launches, so every figure contains the 4 us an empty kernel shows by these time stamps: operators
+        # that read 4.0 us are at that floor, whatever their kernels do.
+        wanted = models.names() if args.zoo_ops == "all" else args.zoo_ops.split(",")
+        table = {}
+        for m in wanted:
+            r = conv_roofline(models, hip, m, 20)
+            log("[bench] %-17s %3d launches, forward pass %7.1f us, back to back %6.0f passes/s" % (m, len(r["per_stage_us"]), r["forward_us"], r["direct_rps"]))
+            table[m] = {"launches": len(r["per_stage_us"]), "forward_us": r["forward_us"], "back_to_back_passes_per_s": r["direct_rps"], "by_op": {}}
+            for op, d in sorted(r["by_op"].items(), key=lambda kv: -kv[1]["us"]):
+                row = {"launches": d["launches"], "us": d["us"], "us_per_launch": d["us"] / d["launches"], "tflops": d["flops"] / d["us"] / 1e6,
+                       "gbytes_per_s": d["bytes"] / d["us"] / 1e3, "frac_of_fp32_mfma_peak": d["flops"] / d["us"] / 1e6 / FP32_MFMA_PEAK_TFLOPS,
+                       "frac_of_hbm_peak": d["bytes"] / d["us"] / 1e3 / 8000.0}
+                table[m]["by_op"][op] = row
+                log("[bench]     %-8s %3d launches %8.1f us (%5.2f each)  %6.2f TFLOP/s (%4.1f%% of fp32 MFMA)  %7.1f GB/s (%4.1f%% of HBM)" %
+                    (op, row["launches"], row["us"], row["us_per_launch"], row["tflops"], 100 * row["frac_of_fp32_mfma_peak"],
+                     row["gbytes_per_s"], 100 * row["frac_of_hbm_peak"]))
+        print(json.dumps({"zoo_ops": table}), flush=True)
         return
     os.environ.setdefault("LLIS_MODEL_SEED", "1")
     job = serve.job_path("tvm_" + {"mobilenetv2": "mobilenet"}.get(args.model, args.model))
