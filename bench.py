@@ -39,10 +39,12 @@ def log(*a):
 CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 7.10e6}  # 17 launches: 20 convs, 3 of them sharing a launch with another
 
 
-def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2, unfair=1e6):
+def serve_arm(serve, sched, streams, jobs, concurrency, steps, warmup, iat_us=0.0, seed=1, mem_marker=True, extra_kernels=2, unfair=1e6,
+              dist="exp", ln_sigma=2.0):
     name = "bench%d_%s_%d" % (os.getpid(), sched, int(time.time() * 1000) % 100000)
     with serve.Server(name, sched, num_streams=streams, mem_marker=mem_marker, cpu=4, extra_kernels=extra_kernels, unfair=unfair) as srv:
-        r = serve.client_run(srv.name, jobs, iat_us, concurrency, steps, warmup_jobs=warmup, seed=seed, dist="exp", pin_threads=True)
+        r = serve.client_run(srv.name, jobs, iat_us, concurrency, steps, warmup_jobs=warmup, seed=seed, dist=dist, ln_sigma=ln_sigma,
+                             pin_threads=True)
     return r
 
 
@@ -315,7 +317,7 @@ def main():
         log("[bench]   %.1f req/s with the host-to-device copy of every request's input" % pcie_inclusive)
         os.environ["PAELLA_INPUT_RESIDENT"] = "1"
 
-    arms, sweep = {}, []
+    arms, sweep, lognormal_point = {}, [], None
     if not args.no_arms:
         n_arm = max(500, args.steps // 2)
         for label, sched, streams in [("fifo_multi_stream", "fifo", args.concurrency), ("fifo2_kernel_by_kernel", "fifo2", args.num_streams),
@@ -334,6 +336,17 @@ def main():
                 point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"]}
             sweep.append(point)
             log("[bench]   poisson %.0f req/s: full3 p99 %.0f us, fifo p99 %.0f us" % (rate, point["full3"]["p99_us"], point["fifo_multi_stream"]["p99_us"]))
+        # The reference client's default arrival process is log-normal (reference app/client.cpp:133-134, sigma 1.5 or 2): one
+        # point of it at half the saturation rate -- the same mean rate as the first Poisson point, in bursts.
+        rate = 0.5 * min(value, arms["fifo_multi_stream"]["requests_per_s"])
+        point = {"offered_rps": rate, "arrivals": "log-normal, sigma 1.5"}
+        for label, sched, streams in [("full3", "full3", args.num_streams), ("fifo_multi_stream", "fifo", args.concurrency)]:
+            r = serve_arm(serve, sched, streams, jobs, args.concurrency, n_arm, args.warmup // 2, iat_us=1e6 / rate, extra_kernels=args.extra_kernels,
+                          dist="ln", ln_sigma=1.5)
+            point[label] = {"achieved_rps": r["throughput_rps"], "p50_us": r["all"]["p50"], "p99_us": r["all"]["p99"]}
+        lognormal_point = point
+        log("[bench]   log-normal arrivals, %.0f req/s: full3 p50 / p99 %.0f / %.0f us, fifo %.0f / %.0f us" %
+            (rate, point["full3"]["p50_us"], point["full3"]["p99_us"], point["fifo_multi_stream"]["p50_us"], point["fifo_multi_stream"]["p99_us"]))
 
     # The two-tenant mix of the target statement: small CNN : Inception-v3 (299x299) = 9 : 1, full3 against plain
     # multi-stream serving (fifo), first at saturation, then open-loop Poisson at fractions of the lower of the two.
@@ -530,6 +543,7 @@ def main():
         "cpu_baseline_torch": cpu_torch,
         "arms": arms,
         "poisson_sweep": sweep,
+        "lognormal_point": lognormal_point,
         "two_tenant_mix": mix,
         "other_mixes": other_mixes,
         "small_cnn_closed_loop": closed_loop,
