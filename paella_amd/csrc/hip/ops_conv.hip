@@ -577,27 +577,54 @@ struct DwArgs {
     llis::job::FinishedBlockNotifier* notifier;
 };
 
+// All taps of one output element.  With the filter size known the loads of a window leave back to back (a tap outside the
+// image reads element 0 of the channel and is replaced by zero afterwards) instead of one dependent trip to memory per tap;
+// the sum runs in the same tap order either way, and a skipped tap and an added zero give the same bits.
+template <int R, int S>
+__device__ __forceinline__ float dw_window(const DwArgs& p, const float* xc, const float* wc, float acc, int h0, int w0) {
+    float v[R * S], wt[R * S];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int h = h0 + r * p.dh, w = w0 + s * p.dw;
+            const bool ok = (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
+            const float x = xc[ok ? h * p.W + w : 0];
+            v[r * S + s] = ok ? x : 0.f;
+            wt[r * S + s] = wc[r * S + s];
+        }
+#pragma unroll
+    for (int t = 0; t < R * S; ++t) acc = fmaf(v[t], wt[t], acc);
+    return acc;
+}
+
 __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
     paella::hook_entry(p.notifier, p.job_id);
-    const int c = blockIdx.y;
-    const int pix = blockIdx.x * 256 + threadIdx.x;
     const int PQ = p.P * p.Q;
-    if (pix < PQ) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;  // over (channel, pixel): small feature maps still fill their workgroups
+    if (idx < p.C * PQ) {
+        const int c = idx / PQ;
+        const int pix = idx - c * PQ;
         const int ho = pix / p.Q;
         const int wo = pix - ho * p.Q;
         const float* xc = p.x + (size_t)c * p.H * p.W;
         const float* wc = p.w + (size_t)c * p.R * p.S;
         float acc = p.bias ? p.bias[c] : 0.f;
-        for (int r = 0; r < p.R; ++r) {
-            const int h = ho * p.sh - p.ph + r * p.dh;
-            if ((unsigned)h >= (unsigned)p.H) continue;
-            for (int s = 0; s < p.S; ++s) {
-                const int w = wo * p.sw - p.pw + s * p.dw;
-                if ((unsigned)w >= (unsigned)p.W) continue;
-                acc = fmaf(xc[(size_t)h * p.W + w], wc[r * p.S + s], acc);
+        const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
+        if (p.R == 3 && p.S == 3) {
+            acc = dw_window<3, 3>(p, xc, wc, acc, h0, w0);
+        } else {
+            for (int r = 0; r < p.R; ++r) {
+                const int h = h0 + r * p.dh;
+                if ((unsigned)h >= (unsigned)p.H) continue;
+                for (int s = 0; s < p.S; ++s) {
+                    const int w = w0 + s * p.dw;
+                    if ((unsigned)w >= (unsigned)p.W) continue;
+                    acc = fmaf(xc[(size_t)h * p.W + w], wc[r * p.S + s], acc);
+                }
             }
         }
-        const size_t o = (size_t)c * PQ + pix;
+        const size_t o = (size_t)idx;
         if (p.residual) acc += p.residual[o];
         const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
         store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
@@ -746,7 +773,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
     if (d->groups == d->C && d->K == d->C) {
         plan->kind = 1;
         plan->blob_bytes = (size_t)d->C * d->R * d->S * sizeof(float);
-        plan->dims.grid = (unsigned)(((PQ + 255) / 256) * d->C);
+        if ((double)d->C * PQ >= 2147483648.0) return PAELLA_ENOSUP;  // output elements are indexed with 32 bits
+        plan->dims.grid = (unsigned)(((size_t)d->C * PQ + 255) / 256);
         plan->dims.block = 256;
         plan->dims.lds_bytes = 0;
         plan->dims.vgprs = 32;
@@ -1003,8 +1031,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
     a.job_id = job_id;
     a.notifier = nf;
-    dim3 grid((PQ + 255) / 256, d.C);
-    paella::launch(dwconv_kernel, grid, dim3(256), 0, st, a);
+    paella::launch(dwconv_kernel, dim3(plan->dims.grid), dim3(256), 0, st, a);
     return (int)hipGetLastError();
 }
 

@@ -23,6 +23,44 @@ struct PoolArgs {
     llis::job::FinishedBlockNotifier* notifier;
 };
 
+// One window with its size known at compile time: every load of the window leaves before the first result is needed (a tap
+// outside the image reads element 0 of the channel and is ignored afterwards).  Same operations in the same order as the
+// generic loop, so the same bits.
+template <int R, int S>
+__device__ __forceinline__ float pool_window(const PoolArgs& p, const float* xc, int h0, int w0) {
+    float v[R * S];
+    bool ok[R * S];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int h = h0 + r, w = w0 + s;
+            ok[r * S + s] = (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
+            v[r * S + s] = xc[ok[r * S + s] ? h * p.W + w : 0];
+        }
+    if (p.is_avg) {
+        float acc = 0.f;
+        int valid = 0;
+#pragma unroll
+        for (int t = 0; t < R * S; ++t)
+            if (ok[t]) {
+                acc += v[t];
+                ++valid;
+            }
+        int div = valid;
+        if (p.count_include_pad) {
+            const int he = min(h0 + R, p.H + p.ph), we = min(w0 + S, p.W + p.pw);
+            div = (he - h0) * (we - w0);
+        }
+        return div ? acc / (float)div : 0.f;
+    }
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int t = 0; t < R * S; ++t)
+        if (ok[t]) m = fmaxf(m, v[t]);
+    return m;
+}
+
 // Output element number idx (channel-major, then row, then column); does nothing past the last element.
 __device__ __forceinline__ void pool_element(const PoolArgs& p, const int idx) {
     const int PQ = p.P * p.Q;
@@ -33,7 +71,11 @@ __device__ __forceinline__ void pool_element(const PoolArgs& p, const int idx) {
         const int qo = pix - po * p.Q;
         const float* xc = p.x + (size_t)c * p.H * p.W;
         const int h0 = po * p.sh - p.ph, w0 = qo * p.sw - p.pw;
-        if (p.is_avg) {
+        if (p.R == 3 && p.S == 3) {
+            store_out(p.y + idx, pool_window<3, 3>(p, xc, h0, w0));
+        } else if (p.R == 2 && p.S == 2) {
+            store_out(p.y + idx, pool_window<2, 2>(p, xc, h0, w0));
+        } else if (p.is_avg) {
             float acc = 0.f;
             int valid = 0;
             for (int r = 0; r < p.R; ++r) {
