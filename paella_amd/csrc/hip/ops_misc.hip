@@ -54,10 +54,23 @@ __global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x,
         if ((I & 3) == 0) {
             const float4* w4 = reinterpret_cast<const float4*>(wr);
             const float4* x4 = reinterpret_cast<const float4*>(x);
-            for (int i = lane; i < I / 4; i += 64) {
+            // four independent loads and sums per trip: a row of 2048 floats is two trips to memory, not eight
+            const int I4 = I / 4;
+            float a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            int i = lane;
+            for (; i + 192 < I4; i += 256) {
+                const float4 p0 = w4[i], p1 = w4[i + 64], p2 = w4[i + 128], p3 = w4[i + 192];
+                const float4 q0 = x4[i], q1 = x4[i + 64], q2 = x4[i + 128], q3 = x4[i + 192];
+                acc += p0.x * q0.x + p0.y * q0.y + p0.z * q0.z + p0.w * q0.w;
+                a1 += p1.x * q1.x + p1.y * q1.y + p1.z * q1.z + p1.w * q1.w;
+                a2 += p2.x * q2.x + p2.y * q2.y + p2.z * q2.z + p2.w * q2.w;
+                a3 += p3.x * q3.x + p3.y * q3.y + p3.z * q3.z + p3.w * q3.w;
+            }
+            for (; i < I4; i += 64) {
                 const float4 a = w4[i], b = x4[i];
                 acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
             }
+            acc = (acc + a1) + (a2 + a3);
         } else {
             for (int i = lane; i < I; i += 64) acc += wr[i] * x[i];
         }
