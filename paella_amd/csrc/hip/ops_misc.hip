@@ -256,11 +256,27 @@ __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, f
         const int i = (int)(idx - (size_t)c * HW);
         const int lo = (size - 1) / 2, hi = size - 1 - lo;
         float sq = 0.f;
-        for (int cc = max(0, c - lo); cc <= min(C - 1, c + hi); ++cc) {
-            const float v = x[(size_t)cc * HW + i];
-            sq += v * v;
+        if (size == 5) {
+            // the window the served models use: its five loads leave together (a channel outside the tensor reads the
+            // centre instead and counts as zero); same sum in the same order as the loop below
+            float v[5];
+#pragma unroll
+            for (int t = 0; t < 5; ++t) {
+                const int cc = c - 2 + t;
+                const bool ok = cc >= 0 && cc < C;
+                const float u = x[(size_t)(ok ? cc : c) * HW + i];
+                v[t] = ok ? u : 0.f;
+            }
+#pragma unroll
+            for (int t = 0; t < 5; ++t) sq += v[t] * v[t];
+            store_out(y + idx, v[2] / powf(k + alpha / (float)size * sq, beta));
+        } else {
+            for (int cc = max(0, c - lo); cc <= min(C - 1, c + hi); ++cc) {
+                const float v = x[(size_t)cc * HW + i];
+                sq += v * v;
+            }
+            store_out(y + idx, x[idx] / powf(k + alpha / (float)size * sq, beta));
         }
-        store_out(y + idx, x[idx] / powf(k + alpha / (float)size * sq, beta));
     }
     paella::hook_exit(notifier, job_id);
 }
