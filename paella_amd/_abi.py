@@ -78,6 +78,7 @@ OPS_SYMBOLS = {
     "paella_conv2d_pack": (c_int, [ctypes.POINTER(ConvPlan), c_void_p, c_void_p]),
     "paella_conv2d_launch": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 7 + _TAIL),
     "paella_conv2d_plan_takes_input_transform": (c_int, [ctypes.POINTER(ConvPlan)]),
+    "paella_conv2d_transformed_dims": (c_int, [ctypes.POINTER(ConvPlan), ctypes.POINTER(LaunchDims)]),
     "paella_conv2d_launch_transformed": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 3 + [c_int] + [c_void_p] * 6 + _TAIL),
     "paella_conv2d_pair_dims": (c_int, [ctypes.POINTER(ConvPlan), ctypes.POINTER(ConvPlan), ctypes.POINTER(LaunchDims)]),
     "paella_conv2d_launch_pair": (c_int, [ctypes.POINTER(ConvOperands), ctypes.POINTER(ConvOperands)] + _TAIL),

@@ -1053,6 +1053,18 @@ extern "C" int paella_conv2d_plan_takes_input_transform(const paella_conv_plan* 
     return plan && plan->kind == 0 && plan->mi == 1 && plan->ni == 1 && plan->k_order == 1 ? 1 : 0;
 }
 
+extern "C" int paella_conv2d_transformed_dims(const paella_conv_plan* plan, paella_launch_dims* dims) {
+    if (!plan || !dims) return PAELLA_EINVAL;
+    if (!paella_conv2d_plan_takes_input_transform(plan)) return PAELLA_ENOSUP;
+    *dims = plan->dims;
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_pre_kernel(plan->kw))) == hipSuccess && attr.numRegs > 0)
+        dims->vgprs = (unsigned)attr.numRegs;
+    else
+        (void)hipGetLastError();
+    return 0;
+}
+
 extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, const float* x, const float* in_scale, const float* in_shift,
                                                 int in_act, const void* blob_dev, const float* bias, const float* residual,
                                                 const float* slope, float* y, void* workspace, void* stream, uint32_t job_id,

@@ -275,6 +275,7 @@ void pair_up(paella_model* m) {
             if (l.pool < 0) l.dims = m->plans[l.nodes[0]].dims;
             const int pre = m->pre_of[l.nodes[0]];
             if (pre >= 0 && m->absorbed_by[pre] == l.nodes[0]) l.pre = pre;
+            if (pre >= 0) (void)paella_conv2d_transformed_dims(&m->plans[l.nodes[0]].conv, &l.dims);  // the kernel that applies it uses more registers
         } else {
             // the convs whose workgroups run longer go first: the short ones fill in behind them
             std::stable_sort(l.nodes, l.nodes + l.count, [&](int a, int b) {
