@@ -257,3 +257,43 @@ def test_garbage_and_missing_files_are_errors(tmp_path, capfd):
     with pytest.raises(RuntimeError):
         models.describe("onnx:" + str(tmp_path / "lie.onnx"))
     assert "holds" in capfd.readouterr().err
+
+
+def _bn(b, t, c):
+    return b.op("BatchNormalization", [t, b.const(b.randn(c) * 0.2 + 1.0), b.const(b.randn(c)), b.const(b.randn(c) * 0.1),
+                                       b.const(np.abs(b.randn(c)) + 0.5)], epsilon=1e-5)
+
+
+def test_norm_in_front_of_convs_is_launched_only_where_a_reader_cannot_apply_it(tmp_path):
+    """The executor drops a batch-norm (+ ReLU) stage when every reader of its output is a conv that can apply it to its own
+    input (smallest tile, input channels a multiple of 8); the launch plan lists the stage with its first reader."""
+    from paella_amd import models
+
+    def plan_of(build, c, out_c, tag):
+        b = ow.Builder(np.random.default_rng(4))
+        out = build(b)
+        path = tmp_path / (tag + ".onnx")
+        b.save(str(path), [("x", ["N", c, 9, 9])], [(out, ["N", out_c, 9, 9])], opset=11, initializers_as_inputs=False)
+        ow.check(str(path))
+        name = "onnx:" + str(path)
+        return [n["op"] for n in models.describe(name)["nodes"]], models.launch_plan(name)
+
+    conv = lambda b, t, c, k: b.op("Conv", [t, b.const(b.randn(k, c, 3, 3, scale=0.2)), b.const(b.randn(k, scale=0.1))], kernel_shape=[3, 3], pads=[1, 1, 1, 1])
+    # one reader that can
+    ops, plan = plan_of(lambda b: conv(b, b.op("Relu", [_bn(b, "x", 8)]), 8, 16), 8, 16, "one")
+    assert ops == ["eltwise", "conv"] and plan == [[0, 1]]
+    # two readers that can: listed with the first, the second stands alone and applies it too (or shares a launch with nothing)
+    def two(b):
+        t = _bn(b, "x", 8)
+        return b.op("Concat", [conv(b, t, 8, 8), conv(b, t, 8, 8)], axis=1)
+    ops, plan = plan_of(two, 8, 16, "two")
+    assert ops == ["eltwise", "conv", "conv"] and sorted(map(tuple, plan)) == [(0, 1), (2,)]
+    # the normalised tensor is also the residual of the conv: it has to exist
+    def residual(b):
+        t = _bn(b, "x", 8)
+        return b.op("Add", [conv(b, t, 8, 8), t])
+    ops, plan = plan_of(residual, 8, 8, "res")
+    assert ops == ["eltwise", "conv"] and plan == [[0], [1]]
+    # six input channels: the conv reads through the offset table, which has no transform
+    ops, plan = plan_of(lambda b: conv(b, _bn(b, "x", 6), 6, 16), 6, 16, "six")
+    assert ops == ["eltwise", "conv"] and plan == [[0], [1]]

@@ -103,3 +103,34 @@ def test_output_that_a_later_stage_reads_back_cannot_be_bound_to_host_memory(cud
     finally:
         ex.close()
         _abi.hip().llis_hip_host_free(host)
+
+
+@pytest.mark.parametrize("shared", ["two_readers", "also_residual"])
+def test_norm_shared_by_convs_matches_torch(cuda, tmp_path, shared):
+    """A batch-norm on the input read by two convs (both apply it themselves, the norm is not launched), and one that is
+    also the residual of its conv (it has to exist, so it is launched): hand-written files against torch."""
+    import torch.nn.functional as F
+    from paella_amd import models
+    b = ow.Builder(np.random.default_rng(8))
+    c = 8
+    bn = [b.randn(c) * 0.2 + 1.0, b.randn(c), b.randn(c) * 0.1, np.abs(b.randn(c)) + 0.5]
+    t = b.op("BatchNormalization", ["x"] + [b.const(a) for a in bn], epsilon=1e-5)
+    w1, b1, w2, b2 = b.randn(8, c, 3, 3, scale=0.2), b.randn(8, scale=0.1), b.randn(8, c, 3, 3, scale=0.2), b.randn(8, scale=0.1)
+    conv = lambda t, w, bias: b.op("Conv", [t, b.const(w), b.const(bias)], kernel_shape=[3, 3], pads=[1, 1, 1, 1])
+    if shared == "two_readers":
+        out, out_c = b.op("Concat", [conv(t, w1, b1), conv(t, w2, b2)], axis=1), 16
+    else:
+        out, out_c = b.op("Add", [conv(t, w1, b1), t]), 8
+    path = tmp_path / (shared + ".onnx")
+    b.save(str(path), [("x", ["N", c, 11, 13])], [(out, ["N", out_c, 11, 13])], opset=11, initializers_as_inputs=False)
+    ow.check(str(path))
+    x = torch.randn(1, c, 11, 13, generator=torch.Generator().manual_seed(3))
+    tt = lambda a: torch.tensor(np.asarray(a, np.float32))
+    n = F.batch_norm(x, tt(bn[2]), tt(bn[3]), tt(bn[0]), tt(bn[1]), False, 0.0, 1e-5)
+    if shared == "two_readers":
+        ref = torch.cat([F.conv2d(n, tt(w1), tt(b1), padding=1), F.conv2d(n, tt(w2), tt(b2), padding=1)], 1)
+    else:
+        ref = F.conv2d(n, tt(w1), tt(b1), padding=1) + n
+    plan = models.launch_plan("onnx:" + str(path))
+    assert (sorted(map(tuple, plan)) == [(0, 1), (2,)]) if shared == "two_readers" else (plan == [[0], [1]])
+    close(run_on_gpu(str(path), x.numpy()), ref.numpy(), shared)
