@@ -738,7 +738,12 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             splits = 1 << ((tile_hint >> 12) & 0xF);
         } else {
             const int cap = env_int("PAELLA_CONV_WG_CAP", 288);
-            while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= 4) splits *= 2;
+            // Layers of at most 32 tiles (DenseNet's and MobileNetV2's deep, narrow convs on 14 x 14 and 7 x 7 maps) go down to
+            // 2 chunks per wave: with four passes in flight / alone, DenseNet-121 4.09 -> 4.44 / 1.31 -> 1.38 thousand passes per
+            // second, MobileNetV2 14.5 -> 15.5 / 4.82 -> 4.91, Inception-v3 4.84 -> 4.78 / 2.33 -> 2.32, ResNet-18 and -50,
+            // GoogLeNet and SqueezeNet within the run-to-run spread; 2 everywhere costs Inception-v3 5 %.
+            const int min_chunks = n_tiles <= 32 ? 2 : 4;
+            while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= min_chunks) splits *= 2;
         }
         int chunks_per_split = (nchunks + splits - 1) / splits;
         splits = (nchunks + chunks_per_split - 1) / chunks_per_split;  // no empty split
