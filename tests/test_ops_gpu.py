@@ -373,6 +373,9 @@ def test_global_avgpool_eltwise_copy_softmax_lrn_parity(cuda):
     close(ops.softmax(torch.tensor(z, device=cuda)), orc.softmax(z))
     z2 = rnd(4420, 2, scale=3.0)
     close(ops.softmax(torch.tensor(z2, device=cuda)), orc.softmax(z2))
+    for rows, cols in [(1, 1), (257, 8), (300, 9), (5, 3)]:   # either side of the short-row kernel's limit, ragged row counts
+        z3 = rnd(rows, cols, scale=3.0)
+        close(ops.softmax(torch.tensor(z3, device=cuda)), orc.softmax(z3))
     x = rnd(1, 64, 28, 28, scale=3.0)
     close(ops.lrn(torch.tensor(x, device=cuda), 5, 1e-4, 0.75, 1.0), orc.lrn(x, 5, 1e-4, 0.75, 1.0))
     close(ops.lrn(torch.tensor(x, device=cuda), 4, 0.3, 0.6, 2.0), orc.lrn(x, 4, 0.3, 0.6, 2.0))
