@@ -5,6 +5,7 @@
 
 #include "paella_hip.h"
 
+#include <cerrno>
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -31,7 +32,14 @@ void ShmChannelBase<for_gpu>::connect(std::string name, size_t size) {
 
     if (named) {
         std::snprintf(name_, sizeof(name_), "llis:channel:%s", name.c_str());
-        fd_ = shm_open(name_, owner_ ? (O_CREAT | O_RDWR) : O_RDWR, 0600);
+        if (owner_) {
+            // A creator that died without unlinking leaves an object of this name behind (with whatever positions it
+            // held): remove it and insist on a fresh one, so nobody attaches to the stale ring.
+            if (shm_unlink(name_) != 0 && errno != ENOENT) LLIS_WARN_POSIX(-1);
+            fd_ = shm_open(name_, O_CREAT | O_EXCL | O_RDWR, 0600);
+        } else {
+            fd_ = shm_open(name_, O_RDWR, 0600);
+        }
         LLIS_CHECK_POSIX(fd_);
         if (!owner_) {
             // The creator may still be between shm_open and ftruncate: wait for a non-empty object.

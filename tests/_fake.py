@@ -22,8 +22,11 @@ def fake_job(name):
 def run_harness(script, timeout=60):
     """Runs tests/fake_device/lib/sched_harness on a scenario; returns (replies, event log text)."""
     ensure_built()
-    out = subprocess.run([os.path.join(FAKE_LIB, "sched_harness")], input=script, capture_output=True, text=True, timeout=timeout)
-    assert out.returncode == 0, out.stderr
+    # The script steps the device itself; whatever else set in this interpreter's environment (the in-process
+    # serving tests ask the scripted device for a background thread) must not reach the harness.
+    env = {k: v for k, v in os.environ.items() if not k.startswith("FAKE_HIP_")}
+    out = subprocess.run([os.path.join(FAKE_LIB, "sched_harness")], input=script, capture_output=True, text=True, timeout=timeout, env=env)
+    assert out.returncode == 0, "sched_harness exit %d\n--- stderr\n%s\n--- stdout\n%s" % (out.returncode, out.stderr, out.stdout)
     head, _, log = out.stdout.partition("--- event log\n")
     return head.splitlines(), log
 

@@ -25,6 +25,7 @@
 #include <sys/socket.h>
 #include <unistd.h>
 
+#include <csignal>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -60,7 +61,7 @@ struct Harness {
     int sock = -1;
     ClientId client_id = 0;
     std::vector<JobType> types;
-    unsigned completions = 0, wakeups = 0;
+    unsigned completions = 0, wakeups = 0, launches = 0;
 
     void poll(bool drain = true) {
         int idle = 0;
@@ -86,11 +87,33 @@ struct Harness {
     }
 };
 
+// Name of the request ring the server creates, kept for the exit paths that run no destructors.
+char g_c2s_object[128];
+
+void unlink_request_ring() {
+    if (g_c2s_object[0]) shm_unlink(g_c2s_object);
+}
+
+void on_fatal_signal(int sig) {
+    unlink_request_ring();
+    _exit(128 + sig);
+}
+
 }  // namespace
 
 int main() {
+    // The script owns the device: a background thread that completes operations on its own (what the
+    // in-process serving tests ask the scripted device for) would race every "step" of the script.
+    if (const char* autorun = std::getenv("FAKE_HIP_AUTORUN"); autorun && *autorun == '1') {
+        std::fprintf(stderr, "sched_harness: FAKE_HIP_AUTORUN=1 is set; the harness steps the device itself\n");
+        return 4;
+    }
     Harness h;
     h.server_name = "harness" + std::to_string(getpid());
+    std::snprintf(g_c2s_object, sizeof(g_c2s_object), "llis:channel:%s", ipc::c2s_channel_name(h.server_name).c_str());
+    std::atexit(unlink_request_ring);
+    std::set_terminate([] { unlink_request_ring(); std::abort(); });
+    for (int sig : {SIGTERM, SIGINT, SIGHUP, SIGSEGV, SIGABRT, SIGPIPE}) std::signal(sig, on_fatal_signal);
     std::string line;
     while (std::getline(std::cin, line)) {
         std::istringstream in(line);
@@ -171,6 +194,7 @@ int main() {
             h.c2s->write((size_t)slot * h.types[type].slot_size);
             h.c2s->write(reinterpret_cast<void*>((uintptr_t)(1000 * (type + 1) + slot)));
             h.c2s->release_writer_lock();
+            ++h.launches;
             h.poll();
         } else if (cmd == "step") {
             int n = 1;
@@ -214,5 +238,9 @@ int main() {
     std::printf("wakeups %u completions %u pending %u\n", h.wakeups, h.completions, fake_hip_pending());
     std::printf("--- event log\n");
     std::fputs(h.server->get_event_log()->to_text().c_str(), stdout);
+    if (fake_hip_pending() == 0 && h.completions != h.launches) {
+        std::fprintf(stderr, "sched_harness: device idle, but %u completions for %u launches\n", h.completions, h.launches);
+        return 3;
+    }
     return 0;
 }
