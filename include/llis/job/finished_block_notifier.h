@@ -31,19 +31,26 @@ namespace job {
 
 class FinishedBlockNotifier {
   public:
-    // Workgroups per message.  The reference batches 16 on a 40-SM GPU (reference
-    // include/llis/job/finished_block_notifier.h:118); 64 keeps a comparable share of a 256-CU device per
-    // message and quarters the host's message rate.  Grids of up to 64 workgroups send exactly one start
-    // and one end message either way.
+    // Workgroups per message: a property of each notifier, fixed when it is created (create_array), a power of two
+    // of at most 128 (`num` travels in one byte).  The reference batches 16 on a 40-SM GPU (reference
+    // include/llis/job/finished_block_notifier.h:118) and that value is reference_noti_batch_size; the default,
+    // 64, keeps a comparable share of a 256-CU device per message and quarters the host's message rate.  Grids of
+    // up to 16 workgroups send exactly one start and one end message either way.
     static constexpr unsigned noti_batch_size = 64;
+    static constexpr unsigned reference_noti_batch_size = 16;
+    static constexpr unsigned max_noti_batch_size = 128;
+
+    static constexpr bool valid_batch_size(unsigned b) { return b != 0 && b <= max_noti_batch_size && (b & (b - 1)) == 0; }
 
     FinishedBlockNotifier() {}
-    explicit FinishedBlockNotifier(ipc::Gpu2SchedChannel* gpu2sched_channel, ipc::Gpu2SchedChannel* block_time_channel = nullptr) {
+    explicit FinishedBlockNotifier(ipc::Gpu2SchedChannel* gpu2sched_channel, ipc::Gpu2SchedChannel* block_time_channel = nullptr,
+                                   unsigned batch_size = noti_batch_size) {
         gpu2sched_channel_ = gpu2sched_channel->fork();
         if (block_time_channel) {
             block_time_channel_ = block_time_channel->fork();
             measure_block_time_ = 1;
         }
+        batch_mask_ = (valid_batch_size(batch_size) ? batch_size : noti_batch_size) - 1;
     }
     FinishedBlockNotifier(FinishedBlockNotifier&&) = default;
     FinishedBlockNotifier& operator=(FinishedBlockNotifier&&) = default;
@@ -98,9 +105,11 @@ class FinishedBlockNotifier {
 #endif
 
     // Allocates `num` notifiers in device memory, all bound to the given ring (and, when given, to the ring
-    // that receives per-workgroup timing samples).
+    // that receives per-workgroup timing samples), sending one message per `batch_size` workgroups; a batch size
+    // that is no power of two in 1..128 is an error (std::invalid_argument).
     static FinishedBlockNotifier* create_array(unsigned num, ipc::Gpu2SchedChannel* gpu2sched_channel,
-                                               ipc::Gpu2SchedChannel* block_time_channel = nullptr);
+                                               ipc::Gpu2SchedChannel* block_time_channel = nullptr,
+                                               unsigned batch_size = noti_batch_size);
     static void free_array(FinishedBlockNotifier* ptr);
 
   private:
@@ -125,11 +134,12 @@ class FinishedBlockNotifier {
     template <bool ACQUIRE>
     __device__ __forceinline__ void announce(unsigned* counter, uint8_t is_start, JobId job_id) {
         const unsigned num_blocks = gridDim.x * gridDim.y * gridDim.z;
+        const unsigned mask = batch_mask_;  // requested before the atomic, so the two trips to memory overlap
         const unsigned total = atomicInc(counter, num_blocks - 1) + 1;  // wraps to 0 after the last block
-        const unsigned in_batch = total % noti_batch_size;
+        const unsigned in_batch = total & mask;
         unsigned covered = 0;
         if (in_batch == 0) {
-            covered = noti_batch_size;
+            covered = mask + 1;
         } else if (total == num_blocks) {
             covered = in_batch;
         }
@@ -149,6 +159,7 @@ class FinishedBlockNotifier {
     ipc::Gpu2SchedChannel gpu2sched_channel_;
     ipc::Gpu2SchedChannel block_time_channel_;
     unsigned measure_block_time_ = 0;
+    unsigned batch_mask_ = noti_batch_size - 1;
     // ... and, on a cache line of their own, the counters every workgroup bumps atomically: a load of the
     // fields above must not queue behind those atomics.
     alignas(128) unsigned agg_counter_start_ = 0;

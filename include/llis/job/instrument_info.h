@@ -2,7 +2,7 @@
 // The 8-byte message a workgroup sends to the scheduler.  Bit layout (little endian, one ring slot):
 //   byte 0  is_start   1 = workgroups became resident, 0 = workgroups finished, 2 = a copy stage finished
 //   byte 1  smid       compute-unit id of the sender (un-aggregated hooks only)
-//   byte 2  num        how many workgroups this message accounts for (1..16)
+//   byte 2  num        how many workgroups this message accounts for (1..batch size of the sending notifier, at most 128; 16 in the reference)
 //   byte 3  status     1 = slot holds an unread message, 0 = consumed
 //   byte 4-7 job_id
 // Layout and accessor names follow reference include/llis/job/instrument_info.h:9-38; the value 2 of

@@ -39,6 +39,9 @@ struct SchedulerOptions {
     // --measure_block_time: every workgroup also reports its entry and exit clock through a second ring; the
     // profiler keeps the pairs while block-exec-time recording is on (reference: compile-time LLIS_MEASURE_BLOCK_TIME).
     bool measure_block_time = false;
+    // --noti_batch: workgroups covered by one aggregated notification (a power of two, at most 128).  0 = the
+    // library's default of 64; 16 is the reference's constant (reference include/llis/job/finished_block_notifier.h:118).
+    unsigned noti_batch = 0;
 };
 
 class Scheduler {

@@ -202,6 +202,16 @@ int paella_kernel_vgprs(const char* family, unsigned* vgprs);
 /* Same for a conv variant: kind 0 = MFMA implicit GEMM with tile (mi, ni, kw), kind 1 = depthwise. */
 int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs);
 
+/* Workgroups of a kernel that the runtime's occupancy calculator places on one compute unit, for a workgroup of
+ * `block` threads with `lds_bytes` of dynamic LDS (needs a GPU).  What the block-level scheduler's resource model
+ * (llis::server::SmResources::blocks_per_cu; the reference's counterpart is the budget arithmetic of
+ * src/server/sm_resources.cpp:17-66) is checked against.  `form` of a conv: 0 = one conv, 1 = conv on a transformed
+ * input, 2 = group of convs, 3 = group of convs with a pooling operator (forms 1 to 3: mi == ni == 1; 1 and 3: k_order 1). */
+int paella_kernel_occupancy(const char* family, unsigned block, unsigned lds_bytes, int* blocks_per_cu);
+/* vgprs (may be NULL): vector registers per thread of that same kernel, read from the loaded code object. */
+int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, int kw, int k_order, unsigned lds_bytes, int* blocks_per_cu,
+                                 unsigned* vgprs);
+
 /*
  * Direct dispatch.  A queue created here is a user-mode hardware queue owned by this library; its handle can
  * be passed wherever a launch function of this header (or paella_exec_launch_stage / paella_exec_forward)

@@ -26,11 +26,15 @@ extern "C" {
 
 typedef struct paella_ring paella_ring;
 
-/* Workgroups covered by one aggregated message (llis::job::FinishedBlockNotifier::noti_batch_size). */
+/* Workgroups covered by one aggregated message when nothing else is asked for
+ * (llis::job::FinishedBlockNotifier::noti_batch_size; the reference's constant is 16,
+ * reference include/llis/job/finished_block_notifier.h:118). */
 unsigned paella_ring_batch_size(void);
 
 /* A ring of `slots` 64-bit slots in coherent host memory plus `num_notifiers` device-resident notifiers. */
 int paella_ring_create(size_t slots, unsigned num_notifiers, paella_ring** out);
+/* The same with notifiers that send one message per `batch` workgroups (a power of two, at most 128; else -1). */
+int paella_ring_create_batched(size_t slots, unsigned num_notifiers, unsigned batch, paella_ring** out);
 int paella_ring_destroy(paella_ring* ring);
 /* Device pointer to notifier `idx` (an llis::job::FinishedBlockNotifier*). */
 void* paella_ring_notifier(paella_ring* ring, unsigned idx);

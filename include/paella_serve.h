@@ -35,6 +35,8 @@ typedef struct paella_server_options {
     int event_log;             /* 1: record the scheduler event log */
     int cpu;                   /* pin the serving thread to this CPU, -1 = do not pin */
     int measure_block_time;    /* 1: --measure_block_time (per-workgroup entry/exit clocks for the profiler) */
+    unsigned noti_batch;       /* --noti_batch: workgroups per aggregated notification, a power of two <= 128; 0 = default (64);
+                                  16 = the reference's constant (reference include/llis/job/finished_block_notifier.h:118) */
 } paella_server_options;
 
 int paella_server_start(const paella_server_options* options, paella_server** out);

@@ -151,13 +151,42 @@ class JobQueue:
         return entry[2]
 
 
+WAVE_LANES, VGPR_GRANULE, LDS_GRANULE = 64, 8, 1280  # gfx950 allocation units (include/llis/server/sm_resources.h)
+SIMDS_PER_CU, VGPRS_PER_SIMD_LANE, MAX_WAVES_PER_SIMD = 4, 512, 8
+
+
+def _up(v, g):
+    return -(-v // g) * g
+
+
+def wg_charge(st):
+    """(register lanes, LDS bytes, wave-slot threads) one workgroup of the stage takes: whole waves, registers in
+    granules of 8 per lane, LDS in granules of 1280 bytes.  The pooling is reference src/server/sm_resources.cpp:36-66;
+    the reference charges the declared regs x threads, threads and bytes (the CUDA allocation model)."""
+    thr = _up(st.threads, WAVE_LANES)
+    return thr * _up(st.regs, VGPR_GRANULE), _up(st.smem, LDS_GRANULE), thr
+
+
+def blocks_per_cu(threads, regs, smem, lds_per_cu=160 * 1024, max_blocks=32):
+    """Workgroups of one shape a gfx950 compute unit holds: the closed form the runtime's occupancy query follows."""
+    if threads == 0:
+        return 0
+    waves_per_wg = _up(threads, WAVE_LANES) // WAVE_LANES
+    per_simd = MAX_WAVES_PER_SIMD if regs == 0 else min(MAX_WAVES_PER_SIMD, VGPRS_PER_SIMD_LANE // _up(regs, VGPR_GRANULE))
+    n = SIMDS_PER_CU * per_simd // waves_per_wg
+    if smem > 0:
+        n = min(n, lds_per_cu // _up(smem, LDS_GRANULE))
+    return max(min(n, max_blocks), 0)
+
+
 class SmResources:
     def __init__(self, regs, smem, threads, blocks):
         self.free = [regs, smem, threads, blocks]
 
     @staticmethod
     def _need(st, n):
-        return [st.regs * st.threads * n, st.smem * n, st.threads * n, n]
+        r, s, t = wg_charge(st)
+        return [r * n, s * n, t * n, n]
 
     def fits(self, st):
         return all(f >= need for f, need in zip(self.free, self._need(st, st.blocks)))
@@ -192,12 +221,13 @@ class GpuResources:
         if GpuResources._full(r):
             return 0
         n = r.free[3]
+        regs, smem, thr = wg_charge(st)
         if st.threads > 0:
-            if st.regs * st.threads > 0:
-                n = min(n, r.free[0] // (st.regs * st.threads))
-            n = min(n, r.free[2] // st.threads)
+            if regs > 0:
+                n = min(n, r.free[0] // regs)
+            n = min(n, r.free[2] // thr)
         if st.smem > 0:
-            n = min(n, r.free[1] // st.smem)
+            n = min(n, r.free[1] // smem)
         return max(n, 0)
 
     def num_full(self):

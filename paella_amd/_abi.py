@@ -103,6 +103,8 @@ OPS_SYMBOLS = {
     "paella_lrn_launch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_float] + _TAIL),
     "paella_kernel_vgprs": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv_kernel_vgprs": (c_int, [c_int] * 4 + [ctypes.POINTER(c_uint)]),
+    "paella_kernel_occupancy": (c_int, [c_char_p, c_uint, c_uint, ctypes.POINTER(c_int)]),
+    "paella_conv_kernel_occupancy": (c_int, [c_int] * 6 + [c_uint, ctypes.POINTER(c_int), ctypes.POINTER(c_uint)]),
     "paella_ops_time_launches": (c_int, [c_void_p, c_void_p]),
     "paella_direct_queue_create": (c_int, [ctypes.POINTER(c_void_p)]),
     "paella_direct_queue_set_ordered": (c_int, [c_void_p, c_int]),
@@ -114,6 +116,7 @@ OPS_SYMBOLS = {
 RING_SYMBOLS = {
     "paella_ring_batch_size": (c_uint, []),
     "paella_ring_create": (c_int, [c_size_t, c_uint, ctypes.POINTER(c_void_p)]),
+    "paella_ring_create_batched": (c_int, [c_size_t, c_uint, c_uint, ctypes.POINTER(c_void_p)]),
     "paella_ring_destroy": (c_int, [c_void_p]),
     "paella_ring_notifier": (c_void_p, [c_void_p, c_uint]),
     "paella_ring_channel": (c_void_p, [c_void_p]),

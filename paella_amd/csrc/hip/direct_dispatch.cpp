@@ -155,15 +155,6 @@ bool ensure_runtime() {
     return g_rt.ok;
 }
 
-int fence_scope_from_env(const char* name, int fallback) {
-    const char* v = std::getenv(name);
-    if (!v) return fallback;
-    if (!std::strcmp(v, "none")) return HSA_FENCE_SCOPE_NONE;
-    if (!std::strcmp(v, "agent")) return HSA_FENCE_SCOPE_AGENT;
-    if (!std::strcmp(v, "system")) return HSA_FENCE_SCOPE_SYSTEM;
-    return fallback;
-}
-
 void queue_error(hsa_status_t status, hsa_queue_t*, void*) {
     const char* msg = nullptr;
     hsa_status_string(status, &msg);
@@ -288,9 +279,9 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     // Header and setup share the packet's first 32 bits and are published last, with release semantics.
     // Acquire at agent scope: a kernel must not see stale lines of buffers that earlier kernels (on other XCDs)
     // or copies rewrote.  No release: operator kernels write their results through to memory and report
-    // completion themselves, before the packet retires.  Both can be overridden for experiments.
-    static const int acq = fence_scope_from_env("PAELLA_DIRECT_ACQUIRE", HSA_FENCE_SCOPE_AGENT);
-    static const int rel = fence_scope_from_env("PAELLA_DIRECT_RELEASE", HSA_FENCE_SCOPE_NONE);
+    // completion themselves, before the packet retires.
+    constexpr int acq = HSA_FENCE_SCOPE_AGENT;
+    constexpr int rel = HSA_FENCE_SCOPE_NONE;
     const uint16_t header = (uint16_t)((HSA_PACKET_TYPE_KERNEL_DISPATCH << HSA_PACKET_HEADER_TYPE) |
                                        (acq << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
                                        (rel << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE) |
@@ -340,7 +331,7 @@ extern "C" int paella_direct_queue_create(void** out) {
     st = HSA_STATUS_ERROR;
     // Kernel arguments in device memory (written by the host through the PCIe aperture): every wave of a kernel
     // reads them, and fetching them from host memory instead costs about 10 us per kernel on an idle GPU.
-    if (paella::g_rt.have_device_pool && !std::getenv("PAELLA_DIRECT_HOST_KERNARG")) {
+    if (paella::g_rt.have_device_pool) {
         st = hsa_amd_memory_pool_allocate(paella::g_rt.device_pool, ka_bytes, 0, &ka);
         if (st == HSA_STATUS_SUCCESS) st = hsa_amd_agents_allow_access(1, &paella::g_rt.cpu, nullptr, ka);
         if (st != HSA_STATUS_SUCCESS && ka) {

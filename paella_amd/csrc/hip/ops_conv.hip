@@ -35,21 +35,6 @@
 #include "out_store.h"
 #include "pool_body.h"
 
-// Build-time diagnostic (never defined in the shipped library): thread 0 of every workgroup records the
-// 100 MHz wall clock at a few points of the kernel.
-#ifdef PAELLA_CONV_TIMELINE
-__device__ unsigned long long g_conv_timeline[8192 * 12];
-#define CONV_TL(i)                                                                                        \
-    do {                                                                                                  \
-        if (threadIdx.x == 0) {                                                                           \
-            const unsigned b_ = blockIdx.x;                                                               \
-            if (b_ < 8192) g_conv_timeline[b_ * 12 + (i)] = wall_clock64();                               \
-        }                                                                                                 \
-    } while (0)
-#else
-#define CONV_TL(i)
-#endif
-
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -120,24 +105,10 @@ struct PreOp {
     float lo;
 };
 
-// Build-time diagnostic: -DPAELLA_CONV_ABLATE=<bits> removes parts of the kernel to see what bounds it
-// (1 = no MFMA, 2 = no operand loads, 4 = no cross-wave reduction, 8 = no table build, 16 = empty kernel, 32 = no epilogue).  Results are wrong.
-#ifndef PAELLA_CONV_ABLATE
-#define PAELLA_CONV_ABLATE 0
-#endif
-#ifndef PAELLA_CONV_DEPTH
-#define PAELLA_CONV_DEPTH 2
-#endif
-#ifndef PAELLA_CONV_MINB
-#define PAELLA_CONV_MINB 1
-#endif
-
 // One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
 template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
-    CONV_TL(0);
-    if (PAELLA_CONV_ABLATE & 16) return;
     paella::hook_entry(p.notifier, p.job_id);
 
     // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
@@ -223,7 +194,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         st_s = tap - st_r * p.S;
     }
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
-        if (PAELLA_CONV_ABLATE & 2) valid = false;
         const int woff = valid ? (int)((((unsigned)(c * 2 + kk) * (unsigned)p.m_pad) + (unsigned)(m0 + j)) * 16u) : -1;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
@@ -278,7 +248,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // Build this workgroup's slice of the k -> offset table in LDS (a few entries per thread, arithmetic only).
     if (!TAP_MAJOR) {
         const int n_entries = (g_end - g_begin) * 8;
-        for (int i = threadIdx.x; i < ((PAELLA_CONV_ABLATE & 8) ? 0 : n_entries); i += 64 * KW) {
+        for (int i = threadIdx.x; i < n_entries; i += 64 * KW) {
             const int k = g_begin * 8 + i;
             const int c = k / p.RS;
             const int rem = k - c * p.RS;
@@ -296,7 +266,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // store still pending the compiler must assume out-of-order completion and would make every wait in
     // the pipelined loop below a full vmcnt(0).
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
-    CONV_TL(1);
 
     // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
     // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
@@ -332,7 +301,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // chunk's matrix instructions were no better either (23.8 against 24.9 TFLOP/s over a ResNet-18 pass): the loop is
     // bound by what the compute unit's vector cache can take in -- each wave fetches its own 32 x 8 operand
     // fragments, 147 KB per workgroup for a 64-channel 3x3 layer -- not by exposed latency.
-    constexpr int D = (MI * NI == 1) ? PAELLA_CONV_DEPTH : 4;
+    constexpr int D = (MI * NI == 1) ? 2 : 4;
     auto compute = [&](const Frag<MI, NI>& f) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -347,8 +316,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                         const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
                         bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
                     }
-                    if (PAELLA_CONV_ABLATE & 1) acc[mi][ni][t] += av * bv;
-                    else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
                 }
             }
         }
@@ -362,7 +330,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
         }
-        CONV_TL(2);
         const int n = c_end - c_begin;
         const int c_main_end = c_begin + (n / D) * D;
         // Branch-free steady state: whole groups of D chunks.
@@ -384,7 +351,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             if (d < rest) compute(frag[d]);
     }
 
-    CONV_TL(3);
     // Finishes the wave's RPW outputs.  Every operand load comes first, then the arithmetic, then the stores back
     // to back: a load between two stores would make the compiler wait for the earlier store as well (one counter
     // covers both), and a write-through store takes about 0.3 us to be acknowledged.
@@ -415,7 +381,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     };
 
     float mine[RPW];
-    if (KW == 1 || (PAELLA_CONV_ABLATE & 4)) {
+    if (KW == 1) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -442,11 +408,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
     }
 
-    CONV_TL(4);
-    if (PAELLA_CONV_ABLATE & 32) {
-        if (mine[0] == 12345.f) p.y[0] = 0.f;
-        return;
-    }
     if (p.splits == 1) {
         epilogue_all(mine);
     } else {
@@ -459,11 +420,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         for (int rr = 0; rr < RPW; ++rr) store_out(part + (wave * RPW + rr) * 64 + lane, mine[rr]);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        CONV_TL(5);
         __shared__ unsigned arrived;
         if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(p.ws_counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        CONV_TL(6);
         if (arrived == (unsigned)p.splits - 1) {
             const float* all = p.ws_partials + (size_t)tile * p.splits * (NACC * 64) + (size_t)(wave * RPW) * 64 + lane;
             float v[RPW];
@@ -489,16 +448,11 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
     }
 
-    CONV_TL(7);
     paella::hook_exit(p.notifier, p.job_id);
-#ifdef PAELLA_CONV_TIMELINE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    CONV_TL(8);
-#endif
 }
 
 template <int MI, int NI, int KW, bool TAP_MAJOR>
-__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? PAELLA_CONV_MINB : 1) void conv_mfma_kernel(ConvArgs p) {
+__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? 1 : 1) void conv_mfma_kernel(ConvArgs p) {
     conv_tile<MI, NI, KW, TAP_MAJOR>(p, blockIdx.x);
 }
 
@@ -509,7 +463,7 @@ struct ConvPreArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_pre_kernel(ConvPreArgs a) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_kernel(ConvPreArgs a) {
     conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
 }
 
@@ -526,7 +480,7 @@ struct ConvGroupArgs {
 };
 
 template <int KW, bool TAP_MAJOR>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
     int idx = 0;
 #pragma unroll
     for (int i = 1; i < kMaxGroup; ++i)
@@ -547,7 +501,7 @@ struct ConvGroupPoolArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? PAELLA_CONV_MINB : 1) void conv_mfma_group_pool_kernel(ConvGroupPoolArgs g) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_pool_kernel(ConvGroupPoolArgs g) {
     if (blockIdx.x >= g.pool_start) {
         paella::hook_entry(g.pool.notifier, g.pool.job_id);
         paella::pool_element(g.pool, (int)((blockIdx.x - g.pool_start) * (64 * KW) + threadIdx.x));
@@ -669,11 +623,6 @@ FastDiv fast_div(unsigned d) {
     return FastDiv{(unsigned)((((uint64_t)1) << 32) / d + 1), 0u};
 }
 
-int env_int(const char* name, int fallback) {
-    const char* v = std::getenv(name);
-    return v && *v ? std::atoi(v) : fallback;
-}
-
 }  // namespace
 
 extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, int tile_hint, paella_conv_plan* plan) {
@@ -723,21 +672,21 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             // reuse (ResNet-18, thousand passes per second, four queues / one): 32 x 32 everywhere 15.8 / 7.0; 64 x 32 where
             // K is a multiple of 64: 12.1 / 4.9, only from K = 256: 13.2 / 5.6; 32 x 64 on the 56 x 56 layers: 14.4 / 6.4.
             // (at most 4 where the reduction goes through the offset table -- stems: 7.8 against 7.9 us, 4.4 against 4.7)
-            const int kw_max = d->C % 8 == 0 ? env_int("PAELLA_CONV_KW", 8) : 4;
+            const int kw_max = d->C % 8 == 0 ? 8 : 4;
             kw = 2;
             while (kw < kw_max && kw < nchunks) kw <<= 1;
         }
         // Grid-level split of the reduction: layers with few output tiles (small feature maps) would otherwise
         // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU, keep >= 4 chunks per wave.
         // Measured on ResNet-18 with four passes in flight / one pass alone (thousand passes per second), by the cap
-        // on workgroups (PAELLA_CONV_WG_CAP) and the waves per workgroup (PAELLA_CONV_KW): 288 x 8: 15.2 / 6.9;
+        // on workgroups and the waves per workgroup: 288 x 8: 15.2 / 6.9;
         // 288 x 4: 14.5 / 6.1; 144 x 8: 13.7 / 6.1; 144 x 4: 11.9 / 5.1; 576 x 8: 13.8 / 6.0.
         const int n_tiles = tiles(mi, ni);
         int splits = 1;
         if (tile_hint > 0) {
             splits = 1 << ((tile_hint >> 12) & 0xF);
         } else {
-            const int cap = env_int("PAELLA_CONV_WG_CAP", 288);
+            const int cap = 288;
             // Layers of at most 32 tiles (DenseNet's and MobileNetV2's deep, narrow convs on 14 x 14 and 7 x 7 maps) go down to
             // 2 chunks per wave: with four passes in flight / alone, DenseNet-121 4.09 -> 4.44 / 1.31 -> 1.38 thousand passes per
             // second, MobileNetV2 14.5 -> 15.5 / 4.82 -> 4.91, Inception-v3 4.84 -> 4.78 / 2.33 -> 2.32, ResNet-18 and -50,
@@ -754,12 +703,10 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->m_pad = round_up(d->K, 32 * mi);
         plan->k_pad = k_pad;
         // Reduction order: (r, s, c) when whole chunks of 8 share a filter tap, else (c, r, s) with the offset table.
-        plan->k_order = (d->C % 8 == 0 && !std::getenv("PAELLA_CONV_NO_TAP_MAJOR")) ? 1 : 0;
+        plan->k_order = d->C % 8 == 0 ? 1 : 0;
         // Which workgroups share an XCD.  Weights outweigh the input: those that read one slab of weights; else neighbouring pixels.
         plan->wg_order = (double)d->K * d->C * d->R * d->S > (double)d->C * d->H * d->W ? 1 : 0;
-        if (const char* force = std::getenv("PAELLA_CONV_ORDER"))
-            plan->wg_order = force[0] == 's' ? 1 : (force[0] == 'n' ? 0 : (force[0] == 'i' ? 2 : plan->wg_order));
-        plan->fast_div = std::getenv("PAELLA_CONV_NO_FAST_DIV") ? 0 : 1;
+        plan->fast_div = 1;
         plan->blob_bytes = (size_t)(k_pad / 4) * plan->m_pad * sizeof(float4);
         if (plan->blob_bytes >= ((size_t)1 << 31)) return PAELLA_ENOSUP;  // weights are addressed with 32-bit byte offsets
         // Workspace = fixed-size counter area (so that stages of one request, which share the workspace, never
@@ -1089,6 +1036,31 @@ extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, co
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
     paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();
+}
+
+extern "C" int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, int kw, int k_order, unsigned lds_bytes, int* blocks_per_cu,
+                                            unsigned* vgprs) {
+    if (!blocks_per_cu) return PAELLA_EINVAL;
+    const void* fn = nullptr;
+    unsigned block = 64u * (unsigned)kw;
+    if (kind == 1) {
+        fn = reinterpret_cast<const void*>(dwconv_kernel);
+        block = 256;
+    } else if (form == 0) {
+        fn = reinterpret_cast<const void*>(pick_kernel(mi, ni, kw, k_order));
+    } else if (mi == 1 && ni == 1) {
+        if (form == 1 && k_order == 1) fn = reinterpret_cast<const void*>(pick_pre_kernel(kw));
+        else if (form == 2) fn = reinterpret_cast<const void*>(pick_group_kernel(kw, k_order));
+        else if (form == 3 && k_order == 1) fn = reinterpret_cast<const void*>(pick_group_pool_kernel(kw));
+    }
+    if (!fn) return PAELLA_EINVAL;
+    if (int rc = allow_lds(fn, lds_bytes)) return rc;
+    if (vgprs) {
+        hipFuncAttributes attr;
+        if (hipError_t e = hipFuncGetAttributes(&attr, fn)) return (int)e;
+        *vgprs = (unsigned)attr.numRegs;
+    }
+    return (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, fn, (int)block, lds_bytes);
 }
 
 extern "C" int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs) {

@@ -475,16 +475,29 @@ int paella_ops_time_launches(void* start_event, void* stop_event) {
     return 0;
 }
 
+static const void* family_kernel(const char* family) {
+    if (!std::strcmp(family, "dense")) return (const void*)dense_kernel;
+    if (!std::strcmp(family, "dense_long")) return (const void*)dense_long_kernel;
+    if (!std::strcmp(family, "pool")) return (const void*)pool_kernel;
+    if (!std::strcmp(family, "gap")) return (const void*)gap_kernel;
+    if (!std::strcmp(family, "eltwise")) return (const void*)eltwise_kernel<true>;
+    if (!std::strcmp(family, "copy")) return (const void*)copy_kernel;
+    if (!std::strcmp(family, "softmax")) return (const void*)softmax_kernel;
+    if (!std::strcmp(family, "softmax_short")) return (const void*)softmax_short_kernel;
+    if (!std::strcmp(family, "lrn")) return (const void*)lrn_kernel;
+    return nullptr;
+}
+
+int paella_kernel_occupancy(const char* family, unsigned block, unsigned lds_bytes, int* blocks_per_cu) {
+    if (!family || !blocks_per_cu || block == 0) return PAELLA_EINVAL;
+    const void* fn = family_kernel(family);
+    if (!fn) return PAELLA_EINVAL;
+    return (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, fn, (int)block, lds_bytes);
+}
+
 int paella_kernel_vgprs(const char* family, unsigned* vgprs) {
     if (!family || !vgprs) return PAELLA_EINVAL;
-    const void* fn = nullptr;
-    if (!std::strcmp(family, "dense")) fn = (const void*)dense_kernel;
-    else if (!std::strcmp(family, "pool")) fn = (const void*)pool_kernel;
-    else if (!std::strcmp(family, "gap")) fn = (const void*)gap_kernel;
-    else if (!std::strcmp(family, "eltwise")) fn = (const void*)eltwise_kernel<true>;
-    else if (!std::strcmp(family, "copy")) fn = (const void*)copy_kernel;
-    else if (!std::strcmp(family, "softmax")) fn = (const void*)softmax_kernel;
-    else if (!std::strcmp(family, "lrn")) fn = (const void*)lrn_kernel;
+    const void* fn = family_kernel(family);
     if (!fn) return PAELLA_EINVAL;
     hipFuncAttributes attr;
     hipError_t e = hipFuncGetAttributes(&attr, fn);

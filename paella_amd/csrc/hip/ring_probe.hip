@@ -115,12 +115,16 @@ extern "C" {
 unsigned paella_ring_batch_size(void) { return FinishedBlockNotifier::noti_batch_size; }
 
 int paella_ring_create(size_t slots, unsigned num_notifiers, paella_ring** out) {
-    if (!out || slots == 0) return -1;
+    return paella_ring_create_batched(slots, num_notifiers, FinishedBlockNotifier::noti_batch_size, out);
+}
+
+int paella_ring_create_batched(size_t slots, unsigned num_notifiers, unsigned batch, paella_ring** out) {
+    if (!out || slots == 0 || !FinishedBlockNotifier::valid_batch_size(batch)) return -1;
     try {
         paella_ring* r = new paella_ring();
         r->channel.connect(std::string(), slots);
         r->num_notifiers = num_notifiers;
-        if (num_notifiers) r->notifiers = FinishedBlockNotifier::create_array(num_notifiers, &r->channel);
+        if (num_notifiers) r->notifiers = FinishedBlockNotifier::create_array(num_notifiers, &r->channel, nullptr, batch);
         r->scratch_len = 1u << 20;
         void* p = nullptr;
         int rc = llis_hip_device_malloc(&p, r->scratch_len * sizeof(float));

@@ -48,6 +48,7 @@ int paella_server_start(const paella_server_options* o, paella_server** out) {
         so.sched_sleep = o->sched_sleep;
         so.mem_marker = o->mem_marker != 0;
         so.measure_block_time = o->measure_block_time != 0;
+        so.noti_batch = o->noti_batch;
         auto s = std::make_unique<paella_server>();
         s->scheduler = llis::server::SchedulerFactory::create(o->sched, so);
         s->server = std::make_unique<llis::server::Server>(o->name, s->scheduler.get());

@@ -1,5 +1,5 @@
 // llis_server --name NAME --sched {fifo,fifo2,full3} [--num_streams N] [--extra_kernels N] [--unfair X]
-//             [--sched_sleep N] [--mem_notify {marker,hostfunc}] [--device N] [--measure_block_time]
+//             [--sched_sleep N] [--mem_notify {marker,hostfunc}] [--device N] [--measure_block_time] [--noti_batch N]
 // Same options and defaults as reference src/server/server.cpp:203-235; an unknown scheduler name is an
 // error with the list of known ones instead of a null dereference.
 
@@ -19,7 +19,7 @@
 static void usage(const char* argv0) {
     std::fprintf(stderr,
                  "usage: %s --name NAME --sched {fifo,fifo2,full3} [--num_streams 500] [--extra_kernels 2]\n"
-                 "          [--unfair 1000000] [--sched_sleep 0] [--mem_notify marker|hostfunc] [--device 0] [--measure_block_time]\n",
+                 "          [--unfair 1000000] [--sched_sleep 0] [--mem_notify marker|hostfunc] [--device 0] [--measure_block_time] [--noti_batch 64]\n",
                  argv0);
 }
 
@@ -32,7 +32,8 @@ int main(int argc, char** argv) {
                                        {"sched", required_argument, nullptr, 's'},   {"num_streams", required_argument, nullptr, 't'},
                                        {"extra_kernels", required_argument, nullptr, 'e'}, {"unfair", required_argument, nullptr, 'u'},
                                        {"sched_sleep", required_argument, nullptr, 'p'},   {"mem_notify", required_argument, nullptr, 'm'},
-                                       {"device", required_argument, nullptr, 'd'},  {"measure_block_time", no_argument, nullptr, 'B'},  {nullptr, 0, nullptr, 0}};
+                                       {"device", required_argument, nullptr, 'd'},  {"measure_block_time", no_argument, nullptr, 'B'},
+                                       {"noti_batch", required_argument, nullptr, 'b'},  {nullptr, 0, nullptr, 0}};
     for (int c; (c = getopt_long(argc, argv, "h", long_opts, nullptr)) != -1;) {
         switch (c) {
             case 'n': name = optarg; break;
@@ -48,6 +49,7 @@ int main(int argc, char** argv) {
                 break;
             case 'd': device = std::atoi(optarg); break;
             case 'B': opts.measure_block_time = true; break;
+            case 'b': opts.noti_batch = (unsigned)std::strtoul(optarg, nullptr, 10); break;
             default: usage(argv[0]); return c == 'h' ? 1 : 2;
         }
     }

@@ -51,7 +51,8 @@ StreamPoolScheduler::StreamPoolScheduler(const SchedulerOptions& options, size_t
     if (options.measure_block_time) gpu2sched_block_time_channel_.connect(std::string(), options.ring_slots);
     job::Context::set_gpu2sched_block_time_channel(options.measure_block_time ? &gpu2sched_block_time_channel_ : nullptr);
     notifiers_raw_ = job::FinishedBlockNotifier::create_array(options.num_streams, &gpu2sched_channel_,
-                                                              options.measure_block_time ? &gpu2sched_block_time_channel_ : nullptr);
+                                                              options.measure_block_time ? &gpu2sched_block_time_channel_ : nullptr,
+                                                              options.noti_batch ? options.noti_batch : job::FinishedBlockNotifier::noti_batch_size);
     for (unsigned i = 0; i < options.num_streams; ++i) free_notifiers_.push_back(i);
 }
 

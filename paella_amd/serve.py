@@ -11,7 +11,7 @@ c_int, c_uint, c_float, c_double, c_char_p, c_void_p, c_size_t = (ctypes.c_int, 
 
 class ServerOptions(ctypes.Structure):
     _fields_ = [("name", c_char_p), ("sched", c_char_p), ("num_streams", c_uint), ("extra_kernels", c_uint), ("unfair", c_float),
-                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int)]
+                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int), ("noti_batch", c_uint)]
 
 
 class LoadOptions(ctypes.Structure):
@@ -68,9 +68,9 @@ class Server:
     """`with Server('name', 'full3', num_streams=64) as s: ...`; s.event_log() after the block."""
 
     def __init__(self, name, sched, num_streams=500, extra_kernels=2, unfair=1e6, sched_sleep=0, mem_marker=True, event_log=False,
-                 cpu=-1, measure_block_time=False):
+                 cpu=-1, measure_block_time=False, noti_batch=0):
         self.opts = ServerOptions(name.encode(), sched.encode(), num_streams, extra_kernels, unfair, sched_sleep, int(mem_marker),
-                                  int(event_log), cpu, int(measure_block_time))
+                                  int(event_log), cpu, int(measure_block_time), noti_batch)
         self.name = name
         self.handle = c_void_p()
 

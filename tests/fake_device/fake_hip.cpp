@@ -62,8 +62,10 @@ void post(uint8_t is_start, unsigned num, uint32_t job_id) {
     llis::job::Context::get_gpu2sched_channel()->write(info);
 }
 
+unsigned g_batch = llis::job::FinishedBlockNotifier::noti_batch_size;
+
 void post_batches(uint8_t is_start, unsigned n, uint32_t job_id) {
-    constexpr unsigned B = llis::job::FinishedBlockNotifier::noti_batch_size;
+    const unsigned B = g_batch;
     for (unsigned i = 0; i < n / B; ++i) post(is_start, B, job_id);
     if (n % B) post(is_start, n % B, job_id);
 }
@@ -143,6 +145,9 @@ void enqueue(void* stream, Op op) {
 extern "C" {
 
 // ---- control surface for tests and fake job definitions
+// Workgroups per aggregated message of the scripted kernels (what the notifiers of a real device are created with).
+void fake_hip_set_batch(unsigned batch) { g_batch = batch ? batch : llis::job::FinishedBlockNotifier::noti_batch_size; }
+
 int fake_hip_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks) {
     Op op{OP_KERNEL, 0};
     op.job_id = job_id;

@@ -2,7 +2,7 @@
 // with the client side of the wire protocol written out by hand, message by message.  Reads commands on
 // stdin, prints replies and finally the scheduler's event log on stdout.
 //
-//   sched NAME streams N [extra K] [unfair X] [mem marker|hostfunc] [budget REGS SMEM THREADS BLOCKS]
+//   sched NAME streams N [extra K] [unfair X] [mem marker|hostfunc] [budget REGS SMEM THREADS BLOCKS] [batch B]
 //   client                      register a client                      -> "client ID"
 //   job PATH                    register a job type, grow its pool     -> "job TYPE"
 //   launch TYPE [SLOT]          LAUNCH_JOB for slot SLOT of the pool
@@ -38,6 +38,7 @@
 extern "C" int fake_hip_step_oldest(int full);
 extern "C" int fake_hip_step_stream(unsigned index, int full);
 extern "C" unsigned fake_hip_pending(void);
+extern "C" void fake_hip_set_batch(unsigned batch);
 
 using namespace llis;
 
@@ -131,6 +132,7 @@ int main() {
                 else if (key == "extra") in >> opt.extra_kernels;
                 else if (key == "unfair") in >> opt.unfair;
                 else if (key == "mem") { std::string m; in >> m; opt.mem_marker = (m == "marker"); }
+                else if (key == "batch") { in >> opt.noti_batch; fake_hip_set_batch(opt.noti_batch); }
                 else if (key == "budget") { in >> b[0] >> b[1] >> b[2] >> b[3]; have_budget = true; }
             }
             if (have_budget && name == "full3") h.scheduler = std::make_unique<server::SchedulerFull3>(opt, server::SmResources(b[0], b[1], b[2], b[3]));

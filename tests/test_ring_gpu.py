@@ -35,13 +35,27 @@ def ring(cuda):
     lib.paella_ring_destroy(handle)
 
 
+REFERENCE_BATCH = 16  # reference include/llis/job/finished_block_notifier.h:118
+
+
+@pytest.fixture()
+def ring16(cuda):
+    """Notifiers created with the reference's batch size."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+    handle = ctypes.c_void_p()
+    _abi.check(lib.paella_ring_create_batched(4096, 4, REFERENCE_BATCH, ctypes.byref(handle)), "paella_ring_create_batched")
+    yield lib, handle
+    lib.paella_ring_destroy(handle)
+
+
 def batch():
     from paella_amd import _abi
     return _abi.ops().paella_ring_batch_size()
 
 
-def expected_nums(n):
-    b = batch()
+def expected_nums(n, b=None):
+    b = b or batch()
     return sorted([b] * (n // b) + ([n % b] if n % b else []))
 
 
@@ -73,6 +87,37 @@ def test_aggregated_notifier_message_count_and_layout(ring, grid):
             else:
                 finished += k
             assert finished <= started + batch() - 1
+
+
+@pytest.mark.parametrize("n", [1, 5, 16, 17, 200, 1000])
+def test_reference_batch_size_gives_the_reference_message_sequence(ring16, n):
+    """At batch 16 a grid of n workgroups sends ceil(n/16) start and ceil(n/16) end messages, `num` = 16 except one
+    remainder n mod 16 (reference include/llis/job/finished_block_notifier.h:27-43): 2 + 2 for 17, 13 + 13 for 200
+    (12 x 16 + 8), 63 + 63 for 1000 (62 x 16 + 8)."""
+    lib, h = ring16
+    from paella_amd import _abi
+    per_kind = -(-n // REFERENCE_BATCH)
+    assert per_kind == {1: 1, 5: 1, 16: 1, 17: 2, 200: 13, 1000: 63}[n]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for rep in range(2):  # the counters reset themselves
+        _abi.check(lib.paella_ring_probe_launch(h, rep, n, 1, 1, 64, 500 + rep, 0, stream))
+        out = np.zeros(2 * per_kind, np.uint64)
+        assert lib.paella_ring_drain(h, out.ctypes.data, 2 * per_kind, 20.0) == 2 * per_kind
+        torch.cuda.synchronize()
+        assert lib.paella_ring_can_read(h) == 0
+        m = decode(out)
+        assert np.all(m["job_id"] == 500 + rep)
+        for kind in (1, 0):
+            nums = sorted(m["num"][m["is_start"] == kind].tolist())
+            assert nums == expected_nums(n, REFERENCE_BATCH) and sum(nums) == n
+
+
+def test_batch_size_must_be_a_power_of_two_up_to_128(cuda):
+    from paella_amd import _abi
+    lib = _abi.ops()
+    for bad in (0, 3, 48, 256):
+        handle = ctypes.c_void_p()
+        assert lib.paella_ring_create_batched(4096, 1, bad, ctypes.byref(handle)) == -1 and not handle.value
 
 
 def test_raw_hooks_one_message_pair_per_workgroup(ring):

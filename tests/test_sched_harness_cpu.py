@@ -95,3 +95,16 @@ def test_dummy_shape_closed_form_through_the_real_server():
         expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
     expect.append(("E", 0))
     assert core == expect
+
+
+def test_reference_notification_batch_reaches_the_scheduler_in_sixteens():
+    """`batch 16`: the scripted device posts what notifiers created with the reference's batch size post, and the
+    scheduler's bookkeeping (pending / running workgroups) follows message by message: fake_big's 3000 workgroups
+    arrive as 187 x 16 + 8, twice."""
+    budget = (1 << 40, 1 << 40, 1 << 40, 1 << 40)
+    replies, events = check("full3", 2, "launch 3 0\ndrain\n", extra="batch 16 budget %d %d %d %d" % budget, budget=budget)
+    for kind in (1, 0):
+        nums = [e[3] for e in events if e[0] == "B" and e[2] == kind]
+        per_stage = [16] * 187 + [8]
+        assert len(nums) % 188 == 0 and nums == per_stage * (len(nums) // 188)
+    assert [r for r in replies if r.startswith("done")] == ["done 4000"]

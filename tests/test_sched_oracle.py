@@ -67,15 +67,19 @@ def test_fifo2_arrival_order_and_lifo_pools():
 
 
 def test_sm_resources_closed_form():
-    r = sched.SmResources(1000, 100, 64, 4)
+    """One workgroup of 8 threads, 10 registers, 20 bytes of LDS is charged a whole wave of 64 lanes, 16 registers per
+    lane and one 1280-byte LDS granule; the pooling itself is reference src/server/sm_resources.cpp:36-66."""
+    r = sched.SmResources(10000, 5000, 256, 4)
     st = kernel(2, threads=8, regs=10, smem=20)
     assert r.fits(st)
     r.acquire(st, 2)
-    assert r.free == [1000 - 160, 60, 48, 2]
+    assert r.free == [10000 - 2 * 64 * 16, 5000 - 2 * 1280, 256 - 2 * 64, 2]
     assert not r.fits(kernel(3, threads=8, regs=10))      # workgroup slots
-    assert not r.fits(kernel(1, threads=8, regs=10, smem=61))
+    assert r.fits(kernel(1, threads=8, regs=10, smem=1280))
+    assert not r.fits(kernel(1, threads=8, regs=10, smem=1281))  # two granules, 2440 bytes left
+    assert not r.fits(kernel(2, threads=65, regs=10))     # two waves each: 256 lanes, 128 left
     r.release(st, 1)
-    assert r.free == [920, 80, 56, 3]
+    assert r.free == [10000 - 64 * 16, 5000 - 1280, 256 - 64, 3]
 
 
 def test_stage_length_estimator_recurrence():
@@ -186,3 +190,27 @@ def test_jobqueue_fairness_triggers_and_is_fifo_among_equals():
     order = [q.pop().tag for _ in range(4)]
     assert order[0] == 0
     assert 3 in order[:3], "the starved type must be served before type 0 is exhausted"
+
+
+def test_occupancy_closed_form_in_gfx950_units():
+    """Hand-derived: 4 SIMDs, 512 registers per lane and at most 8 waves per SIMD, registers in steps of 8, LDS in steps of
+    1280 bytes out of 160 KiB, at most 32 workgroups per compute unit."""
+    cases = [
+        ((512, 64, 32768), 4),    # 8 waves x 64 regs: 8 waves/SIMD -> 32 waves / 8; LDS 163840 // 33280 = 4
+        ((512, 64, 40960), 4),    # LDS exactly 32 granules: 163840 // 40960 = 4
+        ((512, 64, 40961), 3),    # one byte more takes another granule: 163840 // 42240 = 3
+        ((256, 128, 0), 4),       # 4 waves/SIMD -> 16 waves / 4
+        ((256, 129, 0), 3),       # 129 -> 136 regs: 3 waves/SIMD -> 12 / 4
+        ((256, 32, 0), 8),        # register-unbound: 32 waves / 4
+        ((10, 16, 0), 32),        # a 10-thread workgroup still takes a whole wave; capped by the 32 workgroup slots
+        ((1024, 128, 0), 1),      # 16 waves of 128 regs fill the unit
+        ((1024, 129, 0), 0),      # and do not fit with one register more
+        ((64, 72, 0), 28),        # 512 // 72 = 7 waves/SIMD
+        ((128, 512, 0), 2),       # one wave per SIMD
+    ]
+    for (threads, regs, lds), want in cases:
+        assert sched.blocks_per_cu(threads, regs, lds) == want, (threads, regs, lds)
+    # the pooled budget charges the same units: a 10-thread workgroup with 20 registers and 100 bytes of LDS
+    assert sched.wg_charge(sched.Stage(False, 3, 10, 100, 20)) == (64 * 24, 1280, 64)
+    r = sched.SmResources(64 * 24 * 3, 1280 * 3, 64 * 3, 3)
+    assert r.fits(sched.Stage(False, 3, 10, 100, 20)) and not r.fits(sched.Stage(False, 3, 10, 100, 25))

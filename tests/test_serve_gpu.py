@@ -81,6 +81,26 @@ def test_both_copy_completion_paths_on_the_gpu(cuda, mem_marker):
     np.testing.assert_array_equal(out, 10 * x)
 
 
+def test_vec_add_at_the_reference_batch_size_sends_13_plus_13_messages_per_kernel(cuda):
+    """--noti_batch 16 (the reference's constant, reference include/llis/job/finished_block_notifier.h:118): each of
+    vec_add's ten 200-workgroup kernels reports 12 x 16 + 8 started and 12 x 16 + 8 finished workgroups in 13 + 13
+    messages (reference finished_block_notifier.h:27-43, jobs/vec_add_coroutine/vec_add_coroutine.cu:115-141)."""
+    from paella_amd import serve
+    x = np.arange(32000, dtype=np.float32)
+    with serve.Server(server_name("b16"), "full3", num_streams=4, event_log=True, noti_batch=16) as srv:
+        out, lat = serve.client_single(srv.name, serve.job_path("vec_add_coroutine"), x, 32000, n=2)
+    np.testing.assert_array_equal(out, 10 * x)
+    ev = sched.parse_log(srv.event_log())
+    for kind in (1, 0):
+        nums = [e[3] for e in ev if e[0] == "B" and e[2] == kind]
+        assert len(nums) == 2 * 10 * 13
+        assert sorted(nums) == sorted(2 * 10 * ([16] * 12 + [8]))
+    with serve.Server(server_name("b64"), "full3", num_streams=4, event_log=True) as srv:
+        serve.client_single(srv.name, serve.job_path("vec_add_coroutine"), x, 32000, n=1)
+    nums = [e[3] for e in sched.parse_log(srv.event_log()) if e[0] == "B" and e[2] == 0]
+    assert sorted(nums) == sorted(10 * ([64] * 3 + [8]))
+
+
 def test_plain_job_with_raw_hooks(cuda):
     from paella_amd import serve
     with serve.Server(server_name("hello"), "full3", num_streams=4, event_log=True) as srv:
