@@ -29,7 +29,9 @@ class UnixDatagramSocket {
 
     ssize_t write(const void* buf, size_t count);
     // Never blocks: false when the receiver's queue is full right now (the datagram was not sent).
-    bool try_write(const void* buf, size_t count);
+    // *refused (optional): the failure was ECONNREFUSED -- nobody is bound to the name (any more), or, on some
+    // sandboxed kernels, the queue is full.
+    bool try_write(const void* buf, size_t count, bool* refused = nullptr);
     ssize_t read(void* buf, size_t count);
 
   private:

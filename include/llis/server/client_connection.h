@@ -6,6 +6,7 @@
 #include <llis/ipc/shm_channel.h>
 #include <llis/ipc/unix_datagram_socket.h>
 
+#include <chrono>
 #include <utility>
 
 namespace llis {
@@ -27,29 +28,56 @@ class ClientConnection {
     // never blocks, and one that did not fit is owed (they are all the same byte, so order does not matter).
     // Returns true if the poke is owed rather than sent.
     bool wake() {
+        if (dead_) return false;
         if (owed_wakeups_ == 0 && poke()) return false;
         ++owed_wakeups_;
         return true;
     }
 
-    // Sends as many owed pokes as fit now; returns how many went out.
+    // Sends as many owed pokes as fit now; returns how many are no longer owed (sent, or written off with a peer that has
+    // refused every poke for kDeadAfter: a client that exited without waiting for its requests).
     unsigned retry_wakeups() {
-        unsigned sent = 0;
+        unsigned settled = 0;
         while (owed_wakeups_ != 0 && poke()) {
             --owed_wakeups_;
-            ++sent;
+            ++settled;
         }
-        return sent;
+        if (dead_) {
+            settled += owed_wakeups_;
+            owed_wakeups_ = 0;
+        }
+        return settled;
     }
+
+    // A dead peer gets neither pokes nor completions (its completion ring would fill up and block the serving thread).
+    bool is_dead() const { return dead_; }
+
+    static constexpr std::chrono::milliseconds kDeadAfter{2000};
 
   private:
     bool poke() {
+        if (dead_) return false;
         const bool byte = true;
-        return s2c_socket_.try_write(&byte, sizeof(byte));
+        bool refused = false;
+        if (s2c_socket_.try_write(&byte, sizeof(byte), &refused)) {
+            refusing_ = false;
+            return true;
+        }
+        if (!refused) {
+            refusing_ = false;
+        } else if (!refusing_) {
+            refusing_ = true;
+            refused_since_ = std::chrono::steady_clock::now();
+        } else if (std::chrono::steady_clock::now() - refused_since_ > kDeadAfter) {
+            dead_ = true;
+        }
+        return false;
     }
 
     ClientId client_id_;
     unsigned owed_wakeups_ = 0;
+    bool refusing_ = false, dead_ = false;
+    std::chrono::steady_clock::time_point refused_since_;
     ipc::ShmChannelCpuWriter s2c_channel_;
     ipc::UnixDatagramSocket s2c_socket_;
 };

@@ -40,6 +40,7 @@ class SmResources {
     static constexpr long long kSimdsPerCu = 4;
     static constexpr long long kVgprsPerSimdLane = 512; // unified register file, per lane
     static constexpr long long kMaxWavesPerSimd = 8;
+    static constexpr long long kMaxBlocksPerCu = 32;    // one-wave workgroups can take every wave slot
 
     static long long round_up(long long v, long long g) { return (v + g - 1) / g * g; }
     // What one workgroup takes out of each pool.

@@ -33,8 +33,8 @@ typedef struct llis_hip_device_caps {
     int num_cus;                  /* compute units (256 on MI355X) */
     int wavefront_size;           /* 64 */
     int max_threads_per_cu;       /* resident threads per CU */
-    int max_blocks_per_cu;        /* resident workgroups per CU */
-    int vgprs_per_cu;             /* 32-bit vector registers per CU, counted per thread-lane like CUDA's regsPerMultiprocessor */
+    int max_blocks_per_cu;        /* resident workgroups per CU: one per wave slot (32) */
+    int vgprs_per_cu;             /* vector-register lanes per CU: 4 SIMDs x 512 registers x 64 lanes (131072) */
     int lds_bytes_per_cu;         /* 160 KiB on gfx950 */
     int clock_khz;
     int l2_bytes;

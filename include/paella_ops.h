@@ -47,7 +47,8 @@ enum paella_act { PAELLA_ACT_NONE = 0, PAELLA_ACT_RELU = 1, PAELLA_ACT_RELU6 = 2
 typedef struct paella_launch_dims {
     unsigned grid;        /* number of workgroups */
     unsigned block;       /* threads per workgroup */
-    unsigned lds_bytes;   /* LDS per workgroup */
+    unsigned lds_bytes;   /* LDS per workgroup: what the launch asks for (paella_conv_plan.dims) or, from the *_dims functions
+                             that look at the loaded kernel, that plus the kernel's statically allocated LDS */
     unsigned vgprs;       /* vector registers per thread */
 } paella_launch_dims;
 
@@ -82,6 +83,10 @@ typedef struct paella_conv_plan {
 /* Pure host arithmetic: picks the kernel variant and launch shape.  tile_hint = 0 lets the library
  * choose; otherwise log2(splits)<<12 | mi<<8 | ni<<4 | log2(kw) forces a shape (tuning sweeps and tests). */
 int paella_conv2d_plan(const paella_conv_desc* desc, int has_residual, int tile_hint, paella_conv_plan* plan);
+
+/* Launch shape of paella_conv2d_launch for the scheduler: the plan's, with the register count and the static LDS of the
+ * kernel that is actually launched (read from the loaded code object; the plan's own figures without a device). */
+int paella_conv2d_dims(const paella_conv_plan* plan, paella_launch_dims* dims);
 
 /* Re-lays out OIHW weights [K][C/g][R][S] into the blob the kernel reads (host memory to host memory). */
 int paella_conv2d_pack(const paella_conv_plan* plan, const float* w_oihw, void* blob_host);
@@ -208,9 +213,12 @@ int paella_conv_kernel_vgprs(int kind, int mi, int ni, int kw, unsigned* vgprs);
  * src/server/sm_resources.cpp:17-66) is checked against.  `form` of a conv: 0 = one conv, 1 = conv on a transformed
  * input, 2 = group of convs, 3 = group of convs with a pooling operator (forms 1 to 3: mi == ni == 1; 1 and 3: k_order 1). */
 int paella_kernel_occupancy(const char* family, unsigned block, unsigned lds_bytes, int* blocks_per_cu);
-/* vgprs (may be NULL): vector registers per thread of that same kernel, read from the loaded code object. */
+/* Statically allocated LDS of a kernel family, read from the loaded code object (needs a GPU). */
+int paella_kernel_static_lds(const char* family, unsigned* lds_bytes);
+/* vgprs, static_lds (may be NULL): vector registers per thread and statically allocated LDS of that same kernel, read from
+ * the loaded code object; lds_bytes is the dynamic LDS of the launch. */
 int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, int kw, int k_order, unsigned lds_bytes, int* blocks_per_cu,
-                                 unsigned* vgprs);
+                                 unsigned* vgprs, unsigned* static_lds);
 
 /*
  * Direct dispatch.  A queue created here is a user-mode hardware queue owned by this library; its handle can

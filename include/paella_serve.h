@@ -63,6 +63,8 @@ typedef struct paella_load_options {
     unsigned seed;
     int pin_threads;           /* pin monitor/submit threads to CPUs 0 and 2 like the reference client */
     const char* profile_prefix; /* non-NULL: server-side recording around the measured phase, saved to this prefix */
+    const char* trace_path;    /* non-NULL: replay this "<type> <submit time us>" trace (paella_workload_pregen,
+                                  llis_app_workload_pregen; reference tests/utils/workload_pregen.cpp:107) instead of drawing */
 } paella_load_options;
 
 typedef struct paella_latency_stats {
@@ -78,6 +80,12 @@ typedef struct paella_load_result {
     unsigned queue_full_events, type_full_events;
 } paella_load_result;
 
+/* Writes an arrival trace with the draws of the live generator (type first, then the gap), in the file set of the
+ * reference's tool (reference tests/utils/workload_pregen.cpp:72-115): <prefix>_iat<I>_lns<S>_n<N>_seed<K>.txt plus one
+ * _job<t>.txt per type.  The combined file's path goes to path_out (capacity cap, NUL-terminated).  0 on success. */
+int paella_workload_pregen(double iat_us, int dist_exp, double ln_sigma, unsigned num_jobs, unsigned seed, const char* prefix,
+                           const float* proportions, int num_types, char* path_out, size_t cap);
+
 /* latencies_us (optional) receives the measured latencies in completion order; capacity num_jobs. */
 int paella_client_run(const paella_load_options* options, paella_load_result* result, double* latencies_us);
 
@@ -85,6 +93,31 @@ int paella_client_run(const paella_load_options* options, paella_load_result* re
  * of the last request is returned.  latencies_us (optional, capacity n) in microseconds. */
 int paella_client_single(const char* server_name, const char* job_path, const void* input, size_t in_bytes, void* output,
                          size_t out_bytes, int n, double* latencies_us);
+
+/*
+ * Plain multi-stream serving with no server and no scheduler: `num_streams` HIP streams, each request's whole
+ * forward pass (input copy, every kernel back to back, output copy) issued on one free stream by the submitting
+ * thread, completion found by polling the streams.  The comparison arm the reference keeps as a stand-alone program
+ * (reference tests/simple/tvm_direct_multistream.cpp:143-156,193-301; CUDA-SS with one stream, CUDA-MS with 141,
+ * sosp23_artifact/gen_data_fig11_cuda.sh:34-44).  Same arrival process, caps and statistics as paella_client_run.
+ */
+typedef struct paella_direct_options {
+    int num_types;
+    const char* models[PAELLA_MAX_JOB_TYPES];     /* zoo model names (paella_models.h), e.g. "mnist", "inception_v3" */
+    float proportions[PAELLA_MAX_JOB_TYPES];
+    unsigned max_outstanding[PAELLA_MAX_JOB_TYPES]; /* pooled instances per model */
+    uint64_t seed_weights;     /* seed of the models' weights (the adapters' LLIS_MODEL_SEED) */
+    int num_streams;           /* streams = cap on requests in flight */
+    double iat_us;             /* mean inter-arrival time; 0 = saturation */
+    int dist_exp;              /* 1 exponential (Poisson arrivals), 0 log-normal */
+    double ln_sigma;
+    unsigned num_jobs;         /* measured requests */
+    unsigned warmup_jobs;      /* served before the clock starts, beyond the one run per pooled instance */
+    unsigned seed;             /* of the arrival process */
+    int pin_threads;           /* pin monitor/submit threads to CPUs 0 and 2 like the reference */
+} paella_direct_options;
+
+int paella_direct_multistream_run(const paella_direct_options* options, paella_load_result* result);
 
 #ifdef __cplusplus
 }

@@ -62,8 +62,11 @@ int llis_hip_get_device_caps(llis_hip_device_caps* caps) {
     caps->num_cus = prop.multiProcessorCount;
     caps->wavefront_size = prop.warpSize;
     caps->max_threads_per_cu = prop.maxThreadsPerMultiProcessor;
-    caps->max_blocks_per_cu = prop.maxBlocksPerMultiProcessor > 0 ? prop.maxBlocksPerMultiProcessor : 32;
-    caps->vgprs_per_cu = prop.regsPerMultiprocessor > 0 ? prop.regsPerMultiprocessor : prop.regsPerBlock;
+    // The runtime's properties carry CUDA-shaped figures here (65536 "registers per multiprocessor", 2 "blocks per
+    // multiprocessor"); a gfx950 compute unit has 4 SIMDs of 512 vector registers x 64 lanes and one workgroup slot per
+    // wave slot.
+    caps->max_blocks_per_cu = prop.maxThreadsPerMultiProcessor / prop.warpSize;
+    caps->vgprs_per_cu = 4 * 512 * prop.warpSize;
     caps->lds_bytes_per_cu = (int)(prop.maxSharedMemoryPerMultiProcessor > 0 ? prop.maxSharedMemoryPerMultiProcessor
                                                                              : prop.sharedMemPerBlock);
     caps->clock_khz = prop.clockRate;

@@ -814,6 +814,18 @@ int allow_lds(const void* kern, unsigned lds_bytes) {
     return (int)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
 }
 
+// What the scheduler accounts for a launch of `fn`: the kernel's own register count and, on top of the dynamic LDS already
+// in dims, its statically allocated LDS -- both read from the loaded code object (left as planned without a device).
+void add_kernel_resources(const void* fn, paella_launch_dims* dims) {
+    hipFuncAttributes attr;
+    if (fn && hipFuncGetAttributes(&attr, fn) == hipSuccess && attr.numRegs > 0) {
+        dims->vgprs = (unsigned)attr.numRegs;
+        dims->lds_bytes += (unsigned)attr.sharedSizeBytes;
+    } else {
+        (void)hipGetLastError();
+    }
+}
+
 typedef void (*ConvGroupKernel)(ConvGroupArgs);
 
 ConvGroupKernel pick_group_kernel(int kw, int k_order) {
@@ -844,11 +856,7 @@ extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, in
         }
         dims->block = plans[0]->dims.block;
         dims->vgprs = plans[0]->dims.vgprs;
-        hipFuncAttributes attr;
-        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_group_kernel(plans[0]->kw, plans[0]->k_order))) == hipSuccess && attr.numRegs > 0)
-            dims->vgprs = (unsigned)attr.numRegs;
-        else
-            (void)hipGetLastError();
+        add_kernel_resources(reinterpret_cast<const void*>(pick_group_kernel(plans[0]->kw, plans[0]->k_order)), dims);
     }
     return 0;
 }
@@ -872,8 +880,10 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
         if (i < n) next += m.plan->dims.grid;
     }
     ConvGroupKernel kern = pick_group_kernel(plans[0]->kw, plans[0]->k_order);
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
-    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
+    unsigned dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
+    for (int i = 0; i < n; ++i) dyn_lds = std::max(dyn_lds, plans[i]->dims.lds_bytes);
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
+    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dyn_lds, reinterpret_cast<hipStream_t>(stream), g);
     return (int)hipGetLastError();
 }
 
@@ -912,11 +922,7 @@ extern "C" int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plan
         dims->block = plans[0]->dims.block;
         dims->grid += (unsigned)(((size_t)pa.C * pa.P * pa.Q + dims->block - 1) / dims->block);
         dims->vgprs = plans[0]->dims.vgprs;
-        hipFuncAttributes attr;
-        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_group_pool_kernel(plans[0]->kw))) == hipSuccess && attr.numRegs > 0)
-            dims->vgprs = (unsigned)attr.numRegs;
-        else
-            (void)hipGetLastError();
+        add_kernel_resources(reinterpret_cast<const void*>(pick_group_pool_kernel(plans[0]->kw)), dims);
     }
     return 0;
 }
@@ -943,8 +949,10 @@ extern "C" int paella_conv2d_launch_group_pool(const paella_conv_operands* membe
     g.pool_start = next;
     if (!paella::pool_fill_args(pool, pool_x, pool_y, job_id, notifier, &g.pool)) return PAELLA_EINVAL;
     ConvGroupPoolKernel kern = pick_group_pool_kernel(plans[0]->kw);
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dims.lds_bytes)) return rc;
-    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), g);
+    unsigned dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
+    for (int i = 0; i < n; ++i) dyn_lds = std::max(dyn_lds, plans[i]->dims.lds_bytes);
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
+    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dyn_lds, reinterpret_cast<hipStream_t>(stream), g);
     return (int)hipGetLastError();
 }
 
@@ -1009,11 +1017,15 @@ extern "C" int paella_conv2d_transformed_dims(const paella_conv_plan* plan, pael
     if (!plan || !dims) return PAELLA_EINVAL;
     if (!paella_conv2d_plan_takes_input_transform(plan)) return PAELLA_ENOSUP;
     *dims = plan->dims;
-    hipFuncAttributes attr;
-    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pick_pre_kernel(plan->kw))) == hipSuccess && attr.numRegs > 0)
-        dims->vgprs = (unsigned)attr.numRegs;
-    else
-        (void)hipGetLastError();
+    add_kernel_resources(reinterpret_cast<const void*>(pick_pre_kernel(plan->kw)), dims);
+    return 0;
+}
+
+extern "C" int paella_conv2d_dims(const paella_conv_plan* plan, paella_launch_dims* dims) {
+    if (!plan || !dims) return PAELLA_EINVAL;
+    *dims = plan->dims;
+    add_kernel_resources(plan->kind == 1 ? reinterpret_cast<const void*>(dwconv_kernel)
+                                         : reinterpret_cast<const void*>(pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order)), dims);
     return 0;
 }
 
@@ -1039,7 +1051,7 @@ extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, co
 }
 
 extern "C" int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, int kw, int k_order, unsigned lds_bytes, int* blocks_per_cu,
-                                            unsigned* vgprs) {
+                                            unsigned* vgprs, unsigned* static_lds) {
     if (!blocks_per_cu) return PAELLA_EINVAL;
     const void* fn = nullptr;
     unsigned block = 64u * (unsigned)kw;
@@ -1055,10 +1067,11 @@ extern "C" int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, 
     }
     if (!fn) return PAELLA_EINVAL;
     if (int rc = allow_lds(fn, lds_bytes)) return rc;
-    if (vgprs) {
+    if (vgprs || static_lds) {
         hipFuncAttributes attr;
         if (hipError_t e = hipFuncGetAttributes(&attr, fn)) return (int)e;
-        *vgprs = (unsigned)attr.numRegs;
+        if (vgprs) *vgprs = (unsigned)attr.numRegs;
+        if (static_lds) *static_lds = (unsigned)attr.sharedSizeBytes;
     }
     return (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, fn, (int)block, lds_bytes);
 }

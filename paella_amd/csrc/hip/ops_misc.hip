@@ -495,6 +495,17 @@ int paella_kernel_occupancy(const char* family, unsigned block, unsigned lds_byt
     return (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, fn, (int)block, lds_bytes);
 }
 
+int paella_kernel_static_lds(const char* family, unsigned* lds_bytes) {
+    if (!family || !lds_bytes) return PAELLA_EINVAL;
+    const void* fn = family_kernel(family);
+    if (!fn) return PAELLA_EINVAL;
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, fn);
+    if (e != hipSuccess) return (int)e;
+    *lds_bytes = (unsigned)attr.sharedSizeBytes;
+    return 0;
+}
+
 int paella_kernel_vgprs(const char* family, unsigned* vgprs) {
     if (!family || !vgprs) return PAELLA_EINVAL;
     const void* fn = family_kernel(family);

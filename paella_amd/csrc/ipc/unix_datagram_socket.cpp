@@ -71,10 +71,12 @@ ssize_t UnixDatagramSocket::write(const void* buf, size_t count) {
     return n;
 }
 
-bool UnixDatagramSocket::try_write(const void* buf, size_t count) {
+bool UnixDatagramSocket::try_write(const void* buf, size_t count, bool* refused) {
     ssize_t n = ::sendto(fd_, buf, count, MSG_DONTWAIT, reinterpret_cast<const sockaddr*>(&remote_), sizeof(remote_));
+    if (refused) *refused = n < 0 && errno == ECONNREFUSED;
     if (n >= 0) return true;
-    // A receiver whose queue is full reports EAGAIN on Linux; some sandboxed kernels report ECONNREFUSED.
+    // A receiver whose queue is full reports EAGAIN on Linux; some sandboxed kernels report ECONNREFUSED, which is also
+    // what a receiver that no longer exists gives: the caller tells the two apart by how long it lasts.
     if (errno == EAGAIN || errno == EWOULDBLOCK || errno == ENOBUFS || errno == ECONNREFUSED) return false;
     LLIS_CHECK_POSIX(n);
     return false;

@@ -323,10 +323,7 @@ int plan_nodes(paella_model* m, std::vector<size_t>& tensor_off, std::vector<siz
                 st.op = st.conv.kind == 0 ? "conv" : "dwconv";
                 st.flops = st.conv.flops;
                 st.bytes = st.conv.bytes;
-                {
-                    unsigned v = 0;
-                    if (paella_conv_kernel_vgprs(st.conv.kind, st.conv.mi, st.conv.ni, st.conv.kw, &v) == 0 && v) st.dims.vgprs = v;
-                }
+                paella_conv2d_dims(&st.conv, &st.dims);  // registers and static LDS of the kernel this plan launches
                 blob_off[i] = total;
                 total += align256(st.conv.blob_bytes);
                 break;

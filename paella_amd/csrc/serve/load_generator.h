@@ -31,13 +31,13 @@ namespace loadgen {
 
 using Clock = std::chrono::steady_clock;
 
-double us_since_epoch(Clock::time_point t) { return std::chrono::duration<double, std::micro>(t.time_since_epoch()).count(); }
+inline double us_since_epoch(Clock::time_point t) { return std::chrono::duration<double, std::micro>(t.time_since_epoch()).count(); }
 
 struct Stats {
     double mean = 0, p50 = 0, p90 = 0, p95 = 0, p99 = 0, max = 0, sd = 0;
 };
 
-Stats summarize(std::vector<double>& v) {
+inline Stats summarize(std::vector<double>& v) {
     Stats s;
     if (v.empty()) return s;
     std::sort(v.begin(), v.end());
@@ -83,7 +83,14 @@ class LoadGenerator {
         latencies_per_type_.resize(types);
     }
 
-    void add_instance(unsigned type, llis::client::JobInstanceRef* inst) { free_instances_[type].push_back(inst); }
+    void add_instance(unsigned type, llis::client::JobInstanceRef* inst) {
+        free_instances_[type].push_back(inst);
+        // Job reference ids are handed out server-wide, so they equal the type index only for the first client of a
+        // server (which is what reference app/client.cpp:77 relies on); keep the mapping instead.
+        const unsigned ref = inst->get_job_ref_id();
+        if (ref >= type_of_ref_.size()) type_of_ref_.resize(ref + 1, 0);
+        type_of_ref_[ref] = type;
+    }
 
     void publish_free_counts() {
         for (size_t t = 0; t < free_instances_.size(); ++t) free_counts_[t].store((unsigned)free_instances_[t].size(), std::memory_order_release);
@@ -164,7 +171,7 @@ class LoadGenerator {
             const auto now = Clock::now();
             const double latency = us_since_epoch(now) - inst->get_start_time();
             const double t = std::chrono::duration<double, std::micro>(now - very_start).count();
-            const unsigned type = inst->get_job_ref_id();
+            const unsigned type = type_of_ref_[inst->get_job_ref_id()];
             {
                 std::lock_guard<std::mutex> lk(mtx_);
                 free_instances_[type].push_back(inst);
@@ -258,6 +265,7 @@ class LoadGenerator {
     std::vector<unsigned> outstanding_per_type_;
     std::atomic<int> num_outstanding_{0};
 
+    std::vector<unsigned> type_of_ref_;
     std::vector<std::pair<unsigned, double>> trace_;
     std::vector<double> latencies_;
     std::vector<std::vector<double>> latencies_per_type_;

@@ -3,6 +3,7 @@
 #include "paella_serve.h"
 
 #include "load_generator.h"
+#include "workload_pregen.h"
 
 #include <llis/server/scheduler.h>
 #include <llis/server/server.h>
@@ -114,6 +115,7 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         opt.seed = o->seed;
         opt.pin_threads = o->pin_threads != 0;
         if (o->profile_prefix) opt.profile_prefix = o->profile_prefix;
+        if (o->trace_path) opt.trace_path = o->trace_path;
 
         std::vector<float> props_cum;
         std::vector<unsigned> max_outstanding;
@@ -154,6 +156,17 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         std::fprintf(stderr, "paella_client_run: %s\n", e.what());
         return -1;
     }
+}
+
+int paella_workload_pregen(double iat_us, int dist_exp, double ln_sigma, unsigned num_jobs, unsigned seed, const char* prefix,
+                           const float* proportions, int num_types, char* path_out, size_t cap) {
+    if (iat_us <= 0 || num_jobs == 0 || !prefix || !proportions || num_types <= 0 || !path_out || cap == 0) return -1;
+    std::vector<float> props_cum;
+    for (int t = 0; t < num_types; ++t) props_cum.push_back(proportions[t] + (t ? props_cum.back() : 0.f));
+    const std::string path = llis::loadgen::write_pregen_trace(iat_us, dist_exp != 0, ln_sigma, num_jobs, seed, prefix, props_cum);
+    if (path.empty() || path.size() + 1 > cap) return -1;
+    std::memcpy(path_out, path.c_str(), path.size() + 1);
+    return 0;
 }
 
 int paella_client_single(const char* server_name, const char* job_path, const void* input, size_t in_bytes, void* output, size_t out_bytes,

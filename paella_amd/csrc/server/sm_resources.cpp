@@ -15,7 +15,11 @@ SmResources::SmResources() {
     llis_hip_device_caps caps;
     LLIS_CHECK_HIP(llis_hip_get_device_caps(&caps));
     const long long cus = caps.num_cus;
-    init(cus * caps.vgprs_per_cu, cus * caps.lds_bytes_per_cu, cus * caps.max_threads_per_cu, cus * caps.max_blocks_per_cu);
+    // Register lanes and wave slots of a compute unit in the hardware's own units (the runtime's device properties
+    // carry a CUDA-shaped "registers per multiprocessor" of 65536, half of what the four SIMDs hold, and 2 for the
+    // resident workgroups per compute unit, where one-wave workgroups can fill all 32 wave slots).
+    init(cus * kSimdsPerCu * kVgprsPerSimdLane * kWaveLanes, cus * caps.lds_bytes_per_cu, cus * kSimdsPerCu * kMaxWavesPerSimd * kWaveLanes,
+         cus * kMaxBlocksPerCu);
 }
 
 void SmResources::init(long long nregs, long long smem, long long nthrs, long long nblocks) {

@@ -18,7 +18,7 @@ class LoadOptions(ctypes.Structure):
     _fields_ = [("server_name", c_char_p), ("num_types", c_int), ("job_paths", c_char_p * MAX_TYPES), ("proportions", c_float * MAX_TYPES),
                 ("max_outstanding", c_uint * MAX_TYPES), ("iat_us", c_double), ("dist_exp", c_int), ("ln_sigma", c_double),
                 ("concurrency", c_int), ("num_jobs", c_uint), ("warmup_jobs", c_uint), ("seed", c_uint), ("pin_threads", c_int),
-                ("profile_prefix", c_char_p)]
+                ("profile_prefix", c_char_p), ("trace_path", c_char_p)]
 
 
 class LatencyStats(ctypes.Structure):
@@ -34,11 +34,20 @@ class LoadResult(ctypes.Structure):
                 ("queue_full_events", c_uint), ("type_full_events", c_uint)]
 
 
+class DirectOptions(ctypes.Structure):
+    _fields_ = [("num_types", c_int), ("models", c_char_p * MAX_TYPES), ("proportions", c_float * MAX_TYPES),
+                ("max_outstanding", c_uint * MAX_TYPES), ("seed_weights", ctypes.c_uint64), ("num_streams", c_int), ("iat_us", c_double),
+                ("dist_exp", c_int), ("ln_sigma", c_double), ("num_jobs", c_uint), ("warmup_jobs", c_uint), ("seed", c_uint),
+                ("pin_threads", c_int)]
+
+
 SERVE_SYMBOLS = {
     "paella_server_start": (c_int, [ctypes.POINTER(ServerOptions), ctypes.POINTER(c_void_p)]),
     "paella_server_stop": (c_int, [c_void_p]),
     "paella_server_event_log": (c_size_t, [c_void_p, c_void_p, c_size_t]),
     "paella_client_run": (c_int, [ctypes.POINTER(LoadOptions), ctypes.POINTER(LoadResult), c_void_p]),
+    "paella_direct_multistream_run": (c_int, [ctypes.POINTER(DirectOptions), ctypes.POINTER(LoadResult)]),
+    "paella_workload_pregen": (c_int, [c_double, c_int, c_double, c_uint, c_uint, c_char_p, ctypes.POINTER(c_float), c_int, c_char_p, c_size_t]),
     "paella_client_single": (c_int, [c_char_p, c_char_p, c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p]),
 }
 
@@ -94,7 +103,7 @@ class Server:
 
 
 def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, seed=1, dist="exp", ln_sigma=2.0, pin_threads=False,
-               want_latencies=False, profile_prefix=None):
+               want_latencies=False, profile_prefix=None, trace_path=None):
     """jobs = [(path, proportion, max_outstanding), ...].  Returns a dict of the run's statistics."""
     import numpy as np
     o = LoadOptions()
@@ -109,6 +118,7 @@ def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, 
     o.iat_us, o.dist_exp, o.ln_sigma = iat_us, int(dist == "exp"), ln_sigma
     o.concurrency, o.num_jobs, o.warmup_jobs, o.seed, o.pin_threads = concurrency, num_jobs, warmup_jobs, seed, int(pin_threads)
     o.profile_prefix = profile_prefix.encode() if profile_prefix else None
+    o.trace_path = trace_path.encode() if trace_path else None
     res = LoadResult()
     lat = np.zeros(num_jobs, np.float64) if want_latencies else None
     if lib().paella_client_run(ctypes.byref(o), ctypes.byref(res), lat.ctypes.data if want_latencies else None) != 0:
@@ -131,3 +141,38 @@ def client_single(server_name, path, x, out_floats, n=1):
                                   lat.ctypes.data) != 0:
         raise RuntimeError("paella_client_single failed")
     return out, lat
+
+
+def _result_dict(r, n_types):
+    return {"elapsed_us": r.elapsed_us, "throughput_rps": r.throughput_rps, "all": r.all.as_dict(),
+            "per_type": [r.per_type[i].as_dict() for i in range(n_types)],
+            "queue_full_events": r.queue_full_events, "type_full_events": r.type_full_events}
+
+
+def direct_multistream(tenants, iat_us, num_streams, num_jobs, warmup_jobs=0, seed=1, dist="exp", ln_sigma=2.0, pin_threads=False,
+                       seed_weights=1):
+    """Plain multi-stream serving without a server (paella_direct_multistream_run).  tenants = [(zoo model name, proportion,
+    pooled instances), ...]; one stream per request in flight."""
+    o = DirectOptions()
+    o.num_types = len(tenants)
+    keep = []
+    for i, (model, prop, mo) in enumerate(tenants):
+        keep.append(model.encode())
+        o.models[i] = keep[-1]
+        o.proportions[i] = prop
+        o.max_outstanding[i] = mo
+    o.seed_weights, o.num_streams, o.iat_us, o.dist_exp, o.ln_sigma = seed_weights, num_streams, iat_us, int(dist == "exp"), ln_sigma
+    o.num_jobs, o.warmup_jobs, o.seed, o.pin_threads = num_jobs, warmup_jobs, seed, int(pin_threads)
+    r = LoadResult()
+    if lib().paella_direct_multistream_run(ctypes.byref(o), ctypes.byref(r)) != 0:
+        raise RuntimeError("paella_direct_multistream_run failed")
+    return _result_dict(r, len(tenants))
+
+
+def workload_pregen(prefix, proportions, iat_us, num_jobs, seed=1, dist="ln", ln_sigma=1.5):
+    """Writes an arrival trace (paella_workload_pregen); returns the combined file's path."""
+    props = (c_float * len(proportions))(*proportions)
+    buf = ctypes.create_string_buffer(4096)
+    if lib().paella_workload_pregen(iat_us, int(dist == "exp"), ln_sigma, num_jobs, seed, str(prefix).encode(), props, len(proportions), buf, 4096) != 0:
+        raise RuntimeError("paella_workload_pregen failed")
+    return buf.value.decode()

@@ -124,3 +124,21 @@ def test_product_has_no_cpu_compute_path():
                     if re.search(r"\boracle\b", open(os.path.join(dirpath, f), errors="ignore").read()):
                         offenders.append(os.path.join(dirpath, f))
     assert not offenders, offenders
+
+
+REFERENCE = "/root/reference"
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE), reason="the reference tree is not on this machine")
+@pytest.mark.parametrize("source", ["app/client.cpp", "tests/client/client.cpp", "tests/client/client_concurrent_runs.cpp",
+                                    "tests/client/client_single_latency.cpp", "tests/client/client_concurrent_run_latencies.cpp",
+                                    "tests/client/client_concurrent_run_latencies_set_load.cpp"])
+def test_reference_client_programs_compile_against_these_headers(source):
+    """The client API is a drop-in boundary: the reference's own load generator and client test programs must compile
+    unchanged against include/llis/client/*.h (syntax and types only; nothing of the reference is built or run)."""
+    import subprocess
+    path = os.path.join(REFERENCE, source)
+    if not os.path.exists(path):
+        pytest.skip(source + " is not in this copy of the reference")
+    out = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I" + os.path.join(ROOT, "include"), path], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr[-3000:]

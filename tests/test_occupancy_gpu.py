@@ -14,7 +14,7 @@ def model_blocks_per_cu(threads, regs, lds, caps):
     from paella_amd import _abi
     lib = ctypes.CDLL(os.path.join(_abi.LIB_DIR, "libllis_server.so"), mode=ctypes.RTLD_GLOBAL)
     lib.llis_sm_resources_blocks_per_cu.restype = ctypes.c_uint
-    return lib.llis_sm_resources_blocks_per_cu(threads, regs, lds, caps.lds_bytes_per_cu, caps.max_blocks_per_cu)
+    return lib.llis_sm_resources_blocks_per_cu(threads, regs, lds, caps.lds_bytes_per_cu, 32)
 
 
 @pytest.fixture(scope="module")
@@ -23,8 +23,7 @@ def caps(cuda):
     c = _abi.DeviceCaps()
     _abi.check(_abi.hip().llis_hip_get_device_caps(ctypes.byref(c)))
     # the constants the model is written in
-    assert c.wavefront_size == 64 and c.vgprs_per_cu == 4 * 512 * 64 and c.max_threads_per_cu == 4 * 8 * 64
-    assert c.lds_bytes_per_cu == 160 * 1024
+    assert c.wavefront_size == 64 and c.max_threads_per_cu == 4 * 8 * 64 and c.lds_bytes_per_cu == 160 * 1024
     return c
 
 
@@ -36,10 +35,11 @@ FAMILIES = [("dense", 256), ("dense_long", 512), ("pool", 256), ("gap", 256), ("
 def test_memory_bound_kernels(caps, family, block):
     from paella_amd import _abi
     lib = _abi.ops()
-    regs, got = ctypes.c_uint(), ctypes.c_int()
+    regs, lds, got = ctypes.c_uint(), ctypes.c_uint(), ctypes.c_int()
     _abi.check(lib.paella_kernel_vgprs(family.encode(), ctypes.byref(regs)))
+    _abi.check(lib.paella_kernel_static_lds(family.encode(), ctypes.byref(lds)))
     _abi.check(lib.paella_kernel_occupancy(family.encode(), block, 0, ctypes.byref(got)))
-    assert model_blocks_per_cu(block, regs.value, 0, caps) == got.value, (family, regs.value)
+    assert model_blocks_per_cu(block, regs.value, lds.value, caps) == got.value, (family, regs.value, lds.value)
 
 
 def conv_variants():
@@ -64,9 +64,9 @@ def test_conv_kernels_with_the_planner_lds(caps, kind, form, mi, ni, kw, k_order
     block = 256 if kind == 1 else 64 * kw
     red = 0 if (kind == 1 or kw == 1) else kw * mi * ni * 16 * 64 * 4
     for lds in sorted({red, max(red, 40 * 1024)} if (kind == 0 and k_order == 0) else {red}):
-        regs, got = ctypes.c_uint(), ctypes.c_int()
-        _abi.check(lib.paella_conv_kernel_occupancy(kind, form, mi, ni, kw, k_order, lds, ctypes.byref(got), ctypes.byref(regs)))
-        assert model_blocks_per_cu(block, regs.value, lds, caps) == got.value, (regs.value, lds)
+        regs, static, got = ctypes.c_uint(), ctypes.c_uint(), ctypes.c_int()
+        _abi.check(lib.paella_conv_kernel_occupancy(kind, form, mi, ni, kw, k_order, lds, ctypes.byref(got), ctypes.byref(regs), ctypes.byref(static)))
+        assert model_blocks_per_cu(block, regs.value, lds + static.value, caps) == got.value, (regs.value, lds, static.value)
 
 
 def test_every_zoo_stage_reports_registers_and_fits_the_device(caps):

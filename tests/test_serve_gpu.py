@@ -26,7 +26,8 @@ def device_budget():
     caps = _abi.DeviceCaps()
     _abi.check(_abi.hip().llis_hip_get_device_caps(ctypes.byref(caps)))
     n = caps.num_cus
-    return (n * caps.vgprs_per_cu, n * caps.lds_bytes_per_cu, n * caps.max_threads_per_cu, n * caps.max_blocks_per_cu)
+    # register lanes and wave slots in the hardware's units: 4 SIMDs x 512 registers x 64 lanes, 4 x 8 waves of 64
+    return (n * 4 * 512 * 64, n * caps.lds_bytes_per_cu, n * 4 * 8 * 64, n * 32)
 
 
 def close(got, ref):

@@ -162,3 +162,36 @@ print(json.dumps({"rps": r["throughput_rps"], "count": r["all"]["count"], "out":
     assert out.returncode == 0, out.stderr
     res = json.loads(out.stdout.strip().splitlines()[-1])
     assert res["count"] == 200 and res["out"] == [6, 6, 6, 6] and res["log_lines"] > 1000
+
+
+def test_server_outlives_a_client_killed_mid_run(tmp_path):
+    """A client that dies with requests in flight leaves wake-ups nobody will ever read: the server writes them off
+    after the peer has refused them for two seconds, and a second client is served as if nothing had happened."""
+    name = "ptdead%d" % os.getpid()
+    srv = start_server(name, "full3", FAKE_HIP_OP_US="20")
+    victim = None
+    try:
+        args = ["--server_name", name, "--iat", "100", "--dist", "exp", "--concurrency", "32", "--seed", "1", "--no_pin"]
+        jobs = [fake_job("fake_short"), "0.7", "16", fake_job("fake_mem3"), "0.3", "16"]
+        victim = subprocess.Popen([os.path.join(BIN, "llis_app_client")] + args + ["--num_jobs", "2000000", "--prefix", str(tmp_path / "a")] + jobs,
+                                  env=fake_env(LLIS_CLIENT_KEEP_SERVER="1"), stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        time.sleep(0.5)
+        assert victim.poll() is None, "the first client should still be submitting"
+        victim.kill()
+        victim.wait()
+        time.sleep(2.5)  # longer than the server's patience with a peer that refuses every wake-up
+        assert srv.poll() is None, srv.stderr.read()
+        out = subprocess.run([os.path.join(BIN, "llis_app_client")] + args + ["--num_jobs", "400", "--prefix", str(tmp_path / "b")] + jobs,
+                             env=fake_env(), capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        stats = json.loads(out.stdout.strip().splitlines()[-1])
+        assert stats["num_jobs"] == 400 and sum(stats["per_type_count"]) == 400
+        assert srv.wait(timeout=30) == 0
+    finally:
+        for p in (victim, srv):
+            if p is not None and p.poll() is None:
+                p.kill()
+                p.wait()
+        for f in os.listdir("/dev/shm"):
+            if name in f:
+                os.unlink(os.path.join("/dev/shm", f))
