@@ -98,6 +98,22 @@ int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const voi
                          const float* residual, const float* slope, float* y, void* workspace,
                          void* stream, uint32_t job_id, void* notifier);
 
+/* paella_conv2d_launch for callers that cannot allocate and have no workspace to bring (code under stream capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the split reduction's counters and partial tiles live in a
+ * fixed array inside the library's device image (PAELLA_CONV_STATIC_WORKSPACE_BYTES per GPU, there from load to
+ * process end) instead of a caller-supplied workspace.  No counterpart in the reference.  Same kernels, same results
+ * bit for bit as paella_conv2d_launch.  Performs no device or host allocation.  Limits: plan->workspace_bytes must
+ * not exceed PAELLA_CONV_STATIC_WORKSPACE_BYTES (PAELLA_ETOOBIG otherwise, nothing launched); `stream` must be a HIP
+ * stream, not a direct-dispatch queue (PAELLA_ENOSUP); all calls on one GPU share the one array, so two calls that may
+ * overlap in time on that GPU (different streams, no dependency between them) race -- serialise them.  Every call
+ * first zeroes the counters it will use with a small fill kernel on `stream` (the array keeps whatever the last
+ * call, or an interrupted one, left behind). */
+#define PAELLA_CONV_STATIC_WORKSPACE_BYTES (4u << 20)
+#define PAELLA_ETOOBIG (-4)  /* the request exceeds a fixed capacity of the library */
+int paella_conv2d_launch_static(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
+                                const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
+                                void* notifier);
+
 /* The same conv on a transformed input: x' = in_act(x * in_scale[c] + in_shift[c]) per input channel c, with the
  * zero padding applied AFTER the transform (a padding tap contributes 0, not in_act(in_shift[c])); in_act is
  * PAELLA_ACT_NONE or PAELLA_ACT_RELU.  This is a batch-norm (+ ReLU) stage that stands in front of a conv and cannot

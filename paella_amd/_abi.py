@@ -103,6 +103,7 @@ OPS_SYMBOLS = {
     "paella_lrn_launch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_float] + _TAIL),
     "paella_kernel_vgprs": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv_kernel_vgprs": (c_int, [c_int] * 4 + [ctypes.POINTER(c_uint)]),
+    "paella_conv2d_launch_static": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 6 + _TAIL),
     "paella_kernel_occupancy": (c_int, [c_char_p, c_uint, c_uint, ctypes.POINTER(c_int)]),
     "paella_conv_kernel_occupancy": (c_int, [c_int] * 6 + [c_uint, ctypes.POINTER(c_int), ctypes.POINTER(c_uint), ctypes.POINTER(c_uint)]),
     "paella_kernel_static_lds": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),

@@ -23,6 +23,8 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
+#include <mutex>
 
 #include <cstdio>
 #include <cstdlib>
@@ -995,6 +997,62 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.notifier = nf;
     paella::launch(dwconv_kernel, dim3(plan->dims.grid), dim3(256), 0, st, a);
     return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Allocation-free variant: the split-reduction workspace is a fixed array of the device image.  The array's name is a
+// host-side handle, not a device address: each GPU holds its own copy, whose address is looked up once per device.
+
+static __device__ __align__(256) unsigned char scratch[PAELLA_CONV_STATIC_WORKSPACE_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+__global__ __launch_bounds__(256) void zero_words_kernel(unsigned* p, unsigned n) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// Device address of this GPU's copy of `scratch` (looked up on the first call per device, with that device current).
+int static_workspace(void** out) {
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return PAELLA_ENOSUP;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return (int)e;
+            if (!p) return (int)hipErrorInvalidSymbol;
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int paella_conv2d_launch_static(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
+                                           const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
+                                           void* notifier) {
+    if (!plan) return PAELLA_EINVAL;
+    if (plan->workspace_bytes > PAELLA_CONV_STATIC_WORKSPACE_BYTES) return PAELLA_ETOOBIG;
+    if (paella::direct_queue_lookup(stream)) return PAELLA_ENOSUP;  // the counter fill below needs stream order
+    void* ws = nullptr;
+    if (plan->workspace_bytes) {
+        if (int rc = static_workspace(&ws)) return rc;
+        // One arrival counter per output tile, at the head of the workspace.
+        const unsigned tiles = plan->dims.grid / (unsigned)plan->splits;
+        hipLaunchKernelGGL(zero_words_kernel, dim3((tiles + 255u) / 256u), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                           reinterpret_cast<unsigned*>(ws), tiles);
+        if (hipError_t e = hipGetLastError()) return (int)e;
+    }
+    return paella_conv2d_launch(plan, x, blob_dev, bias, residual, slope, y, ws, stream, job_id, notifier);
 }
 
 typedef void (*ConvPreKernel)(ConvPreArgs);
