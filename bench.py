@@ -242,9 +242,9 @@ class Arm:
     """One way of serving the mix: a scheduler behind the server (with a launch path for the model kernels), or the
     direct no-server multi-stream loop.  run() serves `n` requests at mean inter-arrival `iat_us` (0 = saturation)."""
 
-    def __init__(self, serve, label, sched, dispatch, streams, tenants, extra_kernels):
+    def __init__(self, serve, label, sched, dispatch, streams, tenants, extra_kernels, unfair=1e6):
         self.serve, self.label, self.sched, self.dispatch, self.streams = serve, label, sched, dispatch, streams
-        self.tenants, self.extra_kernels = tenants, extra_kernels
+        self.tenants, self.extra_kernels, self.unfair = tenants, extra_kernels, unfair
         self.cap = sum(t[4] for t in tenants)
         self.srv = None
 
@@ -252,7 +252,7 @@ class Arm:
         if self.sched != "direct":
             os.environ["PAELLA_DISPATCH"] = self.dispatch
             name = "bench%d_%s_%d" % (os.getpid(), self.sched, int(time.time() * 1000) % 100000)
-            self.srv = self.serve.Server(name, self.sched, num_streams=self.streams, cpu=4, extra_kernels=self.extra_kernels)
+            self.srv = self.serve.Server(name, self.sched, num_streams=self.streams, cpu=4, extra_kernels=self.extra_kernels, unfair=self.unfair)
             self.srv.__enter__()
         return self
 
@@ -338,6 +338,7 @@ def main():
     ap.add_argument("--num-streams", type=int, default=128)
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--extra-kernels", type=int, default=16, help="full3: kernels admitted beyond the occupancy budget")
+    ap.add_argument("--unfair", type=float, default=1e6, help="full3: deficit threshold of the headline arm (1e6 = shortest remaining work first only)")
     ap.add_argument("--no-arms", action="store_true", help="only the headline search and timed run (plus roofline and CPU baseline)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-side", action="store_true", help="skip the side workloads (other configurations, fairness sweep, probes)")
@@ -440,7 +441,7 @@ def main():
 
     # ---- headline: full3, kernels on direct dispatch
     searches = {}
-    with Arm(serve, "full3", "full3", "direct", streams, tenants, ek) as arm:
+    with Arm(serve, "full3", "full3", "direct", streams, tenants, ek, unfair=args.unfair) as arm:
         rate, sat, pts = search_rate(arm, tenants, slo_us)
         searches["full3"] = {"saturation_rps": sat, "points": pts, "rate_at_slo_rps": rate}
         if rate is None:

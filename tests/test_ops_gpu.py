@@ -304,13 +304,20 @@ def test_conv2d_rejects_what_it_does_not_implement(cuda):
         ops.Conv2d(rnd(8, 8, 3, 3), None, stride=0, in_hw=(8, 8))
 
 
-@pytest.mark.parametrize("c,h,w,r,stride,pad", [(32, 112, 112, 3, 1, 1), (96, 112, 112, 3, 2, 1), (960, 7, 7, 3, 1, 1),
-                                                 (7, 13, 9, 3, 2, 1), (16, 20, 20, 5, 1, 2)])
-def test_depthwise_conv_parity(cuda, c, h, w, r, stride, pad):
+# every depthwise layer shape of MobileNetV2 and of the face detector's backbone, plus ragged cases: odd widths, two channels, a
+# filter larger than the image, dilation, no padding, a very wide image
+DEPTHWISE = [(32, 112, 112, 3, 1, 1, 1), (96, 112, 112, 3, 2, 1, 1), (144, 56, 56, 3, 1, 1, 1), (144, 56, 56, 3, 2, 1, 1), (192, 28, 28, 3, 1, 1, 1),
+             (192, 28, 28, 3, 2, 1, 1), (384, 14, 14, 3, 1, 1, 1), (576, 14, 14, 3, 2, 1, 1), (960, 7, 7, 3, 1, 1, 1), (16, 120, 160, 3, 2, 1, 1),
+             (64, 30, 40, 3, 1, 1, 1), (7, 13, 9, 3, 2, 1, 1), (16, 20, 20, 5, 1, 2, 1), (2, 5, 3, 3, 1, 1, 1), (3, 2, 2, 3, 1, 1, 1), (5, 17, 31, 3, 1, 2, 2),
+             (9, 11, 11, 3, 1, 0, 1), (2, 1, 1, 3, 1, 1, 1), (33, 9, 600, 3, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("c,h,w,r,stride,pad,dil", DEPTHWISE)
+def test_depthwise_conv_parity(cuda, c, h, w, r, stride, pad, dil):
     from paella_amd import ops
     x, wt, b = rnd(1, c, h, w), rnd(c, 1, r, r, scale=0.3), rnd(c, scale=0.1)
-    ref = orc.conv2d(x, wt, b, stride=stride, pad=pad, groups=c, act=orc.ACT_RELU6)
-    conv = ops.Conv2d(wt, b, stride=stride, pad=pad, groups=c, act=ops.ACT_RELU6, in_hw=(h, w))
+    ref = orc.conv2d(x, wt, b, stride=stride, pad=pad, dil=dil, groups=c, act=orc.ACT_RELU6)
+    conv = ops.Conv2d(wt, b, stride=stride, pad=pad, dil=dil, groups=c, act=ops.ACT_RELU6, in_hw=(h, w))
     assert conv.plan.kind == 1
     close(conv(torch.tensor(x, device=cuda)), ref)
 
