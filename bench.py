@@ -466,7 +466,8 @@ def main():
     # ---- the same search for plain multi-stream serving, served (fifo, job by job on HIP streams) and without a server
     arms_at_equal_load, equal_rate = {}, None
     if not args.no_arms:
-        for label, sched, dispatch, nstreams in [("fifo_multi_stream", "fifo", "hip", cap), ("direct_multi_stream", "direct", "hip", cap)]:
+        for label, sched, dispatch, nstreams in [("fifo2_direct_dispatch", "fifo2", "direct", streams), ("fifo_multi_stream", "fifo", "hip", cap),
+                                                 ("direct_multi_stream", "direct", "hip", cap)]:
             with Arm(serve, label, sched, dispatch, nstreams, tenants, ek) as arm:
                 rate_b, sat_b, pts_b = search_rate(arm, tenants, slo_us)
                 searches[label] = {"saturation_rps": sat_b, "points": pts_b, "rate_at_slo_rps": rate_b}

@@ -102,6 +102,14 @@ class FinishedBlockNotifier {
             if (timed && measure_block_time_) send_block_time();  // the member is looked at only when timing was asked for
         }
     }
+
+    // The same again for kernels that find out by themselves when every wave of the workgroup has had its write-through
+    // stores acknowledged (say, by counting waves in LDS): the ONE lane that establishes it calls this, no barrier is
+    // involved, and the other waves may have left the compute unit already.
+    __device__ __forceinline__ void end_from_one_lane(JobId job_id, bool timed) {
+        announce<false>(&agg_counter_end_, 0, job_id);
+        if (timed && measure_block_time_) send_block_time();
+    }
 #endif
 
     // Allocates `num` notifiers in device memory, all bound to the given ring (and, when given, to the ring

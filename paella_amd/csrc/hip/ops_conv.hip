@@ -112,6 +112,10 @@ template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
     paella::hook_entry(p.notifier, p.job_id);
+    // Waves of this workgroup whose result stores have been acknowledged (see the end of this function); cleared here, and
+    // the barrier of the cross-wave sum lies between this store and the first increment.
+    __shared__ unsigned waves_done;
+    if (KW > 1 && threadIdx.x == 0) waves_done = 0;
 
     // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
     extern __shared__ __align__(16) char smem[];
@@ -450,7 +454,19 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
     }
 
-    paella::hook_exit(p.notifier, p.job_id);
+    // End hook without a barrier: every wave waits for its own write-through stores, then counts itself in LDS; the wave that
+    // completes the count reports the workgroup, the others leave the compute unit at once instead of waiting for the report's
+    // round trip to the counter in memory (the wave slots they hold are what other workgroups are waiting for).
+    if (p.notifier) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        bool last = true;
+        if (KW > 1) {
+            unsigned before = 0;
+            if (lane == 0) before = __hip_atomic_fetch_add(&waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            last = __builtin_amdgcn_readfirstlane(before) == (unsigned)KW - 1;
+        }
+        if (last && lane == 0) p.notifier->end_from_one_lane(p.job_id & ~PAELLA_JOB_ID_FLAGS, (p.job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0);
+    }
 }
 
 template <int MI, int NI, int KW, bool TAP_MAJOR>
