@@ -92,6 +92,8 @@ class ModelJob : public llis::job::CoroutineJob {
         zero_in_ = !input_resident_ && in_bytes_ <= zero_copy_limit && paella_exec_bind_input(exec_, staging_) == 0;
         zero_out_ = out_bytes_ <= zero_copy_limit && paella_exec_bind_output(exec_, staging_ + out_off_) == 0;
         timed_ = llis::job::Context::get_gpu2sched_block_time_channel()->is_connected();  // server runs with --measure_block_time
+        const char* starts = std::getenv("PAELLA_UNFIT_STARTS");
+        unfit_starts_ = starts && std::strcmp(starts, "1") == 0;
         const char* dispatch = std::getenv("PAELLA_DISPATCH");
         direct_ = !(dispatch && std::strcmp(dispatch, "hip") == 0) && llis::job::Context::is_stage_by_stage();
         if (direct_) {
@@ -131,8 +133,10 @@ class ModelJob : public llis::job::CoroutineJob {
             if (zero_out_ && last == num_stages_ - 1) set_pre_notify();
             yield();
             if (zero_in_ && s == 0) std::memcpy(staging_, io_ptr, in_bytes_);
-            // Only a kernel admitted beyond the occupancy budget ("unfit") needs its workgroup starts reported.
-            const uint32_t id = get_id() | (is_unfit() ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
+            // Workgroup starts are reported only on request (PAELLA_UNFIT_STARTS=1), and then only by a kernel admitted beyond
+            // the occupancy budget ("unfit"), whose over-subscription credit full3 returns once all its workgroups are resident;
+            // without start messages the credit returns when the kernel ends (reference src/server/scheduler_full3.cpp:196-204).
+            const uint32_t id = get_id() | (is_unfit() && unfit_starts_ ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
             void* target = stream();
             if (direct_) check(paella_direct_queue_shared(&target), "direct queue");
             for (int k = s; k <= last; ++k) {
@@ -175,6 +179,7 @@ class ModelJob : public llis::job::CoroutineJob {
     std::vector<int> group_end_;   // per kernel: index of the last kernel of the group it is issued with
     bool direct_ = true;
     bool timed_ = false;
+    bool unfit_starts_ = false;
     bool input_resident_ = false, input_uploaded_ = false;
     bool zero_in_ = false, zero_out_ = false;
 };

@@ -102,6 +102,37 @@ def test_vec_add_at_the_reference_batch_size_sends_13_plus_13_messages_per_kerne
     assert sorted(nums) == sorted(10 * ([64] * 3 + [8]))
 
 
+@pytest.mark.parametrize("starts", ["0", "1"])
+def test_over_budget_kernels_report_starts_only_on_request(cuda, starts):
+    """ResNet-18 under full3 with several requests in flight: kernels admitted beyond the occupancy budget report their
+    workgroup starts only with PAELLA_UNFIT_STARTS=1 (the credit then returns at full residency, otherwise at the kernel's
+    end: reference src/server/scheduler_full3.cpp:123-144 and :196-204); the answers are the same either way."""
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    desc = models.describe("resnet18")
+    x = om.make_input(desc, 3, "normal")
+    ref = om.run(desc, x, seed=1)
+    old = os.environ.get("PAELLA_UNFIT_STARTS")
+    os.environ["PAELLA_UNFIT_STARTS"] = starts
+    try:
+        with serve.Server(server_name("starts" + starts), "full3", num_streams=64, extra_kernels=16, event_log=True) as srv:
+            jobs = [(serve.job_path("tvm_resnet18"), 1.0, 12)]
+            r = serve.client_run(srv.name, jobs, 0.0, 12, 300, warmup_jobs=50)
+            out, _ = serve.client_single(srv.name, serve.job_path("tvm_resnet18"), x, ref.size, n=2)
+    finally:
+        if old is None:
+            os.environ.pop("PAELLA_UNFIT_STARTS", None)
+        else:
+            os.environ["PAELLA_UNFIT_STARTS"] = old
+    close(out, ref)
+    assert r["all"]["count"] == 300
+    ev = sched.parse_log(srv.event_log())
+    unfit_dispatches = sum(1 for e in ev if e[0] == "D" and e[6] == 1)
+    start_messages = sum(1 for e in ev if e[0] == "B" and e[2] == 1)
+    assert unfit_dispatches > 0, "twelve requests in flight must over-subscribe the budget"
+    assert (start_messages > 0) == (starts == "1")
+
+
 def test_plain_job_with_raw_hooks(cuda):
     from paella_amd import serve
     with serve.Server(server_name("hello"), "full3", num_streams=4, event_log=True) as srv:
