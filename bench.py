@@ -54,7 +54,7 @@ def log(*a):
 # HBM-side bytes per conv launch (mean over the conv launches of one forward pass), from FETCH_SIZE / WRITE_SIZE
 # counter passes of `bench.py --counter-pass MODEL` scaled by the copy-kernel calibration (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); counters cannot be collected from inside this process, so the figures are carried here.
-CONV_TRAFFIC_BYTES_PER_LAUNCH = {"resnet18": 7.10e6}
+CONV_TRAFFIC_BYTES_PER_LAUNCH = {"inception_v3": 10.08e6, "resnet18": 7.13e6, "resnet50": 6.99e6, "mobilenetv2": 1.85e6}
 
 
 def under_counter_collection():
@@ -288,19 +288,25 @@ def meets(point, tenants, slo_us):
     return all(point[t[0] + "_p99_us"] <= slo_us[t[0]] for t in tenants)
 
 
-def search_rate(arm, tenants, slo_us, iters=6):
+def search_rate(arm, tenants, slo_us, iters=7):
     """Highest offered rate (open-loop Poisson) at which every tenant's p99 meets its SLO and the served rate keeps up:
-    closed-loop saturation first, then bisection on the fraction of it.  Returns (rate or None, saturation, points)."""
+    closed-loop saturation first, then bisection on the fraction of it.  A point that misses is measured a second time with
+    another arrival seed before it counts as a miss (one stall of a host thread is enough to spoil the p99 of a 10 000-request
+    point).  Returns (rate or None, saturation, points)."""
     sat = arm.run(0.0, SEARCH_REQUESTS, 512)["throughput_rps"]
     points, lo, hi = [], 0.0, 1.0
     f = 0.5
     for _ in range(iters):
         rate = f * sat
-        p = point_of(arm.run(1e6 / rate, SEARCH_REQUESTS, 512), tenants, rate)
-        p["meets_slo"] = meets(p, tenants, slo_us)
-        points.append(p)
-        log("[bench]     %-22s offered %8.0f req/s: served %8.0f, p99 %s -> %s" %
-            (arm.label, rate, p["achieved_rps"], " / ".join("%.0f" % p[t[0] + "_p99_us"] for t in tenants), "ok" if p["meets_slo"] else "miss"))
+        for attempt, seed in enumerate((1, 2)):
+            p = point_of(arm.run(1e6 / rate, SEARCH_REQUESTS, 512, seed=seed), tenants, rate)
+            p["meets_slo"] = meets(p, tenants, slo_us)
+            p["attempt"] = attempt
+            points.append(p)
+            log("[bench]     %-22s offered %8.0f req/s: served %8.0f, p99 %s -> %s" %
+                (arm.label, rate, p["achieved_rps"], " / ".join("%.0f" % p[t[0] + "_p99_us"] for t in tenants), "ok" if p["meets_slo"] else "miss"))
+            if p["meets_slo"] or p["achieved_rps"] < KEEP_UP * rate:
+                break  # met, or plainly beyond what can be served: no second look
         if p["meets_slo"]:
             lo = f
         else:
