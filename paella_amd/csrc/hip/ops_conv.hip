@@ -695,7 +695,7 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             while (kw < kw_max && kw < nchunks) kw <<= 1;
         }
         // Grid-level split of the reduction: layers with few output tiles (small feature maps) would otherwise
-        // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU, keep >= 4 chunks per wave.
+        // occupy a fraction of the 256 CUs.  Aim at about one workgroup per CU and keep a minimum of chunks per wave (below).
         // Measured on ResNet-18 with four passes in flight / one pass alone (thousand passes per second), by the cap
         // on workgroups and the waves per workgroup: 288 x 8: 15.2 / 6.9;
         // 288 x 4: 14.5 / 6.1; 144 x 8: 13.7 / 6.1; 144 x 4: 11.9 / 5.1; 576 x 8: 13.8 / 6.0.
@@ -705,11 +705,15 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             splits = 1 << ((tile_hint >> 12) & 0xF);
         } else {
             const int cap = 288;
-            // Layers of at most 32 tiles (DenseNet's and MobileNetV2's deep, narrow convs on 14 x 14 and 7 x 7 maps) go down to
-            // 2 chunks per wave: with four passes in flight / alone, DenseNet-121 4.09 -> 4.44 / 1.31 -> 1.38 thousand passes per
-            // second, MobileNetV2 14.5 -> 15.5 / 4.82 -> 4.91, Inception-v3 4.84 -> 4.78 / 2.33 -> 2.32, ResNet-18 and -50,
-            // GoogLeNet and SqueezeNet within the run-to-run spread; 2 everywhere costs Inception-v3 5 %.
-            const int min_chunks = n_tiles <= 32 ? 2 : 4;
+            // How far the split goes is a trade between a kernel's latency (more, smaller workgroups) and the fixed cost of a
+            // workgroup and of the exchange of partial tiles (fewer, larger ones).  Layers under 16 MFLOP go down to 2 chunks per
+            // wave, the others keep 6.  Served by full3 at saturation, median of three runs, requests/s against the earlier rule
+            // (2 chunks for layers of at most 32 tiles, 4 otherwise): Inception-v3 4310 -> 4630, ResNet-50 5490 -> 5605,
+            // GoogLeNet 9520 -> 9500, MobileNetV2 8390 -> 8240, DenseNet-121 3650 -> 3540 (its 25-50 MFLOP pointwise layers on
+            // 14 x 14 maps are a pure chain and would rather be split), small CNN : Inception-v3 = 9 : 1 35.9 -> 37.1 thousand;
+            // four passes in flight without scheduler: Inception-v3 4.81 -> 5.00 thousand passes/s; one launch at a time 9.09 ->
+            // 9.20 us.  Thresholds of 32 and 64 MFLOP gave Inception-v3 4617 and 4443; 5 or 8 chunks instead of 6: 4552, 4588.
+            const int min_chunks = plan->flops < 16e6 ? 2 : 6;
             while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= min_chunks) splits *= 2;
         }
         int chunks_per_split = (nchunks + splits - 1) / splits;
