@@ -4,6 +4,7 @@
 // (reference jobs/tvm_mnist/tvm_mnist.cpp:41 through the TVM runtime); on this platform the equivalent HIP
 // call is the dominant cost of that thread, so the model adapters submit their kernels here instead.
 
+#include <immintrin.h>
 #include "direct_dispatch.h"
 
 #include "paella_ops.h"
@@ -168,6 +169,7 @@ struct DirectQueue {
     hsa_queue_t* queue = nullptr;
     char* kernargs = nullptr;
     uint64_t write_index = 0;  // single producer: the thread that owns the queue
+    uint64_t read_seen = 0;    // read index when this thread last looked
     bool device_kernargs = false;  // kernarg ring lives in device memory, written through the PCIe aperture
     bool ordered = false;      // barrier bit on every packet: kernels run one after the other, like a stream
 };
@@ -212,12 +214,35 @@ const DirectKernel* direct_kernel(const void* host_function) {
     std::abort();
 }
 
+// Copies whole 64-byte lines to write-combining memory (the argument ring behind the PCIe aperture) with the widest
+// streaming store the host has; both pointers 64-byte aligned.
+__attribute__((target("avx512f"))) static void stream_lines_512(char* dst, const char* src, size_t lines) {
+    for (size_t i = 0; i < lines; ++i) _mm512_stream_si512(reinterpret_cast<__m512i*>(dst + i * 64), _mm512_load_si512(src + i * 64));
+}
+__attribute__((target("avx"))) static void stream_lines_256(char* dst, const char* src, size_t lines) {
+    for (size_t i = 0; i < lines * 2; ++i)
+        _mm256_stream_si256(reinterpret_cast<__m256i*>(dst + i * 32), _mm256_load_si256(reinterpret_cast<const __m256i*>(src + i * 32)));
+}
+static void stream_lines_128(char* dst, const char* src, size_t lines) {
+    for (size_t i = 0; i < lines * 4; ++i)
+        _mm_stream_si128(reinterpret_cast<__m128i*>(dst + i * 16), _mm_load_si128(reinterpret_cast<const __m128i*>(src + i * 16)));
+}
+void stream_lines(char* dst, const char* src, size_t lines) {
+    static const int width = __builtin_cpu_supports("avx512f") ? 512 : __builtin_cpu_supports("avx") ? 256 : 128;
+    if (width == 512) stream_lines_512(dst, src, lines);
+    else if (width == 256) stream_lines_256(dst, src, lines);
+    else stream_lines_128(dst, src, lines);
+}
+
 void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3 block, unsigned dynamic_lds, const void* explicit_args,
                      size_t explicit_bytes) {
     hsa_queue_t* hq = q->queue;
     const uint64_t index = q->write_index;
     // Ring full: wait for the packet processor (it drains without any action from this thread).
-    while (index - hsa_queue_load_read_index_scacquire(hq) >= hq->size) {
+    // (The read index is a line the device writes: it is looked at again only when the copy kept here says the ring is full.)
+    if (index - q->read_seen >= hq->size) {
+        while (index - (q->read_seen = hsa_queue_load_read_index_scacquire(hq)) >= hq->size) {
+        }
     }
     const uint32_t slot = (uint32_t)(index & (hq->size - 1));
 
@@ -231,8 +256,11 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
         std::fprintf(stderr, "[paella] direct dispatch: %zu argument bytes for a kernel that takes %u\n", explicit_bytes, kernel->kernarg_bytes);
         std::abort();
     }
-    std::memcpy(ka, explicit_args, explicit_bytes);
-    if (implicit_at > explicit_bytes) std::memset(ka + explicit_bytes, 0, implicit_at - explicit_bytes);
+    // The block is put together in cached memory and goes out in whole 64-byte lines, in ascending order, with streaming
+    // stores: written in pieces, a line leaves the core's write-combining buffers as several partial transactions
+    // (host time of the 51 launches of an Inception-v3 pass, argument ring warm: 36.5 us in pieces, 28.7 us this way).
+    alignas(64) char stage[kKernargSlotBytes];
+    std::memcpy(stage, explicit_args, explicit_bytes);
     struct Implicit {
         uint32_t block_count[3];
         uint16_t group_size[3];
@@ -246,19 +274,29 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     };
     static_assert(sizeof(Implicit) == kImplicitBytes, "implicit kernel argument block is 256 bytes");
     static_assert(offsetof(Implicit, global_offset) == 40 && offsetof(Implicit, grid_dims) == 64 && offsetof(Implicit, dynamic_lds) == 120, "layout");
-    Implicit imp;
-    std::memset(&imp, 0, sizeof(imp));
-    imp.block_count[0] = grid.x;
-    imp.block_count[1] = grid.y;
-    imp.block_count[2] = grid.z;
-    imp.group_size[0] = (uint16_t)block.x;
-    imp.group_size[1] = (uint16_t)block.y;
-    imp.group_size[2] = (uint16_t)block.z;
-    imp.grid_dims = grid.z > 1 ? 3 : (grid.y > 1 ? 2 : 1);
-    imp.dynamic_lds = dynamic_lds;
+    size_t total = explicit_bytes;
     if (kernel->kernarg_bytes > implicit_at) {
+        std::memset(stage + explicit_bytes, 0, implicit_at - explicit_bytes);
+        Implicit imp;
+        std::memset(&imp, 0, sizeof(imp));
+        imp.block_count[0] = grid.x;
+        imp.block_count[1] = grid.y;
+        imp.block_count[2] = grid.z;
+        imp.group_size[0] = (uint16_t)block.x;
+        imp.group_size[1] = (uint16_t)block.y;
+        imp.group_size[2] = (uint16_t)block.z;
+        imp.grid_dims = grid.z > 1 ? 3 : (grid.y > 1 ? 2 : 1);
+        imp.dynamic_lds = dynamic_lds;
         const size_t n = kernel->kernarg_bytes - implicit_at;
-        std::memcpy(ka + implicit_at, &imp, n < sizeof(imp) ? n : sizeof(imp));
+        std::memcpy(stage + implicit_at, &imp, sizeof(imp));
+        total = implicit_at + (n < sizeof(imp) ? n : sizeof(imp));
+    }
+    if (q->device_kernargs) {
+        const size_t lines = (total + 63) / 64;
+        std::memset(stage + total, 0, lines * 64 - total);  // the tail of the last line is padding inside the slot
+        stream_lines(ka, stage, lines);
+    } else {
+        std::memcpy(ka, stage, total);
     }
 
     if (q->device_kernargs) __builtin_ia32_sfence();  // write-combined stores out before the doorbell
@@ -338,7 +376,14 @@ extern "C" int paella_direct_queue_create(void** out) {
             hsa_amd_memory_pool_free(ka);
             ka = nullptr;
         }
-        if (st == HSA_STATUS_SUCCESS) q->device_kernargs = true;
+        if (st == HSA_STATUS_SUCCESS) {
+            q->device_kernargs = true;
+            // Touch every page of the ring now: the first store to a page of the aperture takes a fault (1600 against 400
+            // cycles per launch until the ring has wrapped once).
+            alignas(64) static const char zeros[64] = {0};
+            for (size_t off = 0; off < ka_bytes; off += 64) paella::stream_lines(reinterpret_cast<char*>(ka) + off, zeros, 1);
+            __builtin_ia32_sfence();
+        }
     }
     if (st != HSA_STATUS_SUCCESS) {
         st = hsa_amd_memory_pool_allocate(paella::g_rt.kernarg_pool, ka_bytes, 0, &ka);

@@ -206,7 +206,7 @@ void SchedulerFull3::schedule_job() {
         job::Context::set_current_job(job);
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_START);
         {
-            LLIS_PHASE(kLaunch);
+            LLIS_PHASE_IF(is_mem, kLaunchCopy, kLaunch);
             if (profiler_->recording_run_next_times()) {
                 const auto t0 = std::chrono::steady_clock::now();
                 job->run_next();
