@@ -37,7 +37,19 @@ class Context {
     static void set_stage_by_stage(bool v) { stage_by_stage_ = v; }
     static bool is_stage_by_stage() { return stage_by_stage_; }
 
+    // Functions the serving thread calls once per turn of its loop, after it has looked at its rings: for job libraries
+    // that hold work back and release it from that thread (a function is added once, however often it is registered).
+    // Not in the reference.
+    using PollHook = void (*)();
+    static void add_poll_hook(PollHook fn);
+    static void run_poll_hooks() {
+        for (unsigned i = 0; i < num_poll_hooks_; ++i) poll_hooks_[i]();
+    }
+
   private:
+    static constexpr unsigned kMaxPollHooks = 8;
+    static PollHook poll_hooks_[kMaxPollHooks];
+    static unsigned num_poll_hooks_;
     static bool stage_by_stage_;
     static Job* current_job_;
     static ipc::Gpu2SchedChannel gpu2sched_channel_;

@@ -56,10 +56,14 @@ class FinishedBlockNotifier {
     FinishedBlockNotifier& operator=(FinishedBlockNotifier&&) = default;
 
 #if defined(__HIPCC__)
-    __device__ __forceinline__ void start(JobId job_id) {
+    __device__ __forceinline__ void start(JobId job_id) { start(job_id, gridDim.x * gridDim.y * gridDim.z); }
+
+    // For a launch that carries the kernels of several jobs, each with a notifier of its own: `num_blocks` is the number
+    // of workgroups of the launch that report to THIS notifier (the same value in start and end calls of one kernel).
+    __device__ __forceinline__ void start(JobId job_id, unsigned num_blocks) {
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
             if (measure_block_time_) *entry_clock_slot() = (unsigned)wall_clock64() & 0xFFFFFFu;
-            announce<false>(&agg_counter_start_, 1, job_id);
+            announce<false>(&agg_counter_start_, 1, job_id, num_blocks);
         }
     }
 
@@ -107,7 +111,10 @@ class FinishedBlockNotifier {
     // stores acknowledged (say, by counting waves in LDS): the ONE lane that establishes it calls this, no barrier is
     // involved, and the other waves may have left the compute unit already.
     __device__ __forceinline__ void end_from_one_lane(JobId job_id, bool timed) {
-        announce<false>(&agg_counter_end_, 0, job_id);
+        end_from_one_lane(job_id, timed, gridDim.x * gridDim.y * gridDim.z);
+    }
+    __device__ __forceinline__ void end_from_one_lane(JobId job_id, bool timed, unsigned num_blocks) {
+        announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
         if (timed && measure_block_time_) send_block_time();
     }
 #endif
@@ -141,7 +148,10 @@ class FinishedBlockNotifier {
     // ACQUIRE: the sender first acquires (device scope) what the other workgroups released before their bump.
     template <bool ACQUIRE>
     __device__ __forceinline__ void announce(unsigned* counter, uint8_t is_start, JobId job_id) {
-        const unsigned num_blocks = gridDim.x * gridDim.y * gridDim.z;
+        announce<ACQUIRE>(counter, is_start, job_id, gridDim.x * gridDim.y * gridDim.z);
+    }
+    template <bool ACQUIRE>
+    __device__ __forceinline__ void announce(unsigned* counter, uint8_t is_start, JobId job_id, const unsigned num_blocks) {
         const unsigned mask = batch_mask_;  // requested before the atomic, so the two trips to memory overlap
         const unsigned total = atomicInc(counter, num_blocks - 1) + 1;  // wraps to 0 after the last block
         const unsigned in_batch = total & mask;

@@ -11,9 +11,9 @@ namespace llis {
 namespace server {
 
 struct PhaseClock {
-    enum Phase { kIdle, kRing, kRequests, kLaunch, kLaunchCopy, kCount };
-    unsigned long long cycles[kCount] = {0, 0, 0, 0, 0};
-    unsigned long long events[kCount] = {0, 0, 0, 0, 0};
+    enum Phase { kIdle, kRing, kRequests, kLaunch, kLaunchCopy, kHooks, kCount };
+    unsigned long long cycles[kCount] = {};
+    unsigned long long events[kCount] = {};
     static PhaseClock& get() {
         static PhaseClock clock;
         return clock;
@@ -21,7 +21,7 @@ struct PhaseClock {
     void report() const {
         unsigned long long total = 0;
         for (int i = 0; i < kCount; ++i) total += cycles[i];
-        static const char* const names[kCount] = {"idle polls", "ring messages (excl. launches)", "client requests (excl. launches)", "run_next of kernel stages", "run_next of copy stages + markers"};
+        static const char* const names[kCount] = {"idle polls", "ring messages (excl. launches)", "client requests (excl. launches)", "run_next of kernel stages", "run_next of copy stages + markers", "poll hooks of job libraries"};
         for (int i = 0; i < kCount; ++i)
             std::fprintf(stderr, "[phase] %-34s %6.2f %%  %10llu events  %8.0f cycles/event\n", names[i], 100.0 * cycles[i] / (total ? total : 1),
                          events[i], events[i] ? (double)cycles[i] / events[i] : 0.0);

@@ -153,8 +153,28 @@ int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_pla
 /* The same for 2 to PAELLA_CONV_GROUP_MAX convs, one problem's workgroups after the other's in the order given; every
  * pair of members must meet the conditions above. */
 #define PAELLA_CONV_GROUP_MAX 4
+/* Problems in one launch of the group kernel when the library packs several calls together (below). */
+#define PAELLA_CONV_PACK_MAX 8
 int paella_conv2d_group_dims(const paella_conv_plan* const* plans, int n, paella_launch_dims* dims);
 int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void* stream, uint32_t job_id, void* notifier);
+
+/* Launch packing.  A hardware queue of this device runs one kernel at a time and four run side by side, so at batch 1 a
+ * conv that fills a fifth of the compute units still occupies a queue for its whole latency.  After paella_pack_enable(1)
+ * on a thread, that thread's paella_conv2d_launch / paella_conv2d_launch_group calls on the 32 x 32 tile whose target is
+ * an UNORDERED direct-dispatch queue (the serving path: the scheduler orders a job's stages through the notification
+ * ring) are held back and sent together, up to PAELLA_CONV_PACK_MAX problems of any jobs in one grid, every problem
+ * reporting to its own job id and notifier exactly as if launched alone; results are bit-identical.  Everything else
+ * (HIP streams, ordered queues, other operators, larger tiles) is launched at once as before.  The thread must call
+ * paella_pack_poll() from its loop: it sends what is held as soon as a queue of the shared set (paella_direct_queue_shared)
+ * has no packet waiting, when a launch is full, or after 30 us at the latest, on the least loaded queue of that set, and
+ * returns the number of launches made (negative: error).  paella_pack_flush() sends everything now;
+ * paella_pack_enable(0) flushes and switches packing off.  paella_pack_stats: launches made by the packer and problems
+ * they carried so far in this process; returns the number of calls the calling thread currently holds.  No counterpart in the reference
+ * (its GPUs run kernels of one stream pool side by side without this limit). */
+int paella_pack_enable(int on);
+int paella_pack_poll(void);
+int paella_pack_flush(void);
+int paella_pack_stats(uint64_t* launches, uint64_t* members);
 int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second,
                               void* stream, uint32_t job_id, void* notifier);
 

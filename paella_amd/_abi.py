@@ -84,6 +84,10 @@ OPS_SYMBOLS = {
     "paella_conv2d_launch_pair": (c_int, [ctypes.POINTER(ConvOperands), ctypes.POINTER(ConvOperands)] + _TAIL),
     "paella_conv2d_group_dims": (c_int, [ctypes.POINTER(ctypes.POINTER(ConvPlan)), c_int, ctypes.POINTER(LaunchDims)]),
     "paella_conv2d_launch_group": (c_int, [ctypes.POINTER(ConvOperands), c_int] + _TAIL),
+    "paella_pack_enable": (c_int, [c_int]),
+    "paella_pack_poll": (c_int, []),
+    "paella_pack_flush": (c_int, []),
+    "paella_pack_stats": (c_int, [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]),
     "paella_conv2d_group_pool_dims": (c_int, [ctypes.POINTER(ctypes.POINTER(ConvPlan)), c_int, ctypes.POINTER(PoolDesc), ctypes.POINTER(LaunchDims)]),
     "paella_conv2d_launch_group_pool": (c_int, [ctypes.POINTER(ConvOperands), c_int, ctypes.POINTER(PoolDesc), c_void_p, c_void_p] + _TAIL),
     "paella_dense_dims": (c_int, [c_int, c_int, ctypes.POINTER(LaunchDims)]),

@@ -35,7 +35,7 @@ int g_direct_queue_count = 0;
 namespace {
 
 constexpr uint32_t kQueuePackets = 4096;       // ring size (power of two)
-constexpr uint32_t kKernargSlotBytes = 1280;   // one slot per packet index: explicit args <= 1024 + implicit block 256
+constexpr uint32_t kKernargSlotBytes = 2560;   // one slot per packet index: explicit args <= 2304 + implicit block 256
 constexpr size_t kImplicitBytes = 256;
 
 struct Runtime {
@@ -234,8 +234,10 @@ void stream_lines(char* dst, const char* src, size_t lines) {
     else stream_lines_128(dst, src, lines);
 }
 
+bool direct_queue_ordered(const DirectQueue* q) { return q->ordered; }
+
 void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3 block, unsigned dynamic_lds, const void* explicit_args,
-                     size_t explicit_bytes) {
+                     size_t explicit_bytes, size_t used_bytes) {
     hsa_queue_t* hq = q->queue;
     const uint64_t index = q->write_index;
     // Ring full: wait for the packet processor (it drains without any action from this thread).
@@ -260,7 +262,8 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     // stores: written in pieces, a line leaves the core's write-combining buffers as several partial transactions
     // (host time of the 51 launches of an Inception-v3 pass, argument ring warm: 36.5 us in pieces, 28.7 us this way).
     alignas(64) char stage[kKernargSlotBytes];
-    std::memcpy(stage, explicit_args, explicit_bytes);
+    if (used_bytes == 0 || used_bytes > explicit_bytes) used_bytes = explicit_bytes;
+    std::memcpy(stage, explicit_args, used_bytes);
     struct Implicit {
         uint32_t block_count[3];
         uint16_t group_size[3];
@@ -294,7 +297,14 @@ void direct_dispatch(DirectQueue* q, const DirectKernel* kernel, dim3 grid, dim3
     if (q->device_kernargs) {
         const size_t lines = (total + 63) / 64;
         std::memset(stage + total, 0, lines * 64 - total);  // the tail of the last line is padding inside the slot
-        stream_lines(ka, stage, lines);
+        // lines that hold neither used explicit arguments nor the implicit block stay as they are in the ring
+        const size_t used_lines = (used_bytes + 63) / 64, implicit_line = total > explicit_bytes ? implicit_at / 64 : lines;
+        if (implicit_line > used_lines) {
+            stream_lines(ka, stage, used_lines);
+            stream_lines(ka + implicit_line * 64, stage + implicit_line * 64, lines - implicit_line);
+        } else {
+            stream_lines(ka, stage, lines);
+        }
     } else {
         std::memcpy(ka, stage, total);
     }
@@ -344,6 +354,24 @@ bool direct_device_tick_to_system(uint64_t device_tick, uint64_t* system_tick) {
     return hsa_amd_profiling_convert_tick_to_system_domain(g_rt.gpu, device_tick, system_tick) == HSA_STATUS_SUCCESS;
 }
 
+}  // namespace paella
+
+namespace paella {
+static std::vector<void*> g_shared_queues;  // the process-wide set of paella_direct_queue_shared
+static std::mutex g_shared_mutex;
+static std::atomic<size_t> g_shared_count{0};
+
+uint64_t direct_shared_min_waiting() {
+    // No lock: the set is filled once, under the lock, before its size is published, and never changes afterwards.
+    if (g_shared_count.load(std::memory_order_acquire) == 0) return 0;
+    uint64_t least = ~0ull;
+    for (void* h : g_shared_queues) {
+        DirectQueue* q = static_cast<DirectQueue*>(h);
+        const uint64_t waiting = q->write_index - hsa_queue_load_read_index_relaxed(q->queue);
+        if (waiting < least) least = waiting;
+    }
+    return least;
+}
 }  // namespace paella
 
 // ---- C-ABI --------------------------------------------------------------------------------------
@@ -416,12 +444,11 @@ extern "C" int paella_direct_queue_create(void** out) {
 extern "C" int paella_direct_queue_shared(void** out) {
     // A small process-wide set of unordered queues handed out round-robin: callers whose dependent work is
     // ordered by notifications (the model job adapters on the serving thread) spread their kernels over them.
-    static std::vector<void*> shared;
+    std::vector<void*>& shared = paella::g_shared_queues;
     static size_t next = 0;
     static bool failed = false;
-    static std::mutex mutex;
     if (!out) return PAELLA_EINVAL;
-    std::lock_guard<std::mutex> lock(mutex);
+    std::lock_guard<std::mutex> lock(paella::g_shared_mutex);
     if (shared.empty() && !failed) {
         const char* env = std::getenv("PAELLA_DIRECT_QUEUES");
         long n = env ? std::strtol(env, nullptr, 10) : 4;
@@ -433,6 +460,7 @@ extern "C" int paella_direct_queue_shared(void** out) {
             shared.push_back(q);
         }
         failed = shared.empty();
+        paella::g_shared_count.store(shared.size(), std::memory_order_release);
     }
     if (shared.empty()) {
         *out = nullptr;

@@ -41,8 +41,17 @@ inline DirectQueue* direct_queue_lookup(void* handle) { return g_direct_queue_co
 // if the kernel is not in the embedded code objects.
 const DirectKernel* direct_kernel(const void* host_function);
 
+// `used_bytes` (0 = all): the kernel reads only that much of its explicit arguments (a group launch with fewer members than
+// the argument block has room for); the rest of the block is not written.
 void direct_dispatch(DirectQueue* queue, const DirectKernel* kernel, dim3 grid, dim3 block, unsigned dynamic_lds, const void* explicit_args,
-                     size_t explicit_bytes);
+                     size_t explicit_bytes, size_t used_bytes = 0);
+
+// True while the queue puts the barrier bit on its packets (paella_direct_queue_set_ordered).
+bool direct_queue_ordered(const DirectQueue* queue);
+
+// Fewest packets waiting (written but not yet taken by the packet processor) on any queue of the shared set; 0 when
+// there is no shared set yet.
+uint64_t direct_shared_min_waiting();
 
 // Kernel-argument packing: every argument at its natural alignment, in order (the kernarg segment layout of
 // by-value arguments).
@@ -55,7 +64,7 @@ inline void pack_args(char* buf, size_t& offset, const T& first, const Rest&... 
     pack_args(buf, offset, rest...);
 }
 
-constexpr size_t kMaxExplicitArgBytes = 1024;  // largest: four conv problems in one launch
+constexpr size_t kMaxExplicitArgBytes = 2304;  // largest: eight conv problems in one launch
 
 // Clock bridge for latency probes: the host's reading of the system timestamp, its frequency, and the
 // translation of a device realtime-counter value (what wall_clock64() returns in a kernel) into that domain.

@@ -19,15 +19,16 @@ struct TimingEvents {
 
 TimingEvents& timing_events();  // thread-local; defined in ops_misc.hip
 
+// `used_bytes` (0 = all): how much of the argument block the kernel reads (see direct_dispatch).
 template <typename Kernel, typename... Args>
-inline void launch(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream, Args... args) {
+inline void launch_used(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream, size_t used_bytes, const Args&... args) {
     // `stream` is either a HIP stream or a direct-dispatch queue (paella_direct_queue_create).
     if (DirectQueue* q = direct_queue_lookup(reinterpret_cast<void*>(stream))) {
         alignas(16) char buf[kMaxExplicitArgBytes];
         size_t bytes = 0;
         static_assert((0 + ... + (sizeof(Args) + alignof(Args))) <= kMaxExplicitArgBytes, "kernel arguments do not fit the staging buffer");
         pack_args(buf, bytes, args...);
-        direct_dispatch(q, direct_kernel(reinterpret_cast<const void*>(kernel)), grid, block, lds_bytes, buf, bytes);
+        direct_dispatch(q, direct_kernel(reinterpret_cast<const void*>(kernel)), grid, block, lds_bytes, buf, bytes, used_bytes);
         return;
     }
     const TimingEvents& t = timing_events();
@@ -36,6 +37,11 @@ inline void launch(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hip
     } else {
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
     }
+}
+
+template <typename Kernel, typename... Args>
+inline void launch(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream, const Args&... args) {
+    launch_used(kernel, grid, block, lds_bytes, stream, 0, args...);
 }
 
 }  // namespace paella

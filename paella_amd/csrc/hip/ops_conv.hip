@@ -25,10 +25,12 @@
 #include <algorithm>
 #include <atomic>
 #include <mutex>
+#include <vector>
 
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 
 #include "paella_ops.h"
 #include <llis/job/finished_block_notifier.h>
@@ -70,6 +72,7 @@ struct ConvArgs {
     int act;
     float lo, hi;
     uint32_t job_id;
+    unsigned hook_blocks;           // workgroups of this launch that report to `notifier`; 0: all of them (one job per launch)
     llis::job::FinishedBlockNotifier* notifier;
     // divisors: of the work-list position (pixel tiles per slab, or slabs per pixel tile), channel tiles, output width,
     // chunks per filter tap, filter width; fast_div = 0: operands too large for the shortcut, divide
@@ -111,7 +114,8 @@ struct PreOp {
 template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
-    paella::hook_entry(p.notifier, p.job_id);
+    const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
+    paella::hook_entry(p.notifier, p.job_id, hook_blocks);
     // Waves of this workgroup whose result stores have been acknowledged (see the end of this function); cleared here, and
     // the barrier of the cross-wave sum lies between this store and the first increment.
     __shared__ unsigned waves_done;
@@ -420,6 +424,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         // Deterministic split-k: every workgroup parks its partial tile in the workspace (write-through),
         // bumps the tile's counter, and the workgroup that arrives last adds the partials in split order and
         // runs the epilogue.  The counter is left at zero for the next launch.
+        // Ordering without fences: store_out is a device-scope write-through store, so once s_waitcnt vmcnt(0) has returned
+        // the partial tile is in memory, ahead of the counter bump that follows the barrier; the last arriver reads the
+        // partials with device-scope atomic loads, which do not hit in its own caches.  A release on the bump and an acquire
+        // after it would add a cache write-back and an invalidate per workgroup for data that never sat in a cache.
         const int tile = tile_m * p.n_tiles_n + tile_n;
         float* part = p.ws_partials + ((size_t)tile * p.splits + split) * (NACC * 64);
 #pragma unroll
@@ -465,7 +473,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             if (lane == 0) before = __hip_atomic_fetch_add(&waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             last = __builtin_amdgcn_readfirstlane(before) == (unsigned)KW - 1;
         }
-        if (last && lane == 0) p.notifier->end_from_one_lane(p.job_id & ~PAELLA_JOB_ID_FLAGS, (p.job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0);
+        if (last && lane == 0) p.notifier->end_from_one_lane(p.job_id & ~PAELLA_JOB_ID_FLAGS, (p.job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0, hook_blocks);
     }
 }
 
@@ -490,18 +498,19 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_kernel
 // problem's workgroups after the other's.  All use the smallest tile and the same wave count; the hooks see one
 // kernel of as many workgroups as the problems have together.  A workgroup finds its problem by its id and reads
 // that problem's arguments (an index into the argument block, the same for the whole workgroup).
-constexpr int kMaxGroup = PAELLA_CONV_GROUP_MAX;
+constexpr int kMaxGroup = PAELLA_CONV_GROUP_MAX;  // members of one call (one request's independent convs)
+constexpr int kPackMax = PAELLA_CONV_PACK_MAX;    // members of one launch (the kernels of several requests packed together)
 
 struct ConvGroupArgs {
-    ConvArgs prob[kMaxGroup];
-    unsigned start[kMaxGroup];  // first workgroup id of each problem; 0xFFFFFFFF for unused entries
+    unsigned start[kPackMax];  // first workgroup id of each problem; 0xFFFFFFFF for unused entries
+    ConvArgs prob[kPackMax];   // only the used entries are written to the argument ring
 };
 
 template <int KW, bool TAP_MAJOR>
 __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
     int idx = 0;
 #pragma unroll
-    for (int i = 1; i < kMaxGroup; ++i)
+    for (int i = 1; i < kPackMax; ++i)
         if (blockIdx.x >= g.start[i]) idx = i;
     conv_tile<1, 1, KW, TAP_MAJOR>(g.prob[idx], blockIdx.x - g.start[idx]);
 }
@@ -812,6 +821,7 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
     a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
     a.job_id = job_id;
+    a.hook_blocks = 0;
     a.notifier = nf;
     a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
     a.n_tiles_m = plan->m_pad / (32 * plan->mi);
@@ -883,6 +893,165 @@ extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, in
     return 0;
 }
 
+namespace {
+
+// One launch of the group kernel over the first n entries of g (their start[] filled, the rest marked unused here).
+int launch_group_args(ConvGroupArgs& g, int n, int kw, int k_order, unsigned grid, unsigned dyn_lds, void* stream) {
+    for (int i = n; i < kPackMax; ++i) g.start[i] = 0xFFFFFFFFu;
+    ConvGroupKernel kern = pick_group_kernel(kw, k_order);
+    if (!kern) return PAELLA_EINVAL;
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
+    paella::launch_used(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(stream),
+                        offsetof(ConvGroupArgs, prob) + (size_t)n * sizeof(ConvArgs), g);
+    return (int)hipGetLastError();
+}
+
+// ---- Launch packing ---------------------------------------------------------------------------------------------
+// A hardware queue of this device runs one kernel at a time, and four queues is all that run side by side: a conv that
+// fills a fifth of the machine still takes a queue for its whole latency.  With packing on (paella_pack_enable, per
+// thread), conv launches on the 32 x 32 tile that are bound for an unordered direct-dispatch queue are held back and go
+// out together, up to kPackMax problems in one grid of the group kernel, each with its own job id and notifier.  The
+// holder (the serving thread) calls paella_pack_poll() from its loop: what is held goes out as soon as a queue of the
+// shared set has nothing waiting, when a launch is full, or after kPackHoldNs at the latest.
+struct PackItem {
+    int n = 0;               // problems of one call (one job's stage)
+    unsigned grid = 0;       // their workgroups together: what the job's notifier counts
+    unsigned dyn_lds = 0;
+    ConvArgs args[kMaxGroup];
+    unsigned grids[kMaxGroup];
+};
+
+struct PackList {
+    std::vector<PackItem> items;
+    int members = 0;
+};
+
+struct PackState {
+    bool enabled = false;
+    int held = 0;                 // items over all lists
+    uint64_t first_held_ns = 0;
+    PackList lists[4][2];         // by log2(waves per workgroup) and reduction order
+};
+
+std::atomic<uint64_t> g_pack_launches{0}, g_pack_members{0};  // over all threads, for reports
+
+thread_local PackState g_pack;
+constexpr uint64_t kPackHoldNs = 30000;
+
+uint64_t now_ns() {
+    timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (uint64_t)ts.tv_sec * 1000000000ull + (uint64_t)ts.tv_nsec;
+}
+
+int kw_index(int kw) { return kw == 1 ? 0 : kw == 2 ? 1 : kw == 4 ? 2 : 3; }
+
+// Holds the call back if packing applies to it.  Returns false when the caller must launch it itself.
+bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n, void* stream) {
+    if (!g_pack.enabled || paella::timing_events().start != nullptr) return false;
+    paella::DirectQueue* q = paella::direct_queue_lookup(stream);
+    if (!q || paella::direct_queue_ordered(q)) return false;
+    PackList& list = g_pack.lists[kw_index(plans[0]->kw)][plans[0]->k_order ? 1 : 0];
+    list.items.emplace_back();
+    PackItem& it = list.items.back();
+    it.n = n;
+    for (int i = 0; i < n; ++i) {
+        it.args[i] = args[i];
+        it.grids[i] = plans[i]->dims.grid;
+        it.grid += plans[i]->dims.grid;
+        it.dyn_lds = std::max(it.dyn_lds, plans[i]->dims.lds_bytes);
+    }
+    for (int i = 0; i < n; ++i) it.args[i].hook_blocks = it.grid;
+    list.members += n;
+    if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
+    return true;
+}
+
+// Sends the held items of one list, oldest first, as few launches as kPackMax problems per launch allow; with
+// only_full, stops before a launch that would go out with room to spare.
+int pack_send(PackList& list, int kw, int k_order, bool only_full) {
+    int launches = 0;
+    size_t done = 0;
+    while (done < list.items.size()) {
+        if (only_full && list.members < kPackMax) break;
+        ConvGroupArgs g;
+        int n = 0;
+        unsigned grid = 0, dyn_lds = 0;
+        size_t i = done;
+        for (; i < list.items.size() && n + list.items[i].n <= kPackMax; ++i) {
+            const PackItem& it = list.items[i];
+            for (int k = 0; k < it.n; ++k) {
+                g.prob[n] = it.args[k];
+                g.start[n] = grid;
+                grid += it.grids[k];
+                ++n;
+            }
+            dyn_lds = std::max(dyn_lds, it.dyn_lds);
+        }
+        void* target = nullptr;
+        if (paella_direct_queue_shared(&target) != 0) return -1;
+        int rc;
+        if (n == 1) {  // nothing to share the launch with: the plain kernel, whose argument block is a quarter of the group's
+            ConvKernel kern = pick_kernel(1, 1, kw, k_order);
+            g.prob[0].hook_blocks = 0;
+            rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds);
+            if (rc == 0) {
+                paella::launch(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(target), g.prob[0]);
+                rc = (int)hipGetLastError();
+            }
+        } else {
+            rc = launch_group_args(g, n, kw, k_order, grid, dyn_lds, target);
+        }
+        if (rc != 0) return -1;
+        ++launches;
+        g_pack_launches.fetch_add(1, std::memory_order_relaxed);
+        g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
+        for (size_t k = done; k < i; ++k) list.members -= list.items[k].n;
+        g_pack.held -= (int)(i - done);
+        done = i;
+    }
+    list.items.erase(list.items.begin(), list.items.begin() + (long)done);
+    return launches;
+}
+
+int pack_send_all(bool only_full) {
+    int launches = 0;
+    for (int w = 0; w < 4; ++w)
+        for (int o = 0; o < 2; ++o) {
+            PackList& list = g_pack.lists[w][o];
+            if (list.items.empty()) continue;
+            const int r = pack_send(list, 1 << w, o, only_full);
+            if (r < 0) return PAELLA_ENOSUP;
+            launches += r;
+        }
+    if (g_pack.held > 0 && !only_full) g_pack.first_held_ns = now_ns();
+    return launches;
+}
+
+}  // namespace
+
+extern "C" int paella_pack_enable(int on) {
+    if (!on && g_pack.held > 0) {
+        if (int rc = pack_send_all(false); rc < 0) return rc;
+    }
+    g_pack.enabled = on != 0;
+    return 0;
+}
+
+extern "C" int paella_pack_flush(void) { return g_pack.held > 0 ? pack_send_all(false) : 0; }
+
+extern "C" int paella_pack_poll(void) {
+    if (g_pack.held == 0) return 0;
+    if (paella::direct_shared_min_waiting() == 0 || now_ns() - g_pack.first_held_ns >= kPackHoldNs) return pack_send_all(false);
+    return pack_send_all(true);
+}
+
+extern "C" int paella_pack_stats(uint64_t* launches, uint64_t* members) {
+    if (launches) *launches = g_pack_launches.load(std::memory_order_relaxed);
+    if (members) *members = g_pack_members.load(std::memory_order_relaxed);
+    return g_pack.held;
+}
+
 extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void* stream, uint32_t job_id, void* notifier) {
     if (!members || n < 2 || n > kMaxGroup) return PAELLA_EINVAL;
     const paella_conv_plan* plans[kMaxGroup];
@@ -894,19 +1063,16 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
             if (plans[i]->splits > 1 && plans[j]->splits > 1 && members[i].workspace == members[j].workspace) return PAELLA_EINVAL;
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
     ConvGroupArgs g;
-    unsigned next = 0;
-    for (int i = 0; i < kMaxGroup; ++i) {
-        const paella_conv_operands& m = members[i < n ? i : 0];  // unused entries: a valid copy that no workgroup selects
+    unsigned next = 0, dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
+    for (int i = 0; i < n; ++i) {
+        const paella_conv_operands& m = members[i];
         if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, g.prob[i])) return rc;
-        g.start[i] = i < n ? next : 0xFFFFFFFFu;
-        if (i < n) next += m.plan->dims.grid;
+        g.start[i] = next;
+        next += m.plan->dims.grid;
+        dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
-    ConvGroupKernel kern = pick_group_kernel(plans[0]->kw, plans[0]->k_order);
-    unsigned dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
-    for (int i = 0; i < n; ++i) dyn_lds = std::max(dyn_lds, plans[i]->dims.lds_bytes);
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
-    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dyn_lds, reinterpret_cast<hipStream_t>(stream), g);
-    return (int)hipGetLastError();
+    if (pack_hold(plans, g.prob, n, stream)) return 0;
+    return launch_group_args(g, n, plans[0]->kw, plans[0]->k_order, dims.grid, dyn_lds, stream);
 }
 
 namespace {
@@ -1004,6 +1170,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
         if (!kern) return PAELLA_EINVAL;
         ConvArgs a;
         if (int rc = fill_args(plan, x, blob_dev, bias, residual, slope, y, workspace, job_id, nf, a)) return rc;
+        if (plan->mi == 1 && plan->ni == 1 && pack_hold(&plan, &a, 1, stream)) return 0;
         if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
         paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
         return (int)hipGetLastError();

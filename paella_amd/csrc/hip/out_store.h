@@ -22,6 +22,14 @@ __device__ __forceinline__ void hook_entry(llis::job::FinishedBlockNotifier* not
     }
 }
 
+// The same for a workgroup of a launch that carries several jobs' kernels: `blocks` workgroups report to this notifier.
+__device__ __forceinline__ void hook_entry(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id, unsigned blocks) {
+    if (notifier) {
+        if (!(job_id & PAELLA_JOB_ID_NO_START)) notifier->start(job_id & ~PAELLA_JOB_ID_FLAGS, blocks);
+        else if (job_id & PAELLA_JOB_ID_TIME_BLOCKS) notifier->begin_timing();
+    }
+}
+
 // Last statement of every operator kernel (all results written with store_out / store_out4).
 __device__ __forceinline__ void hook_exit(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id) {
     if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_FLAGS, (job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0);

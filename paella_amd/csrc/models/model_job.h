@@ -103,6 +103,11 @@ class ModelJob : public llis::job::CoroutineJob {
                 direct_ = false;
             }
         }
+        // Conv launches of different requests share launches (paella_pack_enable) unless PAELLA_PACK=0: the serving thread
+        // holds them and lets them go from its loop.
+        const char* pack = std::getenv("PAELLA_PACK");
+        pack_ = direct_ && !(pack && std::strcmp(pack, "0") == 0);
+        if (pack_) llis::job::Context::add_poll_hook(&ModelJob::pack_poll);
     }
 
     void body(void* io_ptr) override {
@@ -139,9 +144,11 @@ class ModelJob : public llis::job::CoroutineJob {
             const uint32_t id = get_id() | (is_unfit() && unfit_starts_ ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
             void* target = stream();
             if (direct_) check(paella_direct_queue_shared(&target), "direct queue");
+            if (pack_) enable_packing_on_this_thread();
+            // members of a group wait for what is ahead of them in the queue (a stream orders by itself); the first one
+            // too, so that it is not held back for packing while the others go out
+            if (direct_ && last > s) paella_direct_queue_set_ordered(target, 1);
             for (int k = s; k <= last; ++k) {
-                // members after the first wait for what is ahead of them in the queue (a stream orders by itself)
-                if (direct_ && k == s + 1) paella_direct_queue_set_ordered(target, 1);
                 if (k < last) check(paella_exec_launch_stage(exec_, k, target, 0, nullptr), "stage launch");
                 else check(paella_exec_launch_stage(exec_, k, target, id, get_finished_block_notifier()), "stage launch");
             }
@@ -162,6 +169,17 @@ class ModelJob : public llis::job::CoroutineJob {
   private:
     void* stream() { return reinterpret_cast<void*>(get_cuda_stream()); }
 
+    static void pack_poll() { paella_pack_poll(); }
+
+    // Packing is a property of the launching thread (the serving thread, which also runs pack_poll from its loop).
+    static void enable_packing_on_this_thread() {
+        static thread_local bool on = false;
+        if (!on) {
+            paella_pack_enable(1);
+            on = true;
+        }
+    }
+
     static void check(int rc, const char* what) {
         if (rc != 0) {
             std::fprintf(stderr, "[llis] model job: %s failed: %d (%s)\n", what, rc, rc > 0 ? llis_hip_error_string(rc) : "bad argument");
@@ -178,6 +196,7 @@ class ModelJob : public llis::job::CoroutineJob {
     int num_stages_ = 0;
     std::vector<int> group_end_;   // per kernel: index of the last kernel of the group it is issued with
     bool direct_ = true;
+    bool pack_ = false;
     bool timed_ = false;
     bool unfit_starts_ = false;
     bool input_resident_ = false, input_uploaded_ = false;

@@ -1,3 +1,4 @@
+#include <llis/job/context.h>
 #include <llis/ipc/name_format.h>
 #include <llis/server/scheduler.h>
 #include <llis/server/server.h>
@@ -41,6 +42,10 @@ void Server::poll_once() {
         handle_c2s();
     }
     scheduler_->try_handle_block_start_finish();
+    {
+        LLIS_PHASE(kHooks);
+        job::Context::run_poll_hooks();
+    }
     if (total_owed_wakeups_ != 0 && ++polls_since_retry_ >= 64) retry_owed_wakeups();
 }
 

@@ -10,6 +10,7 @@
 //   hold NAME              create a named ring, write a known message, wait for a line on stdin (layout probe)
 //   socket                 abstract-namespace datagram round trip incl. the non-blocking full-queue path
 
+#include <llis/job/context.h>
 #include <llis/ipc/defs.h>
 #include <llis/ipc/name_format.h>
 #include <llis/ipc/shm_channel.h>
@@ -129,6 +130,20 @@ int main(int argc, char** argv) {
         t0.join();
         std::printf(bad ? "ERROR multiwriter\n" : "OK multiwriter\n");
         return bad != 0;
+    }
+    if (cmd == "pollhooks") {
+        // the serving thread's per-turn hooks: a function registers once however often it is added, hooks run in order
+        static int a = 0, b = 0;
+        llis::job::Context::run_poll_hooks();  // none yet
+        llis::job::Context::add_poll_hook(+[] { ++a; });
+        auto fb = +[] { b += a; };
+        llis::job::Context::add_poll_hook(fb);
+        llis::job::Context::add_poll_hook(fb);
+        llis::job::Context::add_poll_hook(nullptr);
+        for (int i = 0; i < 3; ++i) llis::job::Context::run_poll_hooks();
+        const bool ok = a == 3 && b == 1 + 2 + 3;
+        std::printf(ok ? "OK pollhooks\n" : "ERROR pollhooks %d %d\n", a, b);
+        return !ok;
     }
     if (cmd == "pring") {
         using Info = llis::job::InstrumentInfo;

@@ -1,0 +1,135 @@
+"""Launch packing (paella_pack_*): convs of several jobs held back and sent as one grid must give the bits they give alone,
+and every job's notifier must see exactly its own workgroups."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from test_ring_gpu import decode
+
+pytestmark = pytest.mark.gpu
+
+NO_START = 0x80000000  # PAELLA_JOB_ID_NO_START
+
+
+def layers(cuda, rng):
+    """Ten layers on the 32 x 32 tile with eight waves in tap-major order, with and without a split reduction."""
+    from paella_amd import ops
+    shapes = [  # C, K, H, R, stride, pad
+        (64, 64, 56, 3, 1, 1), (128, 128, 28, 3, 1, 1), (256, 256, 14, 3, 1, 1), (512, 512, 7, 3, 1, 1), (768, 192, 17, 1, 1, 0),
+        (1280, 320, 8, 1, 1, 0), (288, 64, 35, 1, 1, 0), (256, 512, 14, 1, 2, 0), (64, 96, 19, 3, 1, 1), (160, 40, 9, 3, 2, 1),
+    ]
+    out = []
+    for c, k, h, r, st, pd in shapes:
+        w = rng.standard_normal((k, c, r, r)).astype(np.float32) * (1.0 / np.sqrt(c * r * r))
+        b = rng.standard_normal(k).astype(np.float32)
+        conv = ops.Conv2d(w, b, stride=st, pad=pd, act=ops.ACT_RELU, in_hw=(h, h))
+        assert (conv.plan.mi, conv.plan.ni, conv.plan.kw, conv.plan.k_order) == (1, 1, 8, 1)
+        x = torch.tensor(rng.standard_normal((1, c, h, h)).astype(np.float32), device=cuda)
+        out.append((conv, x))
+    return out
+
+
+@pytest.fixture()
+def ring(cuda):
+    from paella_amd import _abi
+    lib = _abi.ops()
+    handle = ctypes.c_void_p()
+    _abi.check(lib.paella_ring_create(8192, 16, ctypes.byref(handle)), "paella_ring_create")
+    yield lib, handle
+    lib.paella_pack_enable(0)
+    lib.paella_ring_destroy(handle)
+
+
+def held(lib):
+    return lib.paella_pack_stats(None, None)
+
+
+def stats(lib):
+    a, b = ctypes.c_uint64(), ctypes.c_uint64()
+    lib.paella_pack_stats(ctypes.byref(a), ctypes.byref(b))
+    return a.value, b.value
+
+
+def test_packed_convs_are_bit_identical_and_report_to_their_own_jobs(ring, cuda):
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(11)
+    ls = layers(cuda, rng)
+    alone = [conv(x) for conv, x in ls]
+    torch.cuda.synchronize()
+    batch = lib.paella_ring_batch_size()
+    with ops.DirectQueue() as q:  # unordered: what the serving path launches on
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            before = stats(lib)
+            outs, want_msgs, grids = [], 0, {}
+            # jobs 1..8 one conv each; job 9 two convs in one call (a request's independent pair): nine calls, ten problems
+            for j in range(8):
+                conv, x = ls[j]
+                y = torch.zeros_like(alone[j])
+                conv(x, out=y, stream=q.handle, job_id=j + 1, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, j)))
+                outs.append(y)
+                grids[j + 1] = conv.plan.dims.grid
+            pair = ops.conv2d_group([ls[8][0], ls[9][0]], [ls[8][1], ls[9][1]], stream=q.handle, job_id=9 | NO_START,
+                                    notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, 8)))
+            outs += pair
+            grids[9] = ls[8][0].plan.dims.grid + ls[9][0].plan.dims.grid
+            assert held(lib) == 9
+            sent = lib.paella_pack_flush()
+            assert sent == 2 and held(lib) == 0  # eight problems in the first launch, the pair in the second
+            after = stats(lib)
+            assert (after[0] - before[0], after[1] - before[1]) == (2, 10)
+            per = lambda n: (n + batch - 1) // batch
+            want_msgs = sum(2 * per(grids[j]) for j in range(1, 9)) + per(grids[9])
+            buf = np.zeros(want_msgs, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want_msgs, 20.0) == want_msgs
+            m = decode(buf)
+            for j in range(1, 10):
+                ends = (m["job_id"] == j) & (m["is_start"] == 0)
+                starts = (m["job_id"] == j) & (m["is_start"] == 1)
+                assert m["num"][ends].sum() == grids[j], j
+                assert m["num"][starts].sum() == (grids[j] if j < 9 else 0), j
+                assert ends.sum() == per(grids[j])
+            extra = np.zeros(1, np.uint64)
+            assert lib.paella_ring_drain(h, extra.ctypes.data, 1, 0.05) == 0  # nothing else was sent
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for a, b in zip(alone, outs):
+        assert torch.equal(a, b)
+
+
+def test_poll_sends_at_once_on_idle_queues_and_ordered_queues_are_not_held(ring, cuda):
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(12)
+    ls = layers(cuda, rng)[:3]
+    alone = [conv(x) for conv, x in ls]
+    torch.cuda.synchronize()
+    with ops.DirectQueue() as q, ops.DirectQueue(ordered=True) as qo:
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            y_ordered = ls[0][0](ls[0][1], stream=qo.handle)  # ordered queue: launched at once
+            assert held(lib) == 0
+            qo.wait()
+            assert torch.equal(y_ordered, alone[0])
+            ys = [torch.zeros_like(a) for a in alone]
+            for k, (conv, x) in enumerate(ls):
+                conv(x, out=ys[k], stream=q.handle, job_id=(k + 1) | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, k)))
+            assert held(lib) == 3
+            assert lib.paella_pack_poll() == 1 and held(lib) == 0  # no queue has anything waiting: one launch of three problems
+            batch = lib.paella_ring_batch_size()
+            want = sum((c.plan.dims.grid + batch - 1) // batch for c, _ in ls)
+            buf = np.zeros(want, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want, 20.0) == want
+            # a HIP stream is never held
+            y_stream = ls[1][0](ls[1][1])
+            assert held(lib) == 0
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for a, b in zip(alone, ys):
+        assert torch.equal(a, b)
+    assert torch.equal(y_stream, alone[1])
