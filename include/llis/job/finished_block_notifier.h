@@ -99,10 +99,14 @@ class FinishedBlockNotifier {
 
     // Same, for callers that know from elsewhere whether timing is on (the flag is then not read here).
     __device__ __forceinline__ void end_written_through(JobId job_id, bool timed) {
+        end_written_through(job_id, timed, gridDim.x * gridDim.y * gridDim.z);
+    }
+    // ... and how many workgroups of the launch report to this notifier (a launch that carries several jobs' kernels).
+    __device__ __forceinline__ void end_written_through(JobId job_id, bool timed, unsigned num_blocks) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
-            announce<false>(&agg_counter_end_, 0, job_id);
+            announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
             if (timed && measure_block_time_) send_block_time();  // the member is looked at only when timing was asked for
         }
     }

@@ -501,9 +501,20 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_kernel
 constexpr int kMaxGroup = PAELLA_CONV_GROUP_MAX;  // members of one call (one request's independent convs)
 constexpr int kPackMax = PAELLA_CONV_PACK_MAX;    // members of one launch (the kernels of several requests packed together)
 
+// A member may also be a pooling operator (an inception module starts with three 1x1 convs and a 3x3 pool that all read
+// the module's input): its workgroups, one output element per thread with this kernel's workgroup size, come after all the
+// convs' (they are the shortest).
+union GroupMember {
+    ConvArgs conv;
+    paella::PoolArgs pool;
+    __host__ __device__ GroupMember() {}
+};
+
 struct ConvGroupArgs {
-    unsigned start[kPackMax];  // first workgroup id of each problem; 0xFFFFFFFF for unused entries
-    ConvArgs prob[kPackMax];   // only the used entries are written to the argument ring
+    unsigned start[kPackMax];  // first workgroup id of each member; 0xFFFFFFFF for unused entries
+    unsigned pool_mask;        // bit i: member i is a pooling operator
+    unsigned reserved;
+    GroupMember m[kPackMax];   // only the used entries are written to the argument ring
 };
 
 template <int KW, bool TAP_MAJOR>
@@ -512,35 +523,19 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kern
 #pragma unroll
     for (int i = 1; i < kPackMax; ++i)
         if (blockIdx.x >= g.start[i]) idx = i;
-    conv_tile<1, 1, KW, TAP_MAJOR>(g.prob[idx], blockIdx.x - g.start[idx]);
-}
-
-// Up to three such convs and one pooling operator in one launch: an inception module starts with three 1x1 convs and
-// a 3x3 pool that all read the module's input.  The pool's workgroups come last (they are the shortest), each thread
-// one output element as in the pooling kernel, with this kernel's workgroup size.
-constexpr int kMaxGroupWithPool = 3;
-
-struct ConvGroupPoolArgs {
-    ConvArgs prob[kMaxGroupWithPool];
-    unsigned start[kMaxGroupWithPool];  // first workgroup id of each conv; 0xFFFFFFFF for unused entries
-    unsigned pool_start;                // first workgroup id of the pool
-    paella::PoolArgs pool;
-};
-
-template <int KW>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_pool_kernel(ConvGroupPoolArgs g) {
-    if (blockIdx.x >= g.pool_start) {
-        paella::hook_entry(g.pool.notifier, g.pool.job_id);
-        paella::pool_element(g.pool, (int)((blockIdx.x - g.pool_start) * (64 * KW) + threadIdx.x));
-        paella::hook_exit(g.pool.notifier, g.pool.job_id);
+    const unsigned bid = blockIdx.x - g.start[idx];
+    if ((g.pool_mask >> idx) & 1u) {
+        const paella::PoolArgs& p = g.m[idx].pool;
+        const unsigned blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
+        paella::hook_entry(p.notifier, p.job_id, blocks);
+        paella::pool_element(p, (int)(bid * (64 * KW) + threadIdx.x));
+        paella::hook_exit(p.notifier, p.job_id, blocks);
         return;
     }
-    int idx = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxGroupWithPool; ++i)
-        if (blockIdx.x >= g.start[i]) idx = i;
-    conv_tile<1, 1, KW, true>(g.prob[idx], blockIdx.x - g.start[idx]);
+    conv_tile<1, 1, KW, TAP_MAJOR>(g.m[idx].conv, bid);
 }
+
+constexpr int kMaxGroupWithPool = 3;  // convs of one call that also carries a pooling operator
 
 // ---------------------------------------------------------------------------------------------------
 // Depthwise conv (groups == C == K): HBM-bound, one thread per output pixel, taps from L1/L2.
@@ -895,14 +890,16 @@ extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, in
 
 namespace {
 
-// One launch of the group kernel over the first n entries of g (their start[] filled, the rest marked unused here).
+// One launch of the group kernel over the first n members of g (their start[] and pool_mask filled; the rest marked
+// unused here).
 int launch_group_args(ConvGroupArgs& g, int n, int kw, int k_order, unsigned grid, unsigned dyn_lds, void* stream) {
     for (int i = n; i < kPackMax; ++i) g.start[i] = 0xFFFFFFFFu;
+    g.reserved = 0;
     ConvGroupKernel kern = pick_group_kernel(kw, k_order);
     if (!kern) return PAELLA_EINVAL;
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
     paella::launch_used(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(stream),
-                        offsetof(ConvGroupArgs, prob) + (size_t)n * sizeof(ConvArgs), g);
+                        offsetof(ConvGroupArgs, m) + (size_t)n * sizeof(GroupMember), g);
     return (int)hipGetLastError();
 }
 
@@ -914,11 +911,15 @@ int launch_group_args(ConvGroupArgs& g, int n, int kw, int k_order, unsigned gri
 // holder (the serving thread) calls paella_pack_poll() from its loop: what is held goes out as soon as a queue of the
 // shared set has nothing waiting, when a launch is full, or after kPackHoldNs at the latest.
 struct PackItem {
-    int n = 0;               // problems of one call (one job's stage)
+    int n = 0;               // convs of one call (one job's stage)
+    bool has_pool = false;   // ... and the pooling operator that goes with them
     unsigned grid = 0;       // their workgroups together: what the job's notifier counts
     unsigned dyn_lds = 0;
     ConvArgs args[kMaxGroup];
     unsigned grids[kMaxGroup];
+    paella::PoolArgs pool;
+    unsigned pool_grid = 0;
+    int members() const { return n + (has_pool ? 1 : 0); }
 };
 
 struct PackList {
@@ -947,7 +948,8 @@ uint64_t now_ns() {
 int kw_index(int kw) { return kw == 1 ? 0 : kw == 2 ? 1 : kw == 4 ? 2 : 3; }
 
 // Holds the call back if packing applies to it.  Returns false when the caller must launch it itself.
-bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n, void* stream) {
+bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n, void* stream, const paella::PoolArgs* pool = nullptr,
+               unsigned pool_grid = 0) {
     if (!g_pack.enabled || paella::timing_events().start != nullptr) return false;
     paella::DirectQueue* q = paella::direct_queue_lookup(stream);
     if (!q || paella::direct_queue_ordered(q)) return false;
@@ -961,8 +963,15 @@ bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n
         it.grid += plans[i]->dims.grid;
         it.dyn_lds = std::max(it.dyn_lds, plans[i]->dims.lds_bytes);
     }
+    if (pool) {
+        it.has_pool = true;
+        it.pool = *pool;
+        it.pool_grid = pool_grid;
+        it.grid += pool_grid;
+        it.pool.hook_blocks = it.grid;
+    }
     for (int i = 0; i < n; ++i) it.args[i].hook_blocks = it.grid;
-    list.members += n;
+    list.members += it.members();
     if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
     return true;
 }
@@ -978,25 +987,37 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         int n = 0;
         unsigned grid = 0, dyn_lds = 0;
         size_t i = done;
-        for (; i < list.items.size() && n + list.items[i].n <= kPackMax; ++i) {
-            const PackItem& it = list.items[i];
-            for (int k = 0; k < it.n; ++k) {
-                g.prob[n] = it.args[k];
+        int total = 0;
+        for (; i < list.items.size() && total + list.items[i].members() <= kPackMax; ++i) total += list.items[i].members();
+        g.pool_mask = 0;
+        for (size_t k = done; k < i; ++k) {  // the convs of every item first ...
+            const PackItem& it = list.items[k];
+            for (int c = 0; c < it.n; ++c) {
+                g.m[n].conv = it.args[c];
                 g.start[n] = grid;
-                grid += it.grids[k];
+                grid += it.grids[c];
                 ++n;
             }
             dyn_lds = std::max(dyn_lds, it.dyn_lds);
+        }
+        for (size_t k = done; k < i; ++k) {  // ... then their pooling operators
+            const PackItem& it = list.items[k];
+            if (!it.has_pool) continue;
+            g.m[n].pool = it.pool;
+            g.start[n] = grid;
+            g.pool_mask |= 1u << n;
+            grid += it.pool_grid;
+            ++n;
         }
         void* target = nullptr;
         if (paella_direct_queue_shared(&target) != 0) return -1;
         int rc;
         if (n == 1) {  // nothing to share the launch with: the plain kernel, whose argument block is a quarter of the group's
             ConvKernel kern = pick_kernel(1, 1, kw, k_order);
-            g.prob[0].hook_blocks = 0;
+            g.m[0].conv.hook_blocks = 0;
             rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds);
             if (rc == 0) {
-                paella::launch(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(target), g.prob[0]);
+                paella::launch(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(target), g.m[0].conv);
                 rc = (int)hipGetLastError();
             }
         } else {
@@ -1006,7 +1027,7 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         ++launches;
         g_pack_launches.fetch_add(1, std::memory_order_relaxed);
         g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
-        for (size_t k = done; k < i; ++k) list.members -= list.items[k].n;
+        for (size_t k = done; k < i; ++k) list.members -= list.items[k].members();
         g_pack.held -= (int)(i - done);
         done = i;
     }
@@ -1063,33 +1084,20 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
             if (plans[i]->splits > 1 && plans[j]->splits > 1 && members[i].workspace == members[j].workspace) return PAELLA_EINVAL;
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
     ConvGroupArgs g;
+    ConvArgs args[kMaxGroup];
     unsigned next = 0, dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
     for (int i = 0; i < n; ++i) {
         const paella_conv_operands& m = members[i];
-        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, g.prob[i])) return rc;
+        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, args[i])) return rc;
+        g.m[i].conv = args[i];
         g.start[i] = next;
         next += m.plan->dims.grid;
         dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
-    if (pack_hold(plans, g.prob, n, stream)) return 0;
+    if (pack_hold(plans, args, n, stream)) return 0;
+    g.pool_mask = 0;
     return launch_group_args(g, n, plans[0]->kw, plans[0]->k_order, dims.grid, dyn_lds, stream);
 }
-
-namespace {
-
-typedef void (*ConvGroupPoolKernel)(ConvGroupPoolArgs);
-
-ConvGroupPoolKernel pick_group_pool_kernel(int kw) {
-    switch (kw) {
-        case 1: return conv_mfma_group_pool_kernel<1>;
-        case 2: return conv_mfma_group_pool_kernel<2>;
-        case 4: return conv_mfma_group_pool_kernel<4>;
-        case 8: return conv_mfma_group_pool_kernel<8>;
-        default: return nullptr;
-    }
-}
-
-}  // namespace
 
 extern "C" int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plans, int n, const paella_pool_desc* pool, paella_launch_dims* dims) {
     if (!plans || n < 1 || n > kMaxGroupWithPool || !pool) return PAELLA_EINVAL;
@@ -1110,7 +1118,7 @@ extern "C" int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plan
         dims->block = plans[0]->dims.block;
         dims->grid += (unsigned)(((size_t)pa.C * pa.P * pa.Q + dims->block - 1) / dims->block);
         dims->vgprs = plans[0]->dims.vgprs;
-        add_kernel_resources(reinterpret_cast<const void*>(pick_group_pool_kernel(plans[0]->kw)), dims);
+        add_kernel_resources(reinterpret_cast<const void*>(pick_group_kernel(plans[0]->kw, 1)), dims);
     }
     return 0;
 }
@@ -1126,22 +1134,24 @@ extern "C" int paella_conv2d_launch_group_pool(const paella_conv_operands* membe
         for (int j = i + 1; j < n; ++j)
             if (plans[i]->splits > 1 && plans[j]->splits > 1 && members[i].workspace == members[j].workspace) return PAELLA_EINVAL;
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
-    ConvGroupPoolArgs g;
-    unsigned next = 0;
-    for (int i = 0; i < kMaxGroupWithPool; ++i) {
-        const paella_conv_operands& m = members[i < n ? i : 0];  // unused entries: a valid copy that no workgroup selects
-        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, g.prob[i])) return rc;
-        g.start[i] = i < n ? next : 0xFFFFFFFFu;
-        if (i < n) next += m.plan->dims.grid;
+    ConvGroupArgs g;
+    ConvArgs args[kMaxGroupWithPool];
+    unsigned next = 0, dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
+    for (int i = 0; i < n; ++i) {
+        const paella_conv_operands& m = members[i];
+        if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, args[i])) return rc;
+        g.m[i].conv = args[i];
+        g.start[i] = next;
+        next += m.plan->dims.grid;
+        dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
-    g.pool_start = next;
-    if (!paella::pool_fill_args(pool, pool_x, pool_y, job_id, notifier, &g.pool)) return PAELLA_EINVAL;
-    ConvGroupPoolKernel kern = pick_group_pool_kernel(plans[0]->kw);
-    unsigned dyn_lds = 0;  // dims.lds_bytes is the scheduler's figure and includes the kernel's static LDS
-    for (int i = 0; i < n; ++i) dyn_lds = std::max(dyn_lds, plans[i]->dims.lds_bytes);
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
-    paella::launch(kern, dim3(dims.grid), dim3(dims.block), dyn_lds, reinterpret_cast<hipStream_t>(stream), g);
-    return (int)hipGetLastError();
+    paella::PoolArgs pa;
+    if (!paella::pool_fill_args(pool, pool_x, pool_y, job_id, notifier, &pa)) return PAELLA_EINVAL;
+    if (pack_hold(plans, args, n, stream, &pa, dims.grid - next)) return 0;
+    g.m[n].pool = pa;
+    g.start[n] = next;
+    g.pool_mask = 1u << n;
+    return launch_group_args(g, n + 1, plans[0]->kw, 1, dims.grid, dyn_lds, stream);
 }
 
 extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_plan* second, paella_launch_dims* dims) {
@@ -1308,7 +1318,7 @@ extern "C" int paella_conv_kernel_occupancy(int kind, int form, int mi, int ni, 
     } else if (mi == 1 && ni == 1) {
         if (form == 1 && k_order == 1) fn = reinterpret_cast<const void*>(pick_pre_kernel(kw));
         else if (form == 2) fn = reinterpret_cast<const void*>(pick_group_kernel(kw, k_order));
-        else if (form == 3 && k_order == 1) fn = reinterpret_cast<const void*>(pick_group_pool_kernel(kw));
+        else if (form == 3 && k_order == 1) fn = reinterpret_cast<const void*>(pick_group_kernel(kw, 1));
     }
     if (!fn) return PAELLA_EINVAL;
     if (int rc = allow_lds(fn, lds_bytes)) return rc;

@@ -34,6 +34,9 @@ __device__ __forceinline__ void hook_entry(llis::job::FinishedBlockNotifier* not
 __device__ __forceinline__ void hook_exit(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id) {
     if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_FLAGS, (job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0);
 }
+__device__ __forceinline__ void hook_exit(llis::job::FinishedBlockNotifier* notifier, uint32_t job_id, unsigned blocks) {
+    if (notifier) notifier->end_written_through(job_id & ~PAELLA_JOB_ID_FLAGS, (job_id & PAELLA_JOB_ID_TIME_BLOCKS) != 0, blocks);
+}
 }  // namespace paella
 
 __device__ __forceinline__ void store_out(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }

@@ -20,6 +20,7 @@ struct PoolArgs {
     int C, H, W, P, Q, R, S, sh, sw, ph, pw;
     int is_avg, count_include_pad;
     uint32_t job_id;
+    unsigned hook_blocks;  // workgroups of the launch that report to `notifier`; 0: all of them (one job per launch)
     llis::job::FinishedBlockNotifier* notifier;
 };
 
@@ -124,6 +125,7 @@ inline bool pool_fill_args(const paella_pool_desc* d, const float* x, float* y, 
     a->sh = d->stride_h; a->sw = d->stride_w; a->ph = d->pad_h; a->pw = d->pad_w;
     a->is_avg = d->is_avg; a->count_include_pad = d->count_include_pad;
     a->job_id = job_id;
+    a->hook_blocks = 0;
     a->notifier = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
     return true;
 }

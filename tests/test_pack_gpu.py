@@ -65,7 +65,7 @@ def test_packed_convs_are_bit_identical_and_report_to_their_own_jobs(ring, cuda)
         try:
             before = stats(lib)
             outs, want_msgs, grids = [], 0, {}
-            # jobs 1..8 one conv each; job 9 two convs in one call (a request's independent pair): nine calls, ten problems
+            # jobs 1..8 one conv each; job 9 two convs in one call (a request's independent pair)
             for j in range(8):
                 conv, x = ls[j]
                 y = torch.zeros_like(alone[j])
@@ -76,17 +76,27 @@ def test_packed_convs_are_bit_identical_and_report_to_their_own_jobs(ring, cuda)
                                     notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, 8)))
             outs += pair
             grids[9] = ls[8][0].plan.dims.grid + ls[9][0].plan.dims.grid
-            assert held(lib) == 9
+            # job 10: two pointwise convs and a 3x3 average pool over one input in one call (the head of an inception module)
+            c288, x288 = ls[6]
+            w2 = rng.standard_normal((48, 288, 1, 1)).astype(np.float32) / 17.0
+            second = ops.Conv2d(w2, None, act=ops.ACT_RELU, in_hw=(35, 35))
+            ref_pool_convs, ref_pool = ops.conv2d_group_pool([c288, second], [x288, x288], x288, 3, 1, pad=1, is_avg=True, count_include_pad=False)
+            torch.cuda.synchronize()
+            got_pool_convs, got_pool = ops.conv2d_group_pool([c288, second], [x288, x288], x288, 3, 1, pad=1, is_avg=True, count_include_pad=False,
+                                                             stream=q.handle, job_id=10 | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, 9)))
+            pool_wgs = (288 * 35 * 35 + 511) // 512
+            grids[10] = c288.plan.dims.grid + second.plan.dims.grid + pool_wgs
+            assert held(lib) == 10
             sent = lib.paella_pack_flush()
-            assert sent == 2 and held(lib) == 0  # eight problems in the first launch, the pair in the second
+            assert sent == 2 and held(lib) == 0  # eight problems in the first launch; the pair, two convs and a pool in the second
             after = stats(lib)
-            assert (after[0] - before[0], after[1] - before[1]) == (2, 10)
+            assert (after[0] - before[0], after[1] - before[1]) == (2, 13)
             per = lambda n: (n + batch - 1) // batch
-            want_msgs = sum(2 * per(grids[j]) for j in range(1, 9)) + per(grids[9])
+            want_msgs = sum(2 * per(grids[j]) for j in range(1, 9)) + per(grids[9]) + per(grids[10])
             buf = np.zeros(want_msgs, np.uint64)
             assert lib.paella_ring_drain(h, buf.ctypes.data, want_msgs, 20.0) == want_msgs
             m = decode(buf)
-            for j in range(1, 10):
+            for j in range(1, 11):
                 ends = (m["job_id"] == j) & (m["is_start"] == 0)
                 starts = (m["job_id"] == j) & (m["is_start"] == 1)
                 assert m["num"][ends].sum() == grids[j], j
@@ -98,6 +108,8 @@ def test_packed_convs_are_bit_identical_and_report_to_their_own_jobs(ring, cuda)
             lib.paella_pack_enable(0)
     torch.cuda.synchronize()
     for a, b in zip(alone, outs):
+        assert torch.equal(a, b)
+    for a, b in zip(ref_pool_convs + [ref_pool], got_pool_convs + [got_pool]):
         assert torch.equal(a, b)
 
 
