@@ -175,6 +175,19 @@ int paella_pack_enable(int on);
 int paella_pack_poll(void);
 int paella_pack_flush(void);
 int paella_pack_stats(uint64_t* launches, uint64_t* members);
+
+/* The same for a job that issues several dependent launches at once on an ORDERED direct-dispatch queue (a model of
+ * small kernels, one scheduler stage): between paella_pack_sequence_begin(key, queue) and paella_pack_sequence_end() the
+ * calling thread's paella_conv2d_launch (32 x 32 tile), paella_pool2d_launch and paella_dense_launch calls on `queue` are
+ * recorded instead of launched; _end holds the sequence, and sequences recorded under one `key` with the same operators
+ * position by position (requests of one model) are later sent together: the k-th launches of up to
+ * PAELLA_CONV_PACK_MAX sequences as one grid, position after position on one queue with the barrier bit set.  Any other
+ * launch in between ends the recording: what was recorded goes to `queue` at once, the launch follows it, and _end does
+ * nothing.  Results are bit-identical.  paella_pack_poll / _flush / _enable(0) send held sequences like held launches.
+ * _begin returns PAELLA_ENOSUP when packing is off on the thread or `queue` is not an ordered direct-dispatch queue
+ * (the caller then launches as usual). */
+int paella_pack_sequence_begin(const void* key, void* queue);
+int paella_pack_sequence_end(void);
 int paella_conv2d_launch_pair(const paella_conv_operands* first, const paella_conv_operands* second,
                               void* stream, uint32_t job_id, void* notifier);
 

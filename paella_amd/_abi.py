@@ -88,6 +88,8 @@ OPS_SYMBOLS = {
     "paella_pack_poll": (c_int, []),
     "paella_pack_flush": (c_int, []),
     "paella_pack_stats": (c_int, [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]),
+    "paella_pack_sequence_begin": (c_int, [c_void_p, c_void_p]),
+    "paella_pack_sequence_end": (c_int, []),
     "paella_conv2d_group_pool_dims": (c_int, [ctypes.POINTER(ctypes.POINTER(ConvPlan)), c_int, ctypes.POINTER(PoolDesc), ctypes.POINTER(LaunchDims)]),
     "paella_conv2d_launch_group_pool": (c_int, [ctypes.POINTER(ConvOperands), c_int, ctypes.POINTER(PoolDesc), c_void_p, c_void_p] + _TAIL),
     "paella_dense_dims": (c_int, [c_int, c_int, ctypes.POINTER(LaunchDims)]),

@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include "direct_dispatch.h"
+#include "pack.h"
 
 namespace paella {
 
@@ -22,6 +23,7 @@ TimingEvents& timing_events();  // thread-local; defined in ops_misc.hip
 // `used_bytes` (0 = all): how much of the argument block the kernel reads (see direct_dispatch).
 template <typename Kernel, typename... Args>
 inline void launch_used(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream, size_t used_bytes, const Args&... args) {
+    pack_sequence_break();  // a launch that the sequence recorder did not take ends the recording (see pack.h)
     // `stream` is either a HIP stream or a direct-dispatch queue (paella_direct_queue_create).
     if (DirectQueue* q = direct_queue_lookup(reinterpret_cast<void*>(stream))) {
         alignas(16) char buf[kMaxExplicitArgBytes];

@@ -38,6 +38,8 @@
 #include "launch.h"
 #include "out_store.h"
 #include "pool_body.h"
+#include "dense_body.h"
+#include "pack.h"
 
 namespace {
 
@@ -504,15 +506,19 @@ constexpr int kPackMax = PAELLA_CONV_PACK_MAX;    // members of one launch (the 
 // A member may also be a pooling operator (an inception module starts with three 1x1 convs and a 3x3 pool that all read
 // the module's input): its workgroups, one output element per thread with this kernel's workgroup size, come after all the
 // convs' (they are the shortest).
+// ... or a dense layer, one wave per output row (launches that carry the same stage of several small models' requests).
 union GroupMember {
     ConvArgs conv;
     paella::PoolArgs pool;
+    paella::DenseArgs dense;
     __host__ __device__ GroupMember() {}
 };
 
+enum MemberKind : unsigned { kMemberConv = 0, kMemberPool = 1, kMemberDense = 2 };
+
 struct ConvGroupArgs {
     unsigned start[kPackMax];  // first workgroup id of each member; 0xFFFFFFFF for unused entries
-    unsigned pool_mask;        // bit i: member i is a pooling operator
+    unsigned kinds;            // two bits per member: MemberKind
     unsigned reserved;
     GroupMember m[kPackMax];   // only the used entries are written to the argument ring
 };
@@ -524,12 +530,21 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kern
     for (int i = 1; i < kPackMax; ++i)
         if (blockIdx.x >= g.start[i]) idx = i;
     const unsigned bid = blockIdx.x - g.start[idx];
-    if ((g.pool_mask >> idx) & 1u) {
+    const unsigned kind = (g.kinds >> (2 * idx)) & 3u;
+    if (kind == kMemberPool) {
         const paella::PoolArgs& p = g.m[idx].pool;
         const unsigned blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
         paella::hook_entry(p.notifier, p.job_id, blocks);
         paella::pool_element(p, (int)(bid * (64 * KW) + threadIdx.x));
         paella::hook_exit(p.notifier, p.job_id, blocks);
+        return;
+    }
+    if (kind == kMemberDense) {
+        const paella::DenseArgs& d = g.m[idx].dense;
+        const unsigned blocks = d.hook_blocks ? d.hook_blocks : gridDim.x;
+        paella::hook_entry(d.notifier, d.job_id, blocks);
+        paella::dense_row(d, (int)(bid * KW + (threadIdx.x >> 6)), (int)(threadIdx.x & 63));
+        paella::hook_exit(d.notifier, d.job_id, blocks);
         return;
     }
     conv_tile<1, 1, KW, TAP_MAJOR>(g.m[idx].conv, bid);
@@ -890,7 +905,7 @@ extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, in
 
 namespace {
 
-// One launch of the group kernel over the first n members of g (their start[] and pool_mask filled; the rest marked
+// One launch of the group kernel over the first n members of g (their start[] and kinds filled; the rest marked
 // unused here).
 int launch_group_args(ConvGroupArgs& g, int n, int kw, int k_order, unsigned grid, unsigned dyn_lds, void* stream) {
     for (int i = n; i < kPackMax; ++i) g.start[i] = 0xFFFFFFFFu;
@@ -927,11 +942,36 @@ struct PackList {
     int members = 0;
 };
 
+// A job's whole ordered launch sequence (a model of small kernels is one scheduler stage), recorded between
+// paella_pack_sequence_begin and _end: the sequences of several requests of one model go out position by position, the
+// k-th launches of all of them in one grid, on one queue with the barrier bit set.
+struct SeqRecord {
+    unsigned kind = kMemberConv;
+    int kw = 4, k_order = 1;   // conv: the kernel variant; pool and dense ride in the <4, tap-major> variant, whose 256-thread
+                               // workgroups make their grids what the stand-alone kernels' are (the scheduler counts on that)
+    unsigned dyn_lds = 0;
+    unsigned units = 0;        // conv: workgroups; pool: output elements; dense: output rows
+    GroupMember m;
+};
+
+struct Sequence {
+    std::vector<SeqRecord> recs;
+};
+
+struct SeqList {
+    const void* key = nullptr;
+    std::vector<Sequence> seqs;
+};
+
 struct PackState {
     bool enabled = false;
-    int held = 0;                 // items over all lists
+    int held = 0;                 // items and sequences over all lists
     uint64_t first_held_ns = 0;
     PackList lists[4][2];         // by log2(waves per workgroup) and reduction order
+    std::vector<SeqList> seq_lists;
+    const void* rec_key = nullptr;  // the sequence being recorded (paella::g_pack_recording says whether one is)
+    void* rec_queue = nullptr;
+    Sequence rec;
 };
 
 std::atomic<uint64_t> g_pack_launches{0}, g_pack_members{0};  // over all threads, for reports
@@ -950,6 +990,18 @@ int kw_index(int kw) { return kw == 1 ? 0 : kw == 2 ? 1 : kw == 4 ? 2 : 3; }
 // Holds the call back if packing applies to it.  Returns false when the caller must launch it itself.
 bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n, void* stream, const paella::PoolArgs* pool = nullptr,
                unsigned pool_grid = 0) {
+    if (paella::g_pack_recording) {
+        if (n != 1 || pool || stream != g_pack.rec_queue) return false;  // the caller's launch then ends the recording
+        SeqRecord r;
+        r.kind = kMemberConv;
+        r.kw = plans[0]->kw;
+        r.k_order = plans[0]->k_order ? 1 : 0;
+        r.dyn_lds = plans[0]->dims.lds_bytes;
+        r.units = plans[0]->dims.grid;
+        r.m.conv = args[0];
+        g_pack.rec.recs.push_back(r);
+        return true;
+    }
     if (!g_pack.enabled || paella::timing_events().start != nullptr) return false;
     paella::DirectQueue* q = paella::direct_queue_lookup(stream);
     if (!q || paella::direct_queue_ordered(q)) return false;
@@ -989,7 +1041,7 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         size_t i = done;
         int total = 0;
         for (; i < list.items.size() && total + list.items[i].members() <= kPackMax; ++i) total += list.items[i].members();
-        g.pool_mask = 0;
+        g.kinds = 0;
         for (size_t k = done; k < i; ++k) {  // the convs of every item first ...
             const PackItem& it = list.items[k];
             for (int c = 0; c < it.n; ++c) {
@@ -1005,7 +1057,7 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
             if (!it.has_pool) continue;
             g.m[n].pool = it.pool;
             g.start[n] = grid;
-            g.pool_mask |= 1u << n;
+            g.kinds |= kMemberPool << (2 * n);
             grid += it.pool_grid;
             ++n;
         }
@@ -1035,8 +1087,91 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
     return launches;
 }
 
+unsigned units_to_grid(const SeqRecord& r) {
+    if (r.kind == kMemberPool) return (r.units + 255u) / 256u;  // one element per thread
+    if (r.kind == kMemberDense) return (r.units + 3u) / 4u;     // one row per wave
+    return r.units;
+}
+
+// The k-th launches of seqs[first .. first + n) as one grid on `queue`; a member with a notifier reports its own workgroups.
+int seq_launch_position(const std::vector<Sequence>& seqs, size_t first, int n, size_t k, void* queue) {
+    const SeqRecord& head = seqs[first].recs[k];
+    ConvGroupArgs g;
+    g.kinds = 0;
+    unsigned grid = 0, dyn_lds = 0;
+    for (int i = 0; i < n; ++i) {
+        const SeqRecord& r = seqs[first + (size_t)i].recs[k];
+        const unsigned wgs = units_to_grid(r);
+        g.m[i] = r.m;
+        if (r.kind == kMemberConv) g.m[i].conv.hook_blocks = wgs;
+        else if (r.kind == kMemberPool) g.m[i].pool.hook_blocks = wgs;
+        else g.m[i].dense.hook_blocks = wgs;
+        g.kinds |= r.kind << (2 * i);
+        g.start[i] = grid;
+        grid += wgs;
+        dyn_lds = std::max(dyn_lds, r.dyn_lds);
+    }
+    g_pack_launches.fetch_add(1, std::memory_order_relaxed);
+    g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
+    if (n == 1 && head.kind == kMemberConv) {
+        ConvKernel kern = pick_kernel(1, 1, head.kw, head.k_order);
+        g.m[0].conv.hook_blocks = 0;
+        if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
+        paella::launch(kern, dim3(grid), dim3(64u * (unsigned)head.kw), dyn_lds, reinterpret_cast<hipStream_t>(queue), g.m[0].conv);
+        return (int)hipGetLastError();
+    }
+    return launch_group_args(g, n, head.kw, head.k_order, grid, dyn_lds, queue);
+}
+
+// Sends seqs[first .. first + n) position by position on one queue of the shared set, with the barrier bit set.
+int seq_send_batch(const std::vector<Sequence>& seqs, size_t first, int n, void* queue) {
+    void* target = queue;
+    if (!target && paella_direct_queue_shared(&target) != 0) return -1;
+    paella::DirectQueue* q = paella::direct_queue_lookup(target);
+    if (!q) return -1;
+    const bool was_ordered = paella::direct_queue_ordered(q);
+    paella_direct_queue_set_ordered(target, 1);
+    int launches = 0;
+    for (size_t k = 0; k < seqs[first].recs.size(); ++k) {
+        if (seq_launch_position(seqs, first, n, k, target) != 0) return -1;
+        ++launches;
+    }
+    if (!was_ordered) paella_direct_queue_set_ordered(target, 0);
+    return launches;
+}
+
+int seq_send(SeqList& list, bool only_full) {
+    int launches = 0;
+    size_t done = 0;
+    while (done < list.seqs.size()) {
+        const size_t left = list.seqs.size() - done;
+        if (only_full && left < (size_t)kPackMax) break;
+        const int n = (int)std::min<size_t>(left, (size_t)kPackMax);
+        const int r = seq_send_batch(list.seqs, done, n, nullptr);
+        if (r < 0) return -1;
+        launches += r;
+        done += (size_t)n;
+        g_pack.held -= n;
+    }
+    list.seqs.erase(list.seqs.begin(), list.seqs.begin() + (long)done);
+    return launches;
+}
+
+bool same_signature(const Sequence& a, const Sequence& b) {
+    if (a.recs.size() != b.recs.size()) return false;
+    for (size_t k = 0; k < a.recs.size(); ++k)
+        if (a.recs[k].kind != b.recs[k].kind || a.recs[k].kw != b.recs[k].kw || a.recs[k].k_order != b.recs[k].k_order) return false;
+    return true;
+}
+
 int pack_send_all(bool only_full) {
     int launches = 0;
+    for (SeqList& list : g_pack.seq_lists) {
+        if (list.seqs.empty()) continue;
+        const int r = seq_send(list, only_full);
+        if (r < 0) return PAELLA_ENOSUP;
+        launches += r;
+    }
     for (int w = 0; w < 4; ++w)
         for (int o = 0; o < 2; ++o) {
             PackList& list = g_pack.lists[w][o];
@@ -1050,6 +1185,76 @@ int pack_send_all(bool only_full) {
 }
 
 }  // namespace
+
+namespace paella {
+
+thread_local bool g_pack_recording = false;
+
+bool pack_record_pool(const PoolArgs& a, void* stream) {
+    if (!g_pack_recording || stream != g_pack.rec_queue) return false;
+    SeqRecord r;
+    r.kind = kMemberPool;
+    r.units = (unsigned)((size_t)a.C * a.P * a.Q);
+    r.m.pool = a;
+    g_pack.rec.recs.push_back(r);
+    return true;
+}
+
+bool pack_record_dense(const DenseArgs& a, void* stream) {
+    if (!g_pack_recording || stream != g_pack.rec_queue) return false;
+    SeqRecord r;
+    r.kind = kMemberDense;
+    r.units = (unsigned)a.O;
+    r.m.dense = a;
+    g_pack.rec.recs.push_back(r);
+    return true;
+}
+
+void pack_sequence_break_slow() {
+    g_pack_recording = false;  // first: the launches below go through the same launch path
+    if (!g_pack.rec.recs.empty()) {
+        std::vector<Sequence> one(1);
+        one[0].recs.swap(g_pack.rec.recs);
+        if (seq_send_batch(one, 0, 1, g_pack.rec_queue) < 0) {
+            std::fprintf(stderr, "[paella] launch packing: a recorded sequence could not be sent\n");
+            std::abort();
+        }
+    }
+}
+
+}  // namespace paella
+
+extern "C" int paella_pack_sequence_begin(const void* key, void* queue) {
+    if (paella::g_pack_recording) return PAELLA_EINVAL;
+    paella::DirectQueue* q = paella::direct_queue_lookup(queue);
+    if (!g_pack.enabled || !q || !paella::direct_queue_ordered(q) || paella::timing_events().start != nullptr) return PAELLA_ENOSUP;
+    g_pack.rec_key = key;
+    g_pack.rec_queue = queue;
+    g_pack.rec.recs.clear();
+    paella::g_pack_recording = true;
+    return 0;
+}
+
+extern "C" int paella_pack_sequence_end(void) {
+    if (!paella::g_pack_recording) return 0;  // never begun, or ended by a launch the recorder does not take: all sent already
+    paella::g_pack_recording = false;
+    if (g_pack.rec.recs.empty()) return 0;
+    SeqList* list = nullptr;
+    for (SeqList& l : g_pack.seq_lists)
+        if (l.key == g_pack.rec_key) list = &l;
+    if (!list) {
+        g_pack.seq_lists.emplace_back();
+        list = &g_pack.seq_lists.back();
+        list->key = g_pack.rec_key;
+    }
+    if (!list->seqs.empty() && !same_signature(list->seqs.front(), g_pack.rec)) {
+        if (seq_send(*list, false) < 0) return PAELLA_ENOSUP;
+    }
+    list->seqs.emplace_back();
+    list->seqs.back().recs.swap(g_pack.rec.recs);
+    if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
+    return 0;
+}
 
 extern "C" int paella_pack_enable(int on) {
     if (!on && g_pack.held > 0) {
@@ -1095,7 +1300,7 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
         dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
     if (pack_hold(plans, args, n, stream)) return 0;
-    g.pool_mask = 0;
+    g.kinds = 0;
     return launch_group_args(g, n, plans[0]->kw, plans[0]->k_order, dims.grid, dyn_lds, stream);
 }
 
@@ -1150,7 +1355,7 @@ extern "C" int paella_conv2d_launch_group_pool(const paella_conv_operands* membe
     if (pack_hold(plans, args, n, stream, &pa, dims.grid - next)) return 0;
     g.m[n].pool = pa;
     g.start[n] = next;
-    g.pool_mask = 1u << n;
+    g.kinds = kMemberPool << (2 * n);
     return launch_group_args(g, n + 1, plans[0]->kw, 1, dims.grid, dyn_lds, stream);
 }
 

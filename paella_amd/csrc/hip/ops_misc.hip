@@ -13,6 +13,8 @@
 #include "launch.h"
 #include "out_store.h"
 #include "pool_body.h"
+#include "dense_body.h"
+#include "pack.h"
 
 namespace {
 
@@ -41,43 +43,11 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // ------------------------------------------------------------------------------------------ dense
-// One wave per output row; lanes stride the row with float4 loads (x stays in L1/L2).
-__global__ __launch_bounds__(256) void dense_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                    const float* __restrict__ bias, float* __restrict__ y, int I, int O,
-                                                    int act, uint32_t job_id, Notifier* notifier) {
-    paella::hook_entry(notifier, job_id);
-    const int lane = threadIdx.x & 63;
-    const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (o < O) {
-        const float* wr = w + (size_t)o * I;
-        float acc = 0.f;
-        if ((I & 3) == 0) {
-            const float4* w4 = reinterpret_cast<const float4*>(wr);
-            const float4* x4 = reinterpret_cast<const float4*>(x);
-            // four independent loads and sums per trip: a row of 2048 floats is two trips to memory, not eight
-            const int I4 = I / 4;
-            float a1 = 0.f, a2 = 0.f, a3 = 0.f;
-            int i = lane;
-            for (; i + 192 < I4; i += 256) {
-                const float4 p0 = w4[i], p1 = w4[i + 64], p2 = w4[i + 128], p3 = w4[i + 192];
-                const float4 q0 = x4[i], q1 = x4[i + 64], q2 = x4[i + 128], q3 = x4[i + 192];
-                acc += p0.x * q0.x + p0.y * q0.y + p0.z * q0.z + p0.w * q0.w;
-                a1 += p1.x * q1.x + p1.y * q1.y + p1.z * q1.z + p1.w * q1.w;
-                a2 += p2.x * q2.x + p2.y * q2.y + p2.z * q2.z + p2.w * q2.w;
-                a3 += p3.x * q3.x + p3.y * q3.y + p3.z * q3.z + p3.w * q3.w;
-            }
-            for (; i < I4; i += 64) {
-                const float4 a = w4[i], b = x4[i];
-                acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
-            }
-            acc = (acc + a1) + (a2 + a3);
-        } else {
-            for (int i = lane; i < I; i += 64) acc += wr[i] * x[i];
-        }
-        acc = wave_sum(acc);
-        if (lane == 0) store_out(y + o, act_apply(acc + (bias ? bias[o] : 0.f), act, 0.f, 0.f, 0.f));
-    }
-    paella::hook_exit(notifier, job_id);
+// One wave per output row (dense_body.h).
+__global__ __launch_bounds__(256) void dense_kernel(paella::DenseArgs a) {
+    paella::hook_entry(a.notifier, a.job_id);
+    paella::dense_row(a, (int)(blockIdx.x * 4 + (threadIdx.x >> 6)), (int)(threadIdx.x & 63));
+    paella::hook_exit(a.notifier, a.job_id);
 }
 
 // Long rows (I >= kDenseLongRow, a multiple of 4): with one wave per row a layer of few, long rows (an embedding
@@ -355,9 +325,11 @@ int paella_dense_launch(const float* x, const float* w, const float* bias, float
     if (dense_long(I))
         paella::launch(dense_long_kernel, dim3(blocks_for(O, 2)), dim3(512), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
                        (Notifier*)notifier);
-    else
-        paella::launch(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias, y, I, O, act, job_id,
-                       (Notifier*)notifier);
+    else {
+        paella::DenseArgs a{x, w, bias, y, I, O, act, job_id, 0u, (Notifier*)notifier};
+        if (paella::pack_record_dense(a, stream)) return 0;
+        paella::launch(dense_kernel, dim3(blocks_for(O, 4)), dim3(256), 0, (hipStream_t)stream, a);
+    }
     return (int)hipGetLastError();
 }
 
@@ -382,6 +354,7 @@ int paella_pool2d_launch(const paella_pool_desc* d, const float* x, float* y, vo
     PoolArgs a;
     if (!x || !y || !paella::pool_fill_args(d, x, y, job_id, notifier, &a)) return PAELLA_EINVAL;
     const int P = a.P, Q = a.Q;
+    if (paella::pack_record_pool(a, stream)) return 0;
     paella::launch(pool_kernel, dim3(blocks_for((size_t)d->C * P * Q, 256)), dim3(256), 0, (hipStream_t)stream, a);
     return (int)hipGetLastError();
 }

@@ -148,10 +148,13 @@ class ModelJob : public llis::job::CoroutineJob {
             // members of a group wait for what is ahead of them in the queue (a stream orders by itself); the first one
             // too, so that it is not held back for packing while the others go out
             if (direct_ && last > s) paella_direct_queue_set_ordered(target, 1);
+            // ... and the whole group is recorded, to go out together with the same group of other requests of this model
+            const bool recording = pack_ && last > s && paella_pack_sequence_begin(model_, target) == 0;
             for (int k = s; k <= last; ++k) {
                 if (k < last) check(paella_exec_launch_stage(exec_, k, target, 0, nullptr), "stage launch");
                 else check(paella_exec_launch_stage(exec_, k, target, id, get_finished_block_notifier()), "stage launch");
             }
+            if (recording) check(paella_pack_sequence_end(), "end of the recorded launch sequence");
             if (direct_ && last > s) paella_direct_queue_set_ordered(target, 0);
             s = last + 1;
         }

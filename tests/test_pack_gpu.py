@@ -145,3 +145,68 @@ def test_poll_sends_at_once_on_idle_queues_and_ordered_queues_are_not_held(ring,
     for a, b in zip(alone, ys):
         assert torch.equal(a, b)
     assert torch.equal(y_stream, alone[1])
+
+
+def small_net(cuda, rng):
+    """The small CNN's operators (conv 5x5, max pool, conv 5x5, max pool, dense) as library calls on one stream or queue."""
+    from paella_amd import ops
+    w1 = rng.standard_normal((8, 1, 5, 5)).astype(np.float32) * 0.2
+    w2 = rng.standard_normal((16, 8, 5, 5)).astype(np.float32) * 0.07
+    c1 = ops.Conv2d(w1, rng.standard_normal(8).astype(np.float32), pad=2, act=ops.ACT_RELU, in_hw=(28, 28))
+    c2 = ops.Conv2d(w2, rng.standard_normal(16).astype(np.float32), pad=2, act=ops.ACT_RELU, in_hw=(14, 14))
+    wd = torch.tensor(rng.standard_normal((10, 256)).astype(np.float32) * 0.06, device=cuda)
+    bd = torch.tensor(rng.standard_normal(10).astype(np.float32), device=cuda)
+
+    keep = []  # held launches read and write the intermediate tensors long after this function has returned
+
+    def run(x, stream=None, job_id=0, notifier=None, gap=False):
+        y1 = c1(x, stream=stream)
+        y2 = ops.pool2d(y1, 2, 2, stream=stream)
+        y3 = c2(y2, stream=stream)
+        y4 = ops.pool2d(y3, 3, 3, stream=stream)
+        keep.extend([y1, y2, y3, y4])
+        if gap:  # an operator the recorder does not take
+            g = ops.global_avgpool(y4, stream=stream)
+        out = ops.dense(y4.reshape(1, 256), wd, bd, stream=stream, job_id=job_id, notifier=notifier)
+        return (out, g) if gap else out
+    return run
+
+
+def test_recorded_sequences_of_several_requests_go_out_together(ring, cuda):
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(13)
+    net = small_net(cuda, rng)
+    xs = [torch.tensor(rng.standard_normal((1, 1, 28, 28)).astype(np.float32), device=cuda) for _ in range(11)]
+    alone = [net(x) for x in xs]
+    torch.cuda.synchronize()
+    key = ctypes.c_void_p(0x1234)
+    with ops.DirectQueue(ordered=True) as q:
+        assert lib.paella_pack_sequence_begin(key, ctypes.c_void_p(q.handle)) == -2  # packing is off on this thread
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            before = stats(lib)
+            outs = []
+            for j, x in enumerate(xs):
+                assert lib.paella_pack_sequence_begin(key, ctypes.c_void_p(q.handle)) == 0
+                outs.append(net(x, stream=q.handle, job_id=(j + 1) | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, j))))
+                assert lib.paella_pack_sequence_end() == 0
+            assert held(lib) == 11
+            assert lib.paella_pack_poll() == 10 and held(lib) == 0  # idle queues: eight requests in five launches, three in five more
+            after = stats(lib)
+            assert (after[0] - before[0], after[1] - before[1]) == (10, 55)
+            buf = np.zeros(11, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, 11, 20.0) == 11  # one end message per request: its dense layer's three workgroups, as launched alone
+            m = decode(buf)
+            assert sorted(m["job_id"]) == list(range(1, 12)) and np.all(m["num"] == 3) and np.all(m["is_start"] == 0)
+            # a sequence with an operator the recorder does not take: sent at once, in order, nothing held
+            assert lib.paella_pack_sequence_begin(key, ctypes.c_void_p(q.handle)) == 0
+            out_gap, g = net(xs[0], stream=q.handle, gap=True)
+            assert lib.paella_pack_sequence_end() == 0 and held(lib) == 0
+            q.wait()
+            assert torch.equal(out_gap, alone[0])
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for a, b in zip(alone, outs):
+        assert torch.equal(a, b)
