@@ -353,6 +353,8 @@ def main():
     ap.add_argument("--zoo-ops", nargs="?", const="all", default=None, metavar="MODELS",
                     help="only this: per operator family of every zoo model (or of the comma-separated ones), launches, time and rates "
                          "of one forward pass, one launch at a time")
+    ap.add_argument("--queue-probe", action="store_true",
+                    help="only: how many kernels run side by side and what sharing a launch gains (paella_queue_concurrency_probe), as a table on stderr")
     ap.add_argument("--roofline-only", default=None, metavar="MODEL",
                     help="only the isolated per-launch timing of one forward pass of MODEL (the leg roofline.achieved comes from)")
     ap.add_argument("--counter-pass", default=None, metavar="MODEL",
@@ -416,6 +418,29 @@ def main():
                     (op, row["launches"], row["us"], row["us_per_launch"], row["tflops"], 100 * row["frac_of_fp32_mfma_peak"],
                      row["gbytes_per_s"], 100 * row["frac_of_hbm_peak"]))
         print(json.dumps({"zoo_ops": table}), flush=True)
+        return
+    if args.queue_probe:
+        import ctypes
+        from paella_amd._abi import ConvDesc
+        lib = _abi.ops()
+        shapes = [("Inception-v3 8x8 1280->320 1x1", 1280, 8, 320, 1, 0), ("Inception-v3 17x17 768->192 1x1", 768, 17, 192, 1, 0),
+                  ("Inception-v3 35x35 288->64 1x1", 288, 35, 64, 1, 0), ("ResNet-18 14x14 256->256 3x3", 256, 14, 256, 3, 1),
+                  ("ResNet-18 56x56 64->64 3x3", 64, 56, 64, 3, 1), ("ResNet-18 7x7 512->512 3x3", 512, 7, 512, 3, 1)]
+        cases = [("1 queue, no barrier bit", 1, 1, 0), ("1 queue, barrier bit", 1, 1, 1), ("2 queues", 1, 2, 1), ("4 queues", 1, 4, 1), ("8 queues", 1, 8, 1),
+                 ("4 queues, 2 per launch", 2, 4, 1), ("4 queues, 4 per launch", 4, 4, 1)]
+        out = {}
+        log("[bench] 16 independent instances of one conv layer, microseconds per conv (200 rounds):")
+        log("[bench] %-34s " % "layer" + " ".join("%24s" % c[0] for c in cases))
+        for name, c, hw, k, r, pad in shapes:
+            d = ConvDesc(c, hw, hw, k, r, r, 1, 1, pad, pad, 1, 1, 1, 1, 0.0, 0.0)
+            row = []
+            for label, per, nq, ordered in cases:
+                us = ctypes.c_double()
+                _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 16, per, nq, ordered, 200, ctypes.byref(us)), "paella_queue_concurrency_probe")
+                row.append(us.value)
+            out[name] = dict(zip([c[0] for c in cases], row))
+            log("[bench] %-34s " % name + " ".join("%24.2f" % v for v in row))
+        print(json.dumps({"queue_probe_us_per_conv": out}))
         return
     if args.roofline_only:
         rl = conv_roofline(models, hip, args.roofline_only, reps=50)

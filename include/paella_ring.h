@@ -73,6 +73,15 @@ int paella_empty_kernel_probe(int iters, double* median_us);
  * the measured denominator next to the published 157.3 TFLOP/s. */
 int paella_mfma_peak_probe(double* tflops);
 
+/* How many kernels the device runs side by side, and what sharing a launch is worth.  `instances` independent copies of
+ * the conv layer `desc` (32 x 32 tile; own input, output and workspace each, shared weights) are launched round-robin over
+ * `queues` direct-dispatch queues (with the barrier bit when `ordered`), `per_launch` (1 .. PAELLA_CONV_GROUP_MAX) of them
+ * in one grid, `reps` times over; *us_per_conv = elapsed / (reps x instances).  One unordered queue against four shows
+ * whether a queue overlaps its kernels; per_launch 1 against 4 shows the gain of packing. */
+struct paella_conv_desc;
+int paella_queue_concurrency_probe(const struct paella_conv_desc* desc, int instances, int per_launch, int queues, int ordered, int reps,
+                                   double* us_per_conv);
+
 #ifdef __cplusplus
 }
 #endif

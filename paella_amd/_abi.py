@@ -137,6 +137,7 @@ RING_SYMBOLS = {
     "paella_empty_kernel_probe": (c_int, [c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_echo": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "paella_mfma_peak_probe": (c_int, [ctypes.POINTER(c_double)]),
+    "paella_queue_concurrency_probe": (c_int, [ctypes.POINTER(ConvDesc), c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_double)]),
 }
 
 

@@ -11,6 +11,7 @@
 
 #include "direct_dispatch.h"
 #include "paella_hip.h"
+#include "paella_ops.h"
 #include "paella_ring.h"
 #include <llis/ipc/shm_primitive_channel.h>
 #include <llis/job/finished_block_notifier.h>
@@ -361,6 +362,81 @@ int paella_mfma_peak_probe(double* tflops) {
     hipFree(sink);
     *tflops = best;
     return 0;
+}
+
+int paella_queue_concurrency_probe(const paella_conv_desc* desc, int instances, int per_launch, int queues, int ordered, int reps,
+                                   double* us_per_conv) {
+    if (!desc || !us_per_conv || instances < 1 || instances > 64 || per_launch < 1 || per_launch > PAELLA_CONV_GROUP_MAX ||
+        instances % per_launch != 0 || queues < 1 || queues > 16 || reps < 1)
+        return -1;
+    paella_conv_plan plan;
+    if (int rc = paella_conv2d_plan(desc, 0, 0, &plan)) return rc;
+    if (plan.kind != 0 || plan.mi != 1 || plan.ni != 1) return -2;
+    const paella_conv_desc& d = *desc;
+    std::vector<float> w((size_t)d.K * d.C * d.R * d.S);
+    unsigned state = 12345u;
+    for (float& v : w) {
+        state = state * 1664525u + 1013904223u;
+        v = ((int)(state >> 16) % 2001 - 1000) * 5e-5f;
+    }
+    std::vector<char> blob(plan.blob_bytes);
+    if (int rc = paella_conv2d_pack(&plan, w.data(), blob.data())) return rc;
+    struct Instance { void *x = nullptr, *y = nullptr, *ws = nullptr; };
+    std::vector<Instance> inst((size_t)instances);
+    std::vector<void*> qs;
+    void *blob_dev = nullptr, *bias = nullptr;
+    const size_t xb = (size_t)d.C * d.H * d.W * 4, yb = (size_t)d.K * plan.P * plan.Q * 4;
+    int rc = 0;
+    auto ok = [&](hipError_t e) { if (e != hipSuccess && rc == 0) rc = (int)e; return e == hipSuccess; };
+    ok(hipMalloc(&blob_dev, plan.blob_bytes)) && ok(hipMemcpy(blob_dev, blob.data(), plan.blob_bytes, hipMemcpyHostToDevice));
+    ok(hipMalloc(&bias, (size_t)d.K * 4)) && ok(hipMemset(bias, 0, (size_t)d.K * 4));
+    for (Instance& in : inst) {
+        ok(hipMalloc(&in.x, xb)) && ok(hipMemset(in.x, 0, xb));
+        ok(hipMalloc(&in.y, yb));
+        if (plan.workspace_bytes) ok(hipMalloc(&in.ws, plan.workspace_bytes)) && ok(hipMemset(in.ws, 0, plan.workspace_bytes));
+    }
+    ok(hipDeviceSynchronize());
+    for (int i = 0; i < queues && rc == 0; ++i) {
+        void* q = nullptr;
+        rc = paella_direct_queue_create(&q);
+        if (rc == 0) {
+            qs.push_back(q);
+            paella_direct_queue_set_ordered(q, ordered);
+        }
+    }
+    double us = 0;
+    for (int pass = 0; pass < 2 && rc == 0; ++pass) {  // a short pass first: the argument rings and the caches are warm afterwards
+        const int n = pass ? reps : std::max(1, reps / 10);
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int r = 0; r < n && rc == 0; ++r) {
+            size_t qi = 0;
+            for (int i = 0; i < instances && rc == 0; i += per_launch) {
+                if (per_launch == 1) {
+                    rc = paella_conv2d_launch(&plan, (const float*)inst[i].x, blob_dev, (const float*)bias, nullptr, nullptr, (float*)inst[i].y, inst[i].ws,
+                                              qs[qi], 0, nullptr);
+                } else {
+                    paella_conv_operands m[PAELLA_CONV_GROUP_MAX];
+                    for (int k = 0; k < per_launch; ++k)
+                        m[k] = paella_conv_operands{&plan, (const float*)inst[i + k].x, blob_dev, (const float*)bias, nullptr, nullptr, (float*)inst[i + k].y,
+                                                    inst[i + k].ws};
+                    rc = paella_conv2d_launch_group(m, per_launch, qs[qi], 0, nullptr);
+                }
+                qi = (qi + 1) % qs.size();
+            }
+        }
+        for (void* q : qs) paella_direct_queue_wait(q);
+        us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / ((double)n * instances);
+    }
+    for (void* q : qs) paella_direct_queue_destroy(q);
+    for (Instance& in : inst) {
+        hipFree(in.x);
+        hipFree(in.y);
+        if (in.ws) hipFree(in.ws);
+    }
+    hipFree(blob_dev);
+    hipFree(bias);
+    *us_per_conv = us;
+    return rc;
 }
 
 }  // extern "C"
