@@ -298,8 +298,11 @@ def search_rate(arm, tenants, slo_us, iters=7):
     f = 0.5
     for _ in range(iters):
         rate = f * sat
+        # 10 240 requests per point, fewer only where they would take more than 1.5 s to arrive (arms whose knee is at a few
+        # hundred requests/s), never under 2048
+        n_point = min(SEARCH_REQUESTS, max(2048, int(rate * 1.5)))
         for attempt, seed in enumerate((1, 2)):
-            p = point_of(arm.run(1e6 / rate, SEARCH_REQUESTS, 512, seed=seed), tenants, rate)
+            p = point_of(arm.run(1e6 / rate, n_point, 512, seed=seed), tenants, rate)
             p["meets_slo"] = meets(p, tenants, slo_us)
             p["attempt"] = attempt
             points.append(p)
@@ -420,7 +423,6 @@ def main():
         print(json.dumps({"zoo_ops": table}), flush=True)
         return
     if args.queue_probe:
-        import ctypes
         from paella_amd._abi import ConvDesc
         lib = _abi.ops()
         shapes = [("Inception-v3 8x8 1280->320 1x1", 1280, 8, 320, 1, 0), ("Inception-v3 17x17 768->192 1x1", 768, 17, 192, 1, 0),

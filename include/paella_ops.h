@@ -174,6 +174,7 @@ int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void*
 int paella_pack_enable(int on);
 int paella_pack_poll(void);
 int paella_pack_flush(void);
+void paella_pack_poll_hook(void); /* paella_pack_poll with the signature of a serving-loop hook (llis::job::Context::add_poll_hook) */
 int paella_pack_stats(uint64_t* launches, uint64_t* members);
 
 /* The same for a job that issues several dependent launches at once on an ORDERED direct-dispatch queue (a model of

@@ -87,6 +87,7 @@ OPS_SYMBOLS = {
     "paella_pack_enable": (c_int, [c_int]),
     "paella_pack_poll": (c_int, []),
     "paella_pack_flush": (c_int, []),
+    "paella_pack_poll_hook": (None, []),
     "paella_pack_stats": (c_int, [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]),
     "paella_pack_sequence_begin": (c_int, [c_void_p, c_void_p]),
     "paella_pack_sequence_end": (c_int, []),

@@ -1272,6 +1272,8 @@ extern "C" int paella_pack_poll(void) {
     return pack_send_all(true);
 }
 
+extern "C" void paella_pack_poll_hook(void) { (void)paella_pack_poll(); }
+
 extern "C" int paella_pack_stats(uint64_t* launches, uint64_t* members) {
     if (launches) *launches = g_pack_launches.load(std::memory_order_relaxed);
     if (members) *members = g_pack_members.load(std::memory_order_relaxed);

@@ -107,7 +107,7 @@ class ModelJob : public llis::job::CoroutineJob {
         // holds them and lets them go from its loop.
         const char* pack = std::getenv("PAELLA_PACK");
         pack_ = direct_ && !(pack && std::strcmp(pack, "0") == 0);
-        if (pack_) llis::job::Context::add_poll_hook(&ModelJob::pack_poll);
+        if (pack_) llis::job::Context::add_poll_hook(&paella_pack_poll_hook);  // one address for every adapter library: registered once
     }
 
     void body(void* io_ptr) override {
@@ -171,8 +171,6 @@ class ModelJob : public llis::job::CoroutineJob {
 
   private:
     void* stream() { return reinterpret_cast<void*>(get_cuda_stream()); }
-
-    static void pack_poll() { paella_pack_poll(); }
 
     // Packing is a property of the launching thread (the serving thread, which also runs pack_poll from its loop).
     static void enable_packing_on_this_thread() {
