@@ -495,6 +495,21 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_kernel
     conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
 }
 
+// The same for up to kPackMax such convs of different requests in one launch (launch packing).
+struct ConvPreGroupArgs {
+    unsigned start[PAELLA_CONV_PACK_MAX];  // first workgroup id of each problem; 0xFFFFFFFF for unused entries
+    ConvPreArgs m[PAELLA_CONV_PACK_MAX];   // only the used entries are written to the argument ring
+};
+
+template <int KW>
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
+        if (blockIdx.x >= g.start[i]) idx = i;
+    conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
+}
+
 // Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
 // projection beside a residual block's first 3x3, the parallel branches of an inception module) share a grid, one
 // problem's workgroups after the other's.  All use the smallest tile and the same wave count; the hooks see one
@@ -969,6 +984,11 @@ struct PackState {
     uint64_t first_held_ns = 0;
     PackList lists[4][2];         // by log2(waves per workgroup) and reduction order
     std::vector<SeqList> seq_lists;
+    struct PreItem {
+        ConvPreArgs a;
+        unsigned grid = 0, dyn_lds = 0;
+    };
+    std::vector<PreItem> pre_lists[4];  // convs with a fused input transform, by log2(waves per workgroup)
     const void* rec_key = nullptr;  // the sequence being recorded (paella::g_pack_recording says whether one is)
     void* rec_queue = nullptr;
     Sequence rec;
@@ -1164,8 +1184,15 @@ bool same_signature(const Sequence& a, const Sequence& b) {
     return true;
 }
 
+int pre_send_all(bool only_full);  // below, with the kernels it launches
+
 int pack_send_all(bool only_full) {
     int launches = 0;
+    {
+        const int r = pre_send_all(only_full);
+        if (r < 0) return PAELLA_ENOSUP;
+        launches += r;
+    }
     for (SeqList& list : g_pack.seq_lists) {
         if (list.seqs.empty()) continue;
         const int r = seq_send(list, only_full);
@@ -1471,6 +1498,90 @@ static ConvPreKernel pick_pre_kernel(int kw) {
     }
 }
 
+namespace {
+
+typedef void (*ConvPreGroupKernel)(ConvPreGroupArgs);
+
+ConvPreGroupKernel pick_pre_group_kernel(int kw) {
+    switch (kw) {
+        case 1: return conv_mfma_pre_group_kernel<1>;
+        case 2: return conv_mfma_pre_group_kernel<2>;
+        case 4: return conv_mfma_pre_group_kernel<4>;
+        case 8: return conv_mfma_pre_group_kernel<8>;
+        default: return nullptr;
+    }
+}
+
+// Launch packing of convs with a fused input transform: held like the plain ones (pack_hold), in lists of their own
+// because they run in a kernel of their own.
+bool pack_hold_pre(const paella_conv_plan* plan, const ConvPreArgs& a, void* stream) {
+    if (paella::g_pack_recording || !g_pack.enabled || paella::timing_events().start != nullptr) return false;
+    paella::DirectQueue* q = paella::direct_queue_lookup(stream);
+    if (!q || paella::direct_queue_ordered(q)) return false;
+    PackState::PreItem it;
+    it.a = a;
+    it.grid = plan->dims.grid;
+    it.dyn_lds = plan->dims.lds_bytes;
+    it.a.conv.hook_blocks = it.grid;
+    g_pack.pre_lists[kw_index(plan->kw)].push_back(it);
+    if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
+    return true;
+}
+
+int pre_send_all(bool only_full) {
+    int launches = 0;
+    for (int w = 0; w < 4; ++w) {
+        std::vector<PackState::PreItem>& list = g_pack.pre_lists[w];
+        size_t done = 0;
+        const int kw = 1 << w;
+        while (done < list.size()) {
+            const size_t left = list.size() - done;
+            if (only_full && left < (size_t)kPackMax) break;
+            const int n = (int)std::min<size_t>(left, (size_t)kPackMax);
+            void* target = nullptr;
+            if (paella_direct_queue_shared(&target) != 0) return -1;
+            unsigned grid = 0, dyn_lds = 0;
+            int rc = 0;
+            if (n == 1) {
+                ConvPreKernel kern = pick_pre_kernel(kw);
+                ConvPreArgs a = list[done].a;
+                a.conv.hook_blocks = 0;
+                rc = allow_lds(reinterpret_cast<const void*>(kern), list[done].dyn_lds);
+                if (rc == 0) {
+                    paella::launch(kern, dim3(list[done].grid), dim3(64u * (unsigned)kw), list[done].dyn_lds, reinterpret_cast<hipStream_t>(target), a);
+                    rc = (int)hipGetLastError();
+                }
+            } else {
+                ConvPreGroupArgs g;
+                for (int i = 0; i < n; ++i) {
+                    g.m[i] = list[done + (size_t)i].a;
+                    g.start[i] = grid;
+                    grid += list[done + (size_t)i].grid;
+                    dyn_lds = std::max(dyn_lds, list[done + (size_t)i].dyn_lds);
+                }
+                for (int i = n; i < kPackMax; ++i) g.start[i] = 0xFFFFFFFFu;
+                ConvPreGroupKernel kern = pick_pre_group_kernel(kw);
+                rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds);
+                if (rc == 0) {
+                    paella::launch_used(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(target),
+                                        offsetof(ConvPreGroupArgs, m) + (size_t)n * sizeof(ConvPreArgs), g);
+                    rc = (int)hipGetLastError();
+                }
+            }
+            if (rc != 0) return -1;
+            ++launches;
+            g_pack_launches.fetch_add(1, std::memory_order_relaxed);
+            g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
+            g_pack.held -= n;
+            done += (size_t)n;
+        }
+        list.erase(list.begin(), list.begin() + (long)done);
+    }
+    return launches;
+}
+
+}  // namespace
+
 extern "C" int paella_conv2d_plan_takes_input_transform(const paella_conv_plan* plan) {
     return plan && plan->kind == 0 && plan->mi == 1 && plan->ni == 1 && plan->k_order == 1 ? 1 : 0;
 }
@@ -1507,6 +1618,7 @@ extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, co
     a.pre.scale = in_scale;
     a.pre.shift = in_shift;
     a.pre.lo = in_act == PAELLA_ACT_RELU ? 0.f : -__builtin_inff();
+    if (pack_hold_pre(plan, a, stream)) return 0;
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
     paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();

@@ -210,3 +210,46 @@ def test_recorded_sequences_of_several_requests_go_out_together(ring, cuda):
     torch.cuda.synchronize()
     for a, b in zip(alone, outs):
         assert torch.equal(a, b)
+
+
+def test_convs_with_a_fused_input_transform_are_packed_among_themselves(ring, cuda):
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(14)
+    cases = []
+    for c, k, hw, r, pad in [(256, 128, 14, 1, 0), (128, 32, 14, 3, 1), (512, 128, 7, 1, 0), (128, 32, 28, 3, 1), (64, 128, 56, 1, 0)]:
+        w = rng.standard_normal((k, c, r, r)).astype(np.float32) / np.sqrt(c * r * r)
+        conv = ops.Conv2d(w, None, pad=pad, in_hw=(hw, hw))
+        assert conv.takes_input_transform()
+        x = torch.tensor(rng.standard_normal((1, c, hw, hw)).astype(np.float32), device=cuda)
+        sc = torch.tensor(rng.uniform(0.5, 1.5, c).astype(np.float32), device=cuda)
+        sh = torch.tensor(rng.standard_normal(c).astype(np.float32) * 0.1, device=cuda)
+        cases.append((conv, x, sc, sh))
+    alone = [conv(x, in_scale=sc, in_shift=sh, in_act=ops.ACT_RELU) for conv, x, sc, sh in cases]
+    torch.cuda.synchronize()
+    batch = lib.paella_ring_batch_size()
+    with ops.DirectQueue() as q:
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            before = stats(lib)
+            outs = []
+            for j, (conv, x, sc, sh) in enumerate(cases):
+                y = torch.zeros_like(alone[j])
+                conv(x, out=y, stream=q.handle, job_id=(j + 1) | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, j)),
+                     in_scale=sc, in_shift=sh, in_act=ops.ACT_RELU)
+                outs.append(y)
+            assert held(lib) == 5
+            assert lib.paella_pack_flush() == 1 and held(lib) == 0
+            after = stats(lib)
+            assert (after[0] - before[0], after[1] - before[1]) == (1, 5)
+            want = sum((c[0].plan.dims.grid + batch - 1) // batch for c in cases)
+            buf = np.zeros(want, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want, 20.0) == want
+            m = decode(buf)
+            for j, c in enumerate(cases):
+                assert m["num"][m["job_id"] == j + 1].sum() == c[0].plan.dims.grid
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for a, b in zip(alone, outs):
+        assert torch.equal(a, b)
