@@ -253,3 +253,81 @@ def test_convs_with_a_fused_input_transform_are_packed_among_themselves(ring, cu
     torch.cuda.synchronize()
     for a, b in zip(alone, outs):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_random_mixes_of_calls_pack_to_the_bits_of_separate_launches(ring, cuda, seed):
+    """Seeded mixes of single convs (both reduction orders, 2 to 8 waves), pairs and conv + pool calls, each under its own job id:
+    whatever way the packer cuts them into launches, outputs equal those of separate launches bit for bit and every notifier
+    counts exactly its own workgroups."""
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(seed)
+
+    def conv_of(c, k, hw, r, stride=1):
+        w = rng.standard_normal((k, c, r, r)).astype(np.float32) / np.sqrt(c * r * r)
+        b = rng.standard_normal(k).astype(np.float32) if rng.random() < 0.7 else None
+        conv = ops.Conv2d(w, b, stride=stride, pad=r // 2, act=ops.ACT_RELU if rng.random() < 0.5 else ops.ACT_NONE, in_hw=(hw, hw))
+        assert (conv.plan.mi, conv.plan.ni) == (1, 1)
+        x = torch.tensor(rng.standard_normal((1, c, hw, hw)).astype(np.float32), device=cuda)
+        return conv, x
+
+    calls = []  # (kind, [(conv, x), ...])
+    for _ in range(14):
+        kind = rng.choice(["single", "single", "single", "pair", "pool"])
+        hw = int(rng.choice([7, 9, 14, 17, 28, 35]))
+        if kind == "single":
+            c = int(rng.choice([3, 5, 8, 16, 24, 64, 160, 512]))
+            calls.append(("single", [conv_of(c, int(rng.choice([8, 24, 40, 96, 200])), hw, int(rng.choice([1, 3])), int(rng.choice([1, 2])))]))
+        else:
+            c = int(rng.choice([16, 64, 192]))  # tap-major, eight waves: what the executor groups
+            members = [conv_of(c, int(rng.choice([32, 48, 96])), hw, 1) for _ in range(2)]
+            if members[0][0].plan.kw != members[1][0].plan.kw:
+                continue
+            members[1] = (members[1][0], members[0][1])  # both read one input, as the branches of a module do
+            calls.append((kind, members))
+    alone = []
+    for kind, members in calls:
+        ys = [conv(x) for conv, x in members]
+        if kind == "pool":
+            ys.append(ops.pool2d(members[0][1], 3, 1, pad=1, is_avg=True, count_include_pad=False))
+        alone.append(ys)
+    torch.cuda.synchronize()
+    batch = lib.paella_ring_batch_size()
+    per = lambda n: (n + batch - 1) // batch
+    with ops.DirectQueue() as q:
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            got, grids = [], []
+            for j, (kind, members) in enumerate(calls):
+                nf = ctypes.c_void_p(lib.paella_ring_notifier(h, j))
+                jid = (j + 1) | NO_START
+                if kind == "single":
+                    conv, x = members[0]
+                    got.append([conv(x, stream=q.handle, job_id=jid, notifier=nf)])
+                    grids.append(conv.plan.dims.grid)
+                elif kind == "pair":
+                    got.append(ops.conv2d_group([m[0] for m in members], [m[1] for m in members], stream=q.handle, job_id=jid, notifier=nf))
+                    grids.append(sum(m[0].plan.dims.grid for m in members))
+                else:
+                    x = members[0][1]
+                    ys, py = ops.conv2d_group_pool([m[0] for m in members], [x, x], x, 3, 1, pad=1, is_avg=True, count_include_pad=False,
+                                                   stream=q.handle, job_id=jid, notifier=nf)
+                    got.append(ys + [py])
+                    block = 64 * members[0][0].plan.kw
+                    grids.append(sum(m[0].plan.dims.grid for m in members) + (x.shape[1] * x.shape[2] * x.shape[3] + block - 1) // block)
+            assert held(lib) == len(calls)
+            assert lib.paella_pack_flush() >= 1 and held(lib) == 0
+            want = sum(per(g) for g in grids)
+            buf = np.zeros(want, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want, 20.0) == want
+            m = decode(buf)
+            for j, g in enumerate(grids):
+                mine = m["job_id"] == j + 1
+                assert m["num"][mine].sum() == g and mine.sum() == per(g) and np.all(m["is_start"][mine] == 0), (j, calls[j][0])
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for ys, zs in zip(alone, got):
+        for a, b in zip(ys, zs):
+            assert torch.equal(a, b)
