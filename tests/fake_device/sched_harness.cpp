@@ -13,6 +13,7 @@
 //   put TYPE SLOT BYTE          fill the slot's input with BYTE;   get TYPE SLOT -> "out B0 B1 ..." (first 8 output bytes)
 //   log                         print the event log so far (also printed at exit)
 
+#include <llis/job/context.h>
 #include <llis/ipc/name_format.h>
 #include <llis/ipc/shm_channel.h>
 #include <llis/ipc/unix_datagram_socket.h>
@@ -63,12 +64,14 @@ struct Harness {
     ClientId client_id = 0;
     std::vector<JobType> types;
     unsigned completions = 0, wakeups = 0, launches = 0;
+    unsigned long long polls = 0;
 
     void poll(bool drain = true) {
         int idle = 0;
         while (idle < 4) {
             const size_t before = server->get_event_log()->events().size();
             server->poll_once();
+            ++polls;
             idle = server->get_event_log()->events().size() == before ? idle + 1 : 0;
             if (drain) drain_client();
         }
@@ -102,7 +105,12 @@ void on_fatal_signal(int sig) {
 
 }  // namespace
 
+static unsigned long long g_hook_calls = 0;
+static void count_poll_hook() { ++g_hook_calls; }
+
 int main() {
+    llis::job::Context::add_poll_hook(&count_poll_hook);
+    llis::job::Context::add_poll_hook(&count_poll_hook);
     // The script owns the device: a background thread that completes operations on its own (what the
     // in-process serving tests ask the scripted device for) would race every "step" of the script.
     if (const char* autorun = std::getenv("FAKE_HIP_AUTORUN"); autorun && *autorun == '1') {
@@ -238,6 +246,8 @@ int main() {
         }
     }
     std::printf("wakeups %u completions %u pending %u\n", h.wakeups, h.completions, fake_hip_pending());
+    // the serving loop's per-turn hooks of job libraries (llis::job::Context::add_poll_hook): once per turn, registered twice
+    std::printf("hooks %llu polls %llu\n", g_hook_calls, h.polls);
     std::printf("--- event log\n");
     std::fputs(h.server->get_event_log()->to_text().c_str(), stdout);
     if (fake_hip_pending() == 0 && h.completions != h.launches) {

@@ -36,6 +36,8 @@ def test_policy_matches_oracle_on_a_mixed_scenario(policy, streams):
     assert len(done) == 6
     summary = [r for r in replies if r.startswith("wakeups")][0].split()
     assert summary[1] == "6" and summary[3] == "6" and summary[5] == "0"  # every request woke the client once
+    hooks = [r for r in replies if r.startswith("hooks")][0].split()
+    assert int(hooks[1]) == int(hooks[3]) > 0  # a job library's hook runs once per turn of the serving loop, however often it registered
 
 
 @pytest.mark.parametrize("mem", ["marker", "hostfunc"])
