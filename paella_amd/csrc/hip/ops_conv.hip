@@ -741,13 +741,17 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             const int cap = 288;
             // How far the split goes is a trade between a kernel's latency (more, smaller workgroups) and the fixed cost of a
             // workgroup and of the exchange of partial tiles (fewer, larger ones).  Layers under 16 MFLOP go down to 2 chunks per
-            // wave, the others keep 6.  Served by full3 at saturation, median of three runs, requests/s against the earlier rule
+            // wave, the others kept 6 at first.  Served by full3 at saturation, median of three runs, requests/s against the earlier rule
             // (2 chunks for layers of at most 32 tiles, 4 otherwise): Inception-v3 4310 -> 4630, ResNet-50 5490 -> 5605,
             // GoogLeNet 9520 -> 9500, MobileNetV2 8390 -> 8240, DenseNet-121 3650 -> 3540 (its 25-50 MFLOP pointwise layers on
             // 14 x 14 maps are a pure chain and would rather be split), small CNN : Inception-v3 = 9 : 1 35.9 -> 37.1 thousand;
             // four passes in flight without scheduler: Inception-v3 4.81 -> 5.00 thousand passes/s; one launch at a time 9.09 ->
             // 9.20 us.  Thresholds of 32 and 64 MFLOP gave Inception-v3 4617 and 4443; 5 or 8 chunks instead of 6: 4552, 4588.
-            const int min_chunks = plan->flops < 16e6 ? 2 : 6;
+            // With launches of several requests packed together (paella_pack_*) the parallelism that splits provided comes from
+            // the other requests, and the same measurement (one box, packing on) moved the larger layers to 9 chunks per wave:
+            // 6 / 8 / 9 / 10 / 12 chunks: Inception-v3 5036 / 5238 / 5286 / 5306 / 5323, ResNet-50 6381 / 6325 / 6438 / 6447 / 6430,
+            // DenseNet-121 5173 / 5159 / 5139 / 5043 / 5013 requests/s, the 9 : 1 mix 43.9 / 44.9 / 44.6 / 44.8 / 44.9 thousand.
+            const int min_chunks = plan->flops < 16e6 ? 2 : 9;
             while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= min_chunks) splits *= 2;
         }
         int chunks_per_split = (nchunks + splits - 1) / splits;
