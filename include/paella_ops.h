@@ -160,10 +160,11 @@ int paella_conv2d_launch_group(const paella_conv_operands* members, int n, void*
 
 /* Launch packing.  A hardware queue of this device runs one kernel at a time and four run side by side, so at batch 1 a
  * conv that fills a fifth of the compute units still occupies a queue for its whole latency.  After paella_pack_enable(1)
- * on a thread, that thread's paella_conv2d_launch / paella_conv2d_launch_group calls on the 32 x 32 tile whose target is
- * an UNORDERED direct-dispatch queue (the serving path: the scheduler orders a job's stages through the notification
+ * on a thread, that thread's paella_conv2d_launch / _launch_group / _launch_group_pool / _launch_transformed calls on the
+ * 32 x 32 tile whose target is an UNORDERED direct-dispatch queue (the serving path: the scheduler orders a job's stages through the notification
  * ring) are held back and sent together, up to PAELLA_CONV_PACK_MAX problems of any jobs in one grid, every problem
- * reporting to its own job id and notifier exactly as if launched alone; results are bit-identical.  Everything else
+ * reporting to its own job id and notifier exactly as if launched alone (convs with a fused input transform share launches
+ * among themselves, the others among themselves); results are bit-identical.  Everything else
  * (HIP streams, ordered queues, other operators, larger tiles) is launched at once as before.  The thread must call
  * paella_pack_poll() from its loop: it sends what is held as soon as a queue of the shared set (paella_direct_queue_shared)
  * has no packet waiting, when a launch is full, or after 30 us at the latest, on the least loaded queue of that set, and
