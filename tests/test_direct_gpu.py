@@ -1,6 +1,8 @@
 """Direct dispatch (AQL packets on the library's own hardware queues) must run the very same kernels as the
 HIP launch path: every result here is compared bit for bit with the stream path, which the other GPU tests
 hold against the CPU oracle."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -105,3 +107,20 @@ def test_model_forward_on_ordered_direct_queue(cuda, model):
                 assert np.array_equal(ex.get_output(), ref)
     finally:
         ex.close()
+
+
+def test_queue_concurrency_probe_runs_and_reports_a_time(cuda):
+    """The probe behind bench.py --queue-probe: rejects shapes it is not for, returns a positive time otherwise, and four
+    queues are not slower than one."""
+    from paella_amd import _abi
+    from paella_amd._abi import ConvDesc
+    lib = _abi.ops()
+    d = ConvDesc(64, 14, 14, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 0.0)
+    us = ctypes.c_double()
+    assert lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 3, 2, 1, 5, ctypes.byref(us)) == -1  # 8 instances, 3 per launch
+    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 1, 1, 20, ctypes.byref(us)), "probe, one queue")
+    one = us.value
+    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 4, 1, 20, ctypes.byref(us)), "probe, four queues")
+    four = us.value
+    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 4, 4, 1, 20, ctypes.byref(us)), "probe, four per launch")
+    assert 0.1 < four <= one * 1.1 and 0.05 < us.value < one * 1.1, (one, four, us.value)
