@@ -116,6 +116,9 @@ struct PreOp {
 template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
+    // A grouped launch starts every conv at a multiple of eight workgroups (see align_start): the ids between the end of one
+    // problem and the start of the next belong to no tile and report to nobody.
+    if (bid >= (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
     // Waves of this workgroup whose result stores have been acknowledged (see the end of this function); cleared here, and
@@ -924,6 +927,11 @@ extern "C" int paella_conv2d_group_dims(const paella_conv_plan* const* plans, in
 
 namespace {
 
+// First workgroup id of the next conv of a grouped launch.  Workgroup ids are dealt round-robin over the eight XCDs, and
+// conv_tile gives the ids of one XCD a contiguous run of the problem's work list (same weights or neighbouring pixels in one
+// L2): that only holds for a problem whose first id is a multiple of eight.
+unsigned align_start(unsigned next) { return (next + 7u) & ~7u; }
+
 // One launch of the group kernel over the first n members of g (their start[] and kinds filled; the rest marked
 // unused here).
 int launch_group_args(ConvGroupArgs& g, int n, int kw, int k_order, unsigned grid, unsigned dyn_lds, void* stream) {
@@ -1069,6 +1077,7 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         for (size_t k = done; k < i; ++k) {  // the convs of every item first ...
             const PackItem& it = list.items[k];
             for (int c = 0; c < it.n; ++c) {
+                grid = align_start(grid);
                 g.m[n].conv = it.args[c];
                 g.start[n] = grid;
                 grid += it.grids[c];
@@ -1126,6 +1135,7 @@ int seq_launch_position(const std::vector<Sequence>& seqs, size_t first, int n, 
     for (int i = 0; i < n; ++i) {
         const SeqRecord& r = seqs[first + (size_t)i].recs[k];
         const unsigned wgs = units_to_grid(r);
+        if (r.kind == kMemberConv) grid = align_start(grid);
         g.m[i] = r.m;
         if (r.kind == kMemberConv) g.m[i].conv.hook_blocks = wgs;
         else if (r.kind == kMemberPool) g.m[i].pool.hook_blocks = wgs;
@@ -1327,14 +1337,18 @@ extern "C" int paella_conv2d_launch_group(const paella_conv_operands* members, i
     for (int i = 0; i < n; ++i) {
         const paella_conv_operands& m = members[i];
         if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, args[i])) return rc;
-        g.m[i].conv = args[i];
-        g.start[i] = next;
-        next += m.plan->dims.grid;
         dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
     if (pack_hold(plans, args, n, stream)) return 0;
+    for (int i = 0; i < n; ++i) {
+        next = align_start(next);
+        g.m[i].conv = args[i];
+        g.m[i].conv.hook_blocks = dims.grid;  // the launch is longer than the workgroups that report: ids skipped by align_start
+        g.start[i] = next;
+        next += plans[i]->dims.grid;
+    }
     g.kinds = 0;
-    return launch_group_args(g, n, plans[0]->kw, plans[0]->k_order, dims.grid, dyn_lds, stream);
+    return launch_group_args(g, n, plans[0]->kw, plans[0]->k_order, next, dyn_lds, stream);
 }
 
 extern "C" int paella_conv2d_group_pool_dims(const paella_conv_plan* const* plans, int n, const paella_pool_desc* pool, paella_launch_dims* dims) {
@@ -1378,18 +1392,26 @@ extern "C" int paella_conv2d_launch_group_pool(const paella_conv_operands* membe
     for (int i = 0; i < n; ++i) {
         const paella_conv_operands& m = members[i];
         if (int rc = fill_args(m.plan, m.x, m.blob_dev, m.bias, m.residual, m.slope, m.y, m.workspace, job_id, nf, args[i])) return rc;
-        g.m[i].conv = args[i];
-        g.start[i] = next;
         next += m.plan->dims.grid;
         dyn_lds = std::max(dyn_lds, m.plan->dims.lds_bytes);
     }
     paella::PoolArgs pa;
     if (!paella::pool_fill_args(pool, pool_x, pool_y, job_id, notifier, &pa)) return PAELLA_EINVAL;
-    if (pack_hold(plans, args, n, stream, &pa, dims.grid - next)) return 0;
+    const unsigned pool_grid = dims.grid - next;
+    if (pack_hold(plans, args, n, stream, &pa, pool_grid)) return 0;
+    next = 0;
+    for (int i = 0; i < n; ++i) {
+        next = align_start(next);
+        g.m[i].conv = args[i];
+        g.m[i].conv.hook_blocks = dims.grid;  // the launch is longer than the workgroups that report: ids skipped by align_start
+        g.start[i] = next;
+        next += plans[i]->dims.grid;
+    }
+    pa.hook_blocks = dims.grid;
     g.m[n].pool = pa;
     g.start[n] = next;
     g.kinds = kMemberPool << (2 * n);
-    return launch_group_args(g, n + 1, plans[0]->kw, 1, dims.grid, dyn_lds, stream);
+    return launch_group_args(g, n + 1, plans[0]->kw, 1, next + pool_grid, dyn_lds, stream);
 }
 
 extern "C" int paella_conv2d_pair_dims(const paella_conv_plan* first, const paella_conv_plan* second, paella_launch_dims* dims) {
@@ -1558,6 +1580,7 @@ int pre_send_all(bool only_full) {
             } else {
                 ConvPreGroupArgs g;
                 for (int i = 0; i < n; ++i) {
+                    grid = align_start(grid);
                     g.m[i] = list[done + (size_t)i].a;
                     g.start[i] = grid;
                     grid += list[done + (size_t)i].grid;
