@@ -54,6 +54,8 @@ class Scheduler {
     }
     virtual void try_handle_block_start_finish() = 0;
     virtual void handle_new_job(std::unique_ptr<job::Job> job) = 0;
+    // No job is in flight: every job handed over has had its last stage's completion handled.
+    virtual bool idle() const { return true; }
 
   protected:
     Server* server_ = nullptr;
@@ -80,6 +82,7 @@ class SchedulerFactory {
 class StreamPoolScheduler : public Scheduler {
   public:
     void try_handle_block_start_finish() final;
+    bool idle() const final { return num_jobs_ == 0; }
 
   protected:
     StreamPoolScheduler(const SchedulerOptions& options, size_t mem2sched_bytes);

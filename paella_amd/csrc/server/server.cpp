@@ -64,7 +64,16 @@ void Server::handle_c2s() {
         case MsgType::GROW_POOL: handle_grow_pool(); break;
         case MsgType::CUDA_PROFILER_START: LLIS_WARN_HIP(llis_hip_profiler_start()); break;
         case MsgType::CUDA_PROFILER_STOP: LLIS_WARN_HIP(llis_hip_profiler_stop()); break;
-        case MsgType::PROFILER_CMD: profiler_.handle_cmd(); break;
+        case MsgType::PROFILER_CMD:
+            // A recording covers whole jobs.  A job whose client was woken when its last stage was dispatched (pre-notify) may
+            // still have that kernel running when the client's next message arrives: the switch, and the requests behind it in
+            // the ring, wait until nothing is in flight (the reference applies the switch at once).
+            while (!scheduler_->idle() && !stop_.load(std::memory_order_acquire)) {
+                scheduler_->try_handle_block_start_finish();
+                job::Context::run_poll_hooks();
+            }
+            profiler_.handle_cmd();
+            break;
         case MsgType::EXIT_CMD: request_stop(); break;
         default: throw std::runtime_error("corrupt request ring: unknown message type " + std::to_string((unsigned)type));
     }

@@ -207,6 +207,10 @@ def test_per_workgroup_timing_reaches_the_profiler(cuda, tmp_path):
     assert sum(d > 100 for d in dur) >= 5 and sum(d < 50 for d in dur) >= 5
     kinfo = [l.split() for l in open(prof + "_kernel_info.txt")]
     assert len(pairs) == sum(int(k[2]) for k in kinfo)  # one sample pair per workgroup of every recorded kernel
+    # ... and the recording covers whole jobs: the server applies the switches when nothing is in flight, so neither the last
+    # kernel of a warm-up run (its client is woken at dispatch) leaks in nor the last kernels of the measured requests drop out:
+    # three dummy_short requests of ten kernels and three small-CNN requests (one stage each) in this seed's draw
+    assert sorted(int(k[2]) for k in kinfo) == [3] * 3 + [5] * 30
 
 
 def test_mixed_model_load_then_outputs_still_correct(cuda):

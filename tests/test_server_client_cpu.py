@@ -68,9 +68,14 @@ def test_profiler_files_have_the_reference_line_formats(tmp_path):
     assert run_next and all(len(l) == 4 and abs(float(l[1]) - float(l[0]) - float(l[2])) < 1e-2 for l in run_next)
     jobs = [l.split() for l in open(prof + "_job_events.txt")]
     assert len(jobs) == 60
+    kernels_finished = 0
     for l in jobs:  # pairs "event time"; a job starts with JOB_SUBMITTED (0) and ends with JOB_FINISHED (6), times non-decreasing
         ev, t = [int(x) for x in l[0::2]], [float(x) for x in l[1::2]]
         assert ev[0] == 0 and ev[-1] == 6 and t == sorted(t)
+        kernels_finished += ev.count(5)
+    # the switches are applied when nothing is in flight, so the recordings cover the same whole jobs: one kernel-info line per
+    # KERNEL_FINISHED event (a job that wakes its client when its last stage is dispatched is still recorded to its end)
+    assert kernels_finished == len(kernel_info)
     res = [l.split() for l in open(prof + "_resource_events.txt")]
     assert res and all(len(l) == 8 and l[2] in ("0", "1", "2") for l in res)
     acquired = sum(int(l[4]) for l in res if l[2] == "0")
