@@ -29,6 +29,13 @@ class Context {
 
     static void set_mem2sched_channel(ipc::ShmChannelCpuReader* channel) { mem2sched_channel_ = channel->fork(); }
     static ipc::ShmChannelCpuWriter* get_mem2sched_channel() { return &mem2sched_channel_; }
+    // Tells the scheduler that the job's copy stage is over (what its own marker or host callback would have told it); for
+    // stages declared with Job::set_completes_itself().  Callable from any thread.  Not in the reference.
+    static void post_mem_completion(Job* job) {
+        mem2sched_channel_.acquire_writer_lock();
+        mem2sched_channel_.write(job);
+        mem2sched_channel_.release_writer_lock();
+    }
 
     // True when the active scheduler issues a job's next stage only after the previous one has been reported
     // finished (fifo2, full3); false when it issues all stages at once and relies on stream order (fifo).

@@ -67,6 +67,7 @@ class Job {
         has_started_ = false;
         is_mem_ = false;
         is_pre_notify_ = false;
+        completes_itself_ = false;
         is_unfit_ = false;
         deficit_counter_ = 0;
         cur_stage_ = -1;
@@ -102,6 +103,14 @@ class Job {
     bool is_pre_notify() const { return is_pre_notify_; }
     void set_pre_notify() { is_pre_notify_ = true; }
     void unset_pre_notify() { is_pre_notify_ = false; }
+
+    // A copy stage that reports its own completion: the job does the stage's work off the serving thread (a host-side copy
+    // handed to a helper thread, say) and calls Context::post_mem_completion(this) when it is done, from any thread; the
+    // scheduler then posts no completion marker behind the stage.  Only under a scheduler that issues stage by stage
+    // (Context::is_stage_by_stage()).  Not in the reference, whose copy stages are all stream operations.
+    bool completes_itself() const { return completes_itself_; }
+    void set_completes_itself() { completes_itself_ = true; }
+    void unset_completes_itself() { completes_itself_ = false; }
 
     // ---- snapshot of the stage that is currently on the GPU
     unsigned get_cur_num_blocks() const { return cur_.num_blocks; }
@@ -203,6 +212,7 @@ class Job {
     StageNeeds cur_;
     bool is_mem_ = false;
     bool is_pre_notify_ = false;
+    bool completes_itself_ = false;
     bool is_running_ = false;
     bool has_started_ = false;
     bool is_unfit_ = false;

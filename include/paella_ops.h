@@ -292,6 +292,19 @@ int paella_direct_queue_shared(void** queue);
 int paella_direct_queue_destroy(void* queue);
 
 /*
+ * Copies `bytes` from src to dst (host memory both) on a helper thread of this library and then calls done(arg) on that
+ * thread; returns at once.  For a job's copy of a request's input into its pinned staging buffer (the reference copies
+ * straight from the client's pinned pool, reference jobs/tvm_mnist/tvm_mnist.cpp:38; here that pool cannot be pinned, so there
+ * is a host-side copy, and on the serving thread it would stop the notification ring from being read for its duration).
+ * The helper makes no GPU runtime call.  Copies are done in submission order; done() must be cheap and must not block.
+ * Returns PAELLA_EBUSY, with nothing copied and done() not called, when the helper is asleep (it sleeps after half a
+ * millisecond without a copy): the caller then copies by itself -- at such rates it has the time, and a wake-up through
+ * the kernel would cost a lone request more than the hand-over saves -- and the helper is awake for the copies that follow.
+ */
+#define PAELLA_EBUSY (-5)  /* not taken now; do it yourself or try again */
+int paella_host_copy_submit(void* dst, const void* src, size_t bytes, void (*done)(void*), void* arg);
+
+/*
  * Measurement aid.  While a pair of events (llis_hip_event_create) is armed on the calling thread, every
  * operator launch made by that thread stamps them with the kernel's own begin and end time on the device, so
  * llis_hip_event_elapsed_ms(start, stop) after a stream synchronize is that launch's execution time, the same

@@ -115,6 +115,7 @@ OPS_SYMBOLS = {
     "paella_conv_kernel_occupancy": (c_int, [c_int] * 6 + [c_uint, ctypes.POINTER(c_int), ctypes.POINTER(c_uint), ctypes.POINTER(c_uint)]),
     "paella_kernel_static_lds": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv2d_dims": (c_int, [ctypes.POINTER(ConvPlan), ctypes.POINTER(LaunchDims)]),
+    "paella_host_copy_submit": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "paella_ops_time_launches": (c_int, [c_void_p, c_void_p]),
     "paella_direct_queue_create": (c_int, [ctypes.POINTER(c_void_p)]),
     "paella_direct_queue_set_ordered": (c_int, [c_void_p, c_int]),

@@ -17,7 +17,8 @@
 //    CNN (5 kernels of at most 25 workgroups) each trip through the scheduler costs more than the kernel;
 //  * request buffers in the client's shared-memory pool cannot be registered with the runtime on this
 //    platform, so both copies go through a per-instance pinned staging buffer (filled on the server
-//    thread just before the H2D copy is issued, drained in on_complete()).
+//    thread just before the H2D copy is issued -- or, under a stage-by-stage scheduler, by a helper thread as a copy stage
+//    of its own -- and drained in on_complete()).
 
 #include <llis/job/context.h>
 #include <llis/job/coroutine_job.h>
@@ -108,6 +109,10 @@ class ModelJob : public llis::job::CoroutineJob {
         const char* pack = std::getenv("PAELLA_PACK");
         pack_ = direct_ && !(pack && std::strcmp(pack, "0") == 0);
         if (pack_) llis::job::Context::add_poll_hook(&paella_pack_poll_hook);  // one address for every adapter library: registered once
+        // The staging copy of an input too large for zero-copy leaves the serving thread unless PAELLA_STAGE_THREAD=0; only
+        // under a scheduler that waits for a stage's completion before it issues the next one.
+        const char* st = std::getenv("PAELLA_STAGE_THREAD");
+        stage_off_thread_ = llis::job::Context::is_stage_by_stage() && !(st && std::strcmp(st, "0") == 0);
     }
 
     void body(void* io_ptr) override {
@@ -116,8 +121,24 @@ class ModelJob : public llis::job::CoroutineJob {
             // no stage of its own: staged just before the first kernel is issued, below
         } else if (!input_resident_) {
             set_is_mem();
-            yield();
-            std::memcpy(staging_, io_ptr, in_bytes_);
+            if (stage_off_thread_) {
+                // The host-side copy into the staging buffer is a copy stage of its own, done by the operator library's helper
+                // thread, which reports it to the scheduler like a finished copy: the serving thread keeps reading its rings.
+                set_completes_itself();
+                yield();
+                const int rc = paella_host_copy_submit(staging_, io_ptr, in_bytes_, &ModelJob::staged, static_cast<llis::job::Job*>(this));
+                if (rc == PAELLA_EBUSY) {  // the helper sleeps: a quiet moment, the copy is done here
+                    std::memcpy(staging_, io_ptr, in_bytes_);
+                    staged(static_cast<llis::job::Job*>(this));
+                } else {
+                    check(rc, "staging copy");
+                }
+                unset_completes_itself();
+                yield();
+            } else {
+                yield();
+                std::memcpy(staging_, io_ptr, in_bytes_);
+            }
             check(llis_hip_memcpy_async(paella_exec_input(exec_), staging_, in_bytes_, LLIS_HIP_H2D, stream()), "H2D");
             unset_is_mem();
         } else if (!input_uploaded_) {
@@ -172,6 +193,8 @@ class ModelJob : public llis::job::CoroutineJob {
   private:
     void* stream() { return reinterpret_cast<void*>(get_cuda_stream()); }
 
+    static void staged(void* job) { llis::job::Context::post_mem_completion(static_cast<llis::job::Job*>(job)); }
+
     // Packing is a property of the launching thread (the serving thread, which also runs pack_poll from its loop).
     static void enable_packing_on_this_thread() {
         static thread_local bool on = false;
@@ -198,6 +221,7 @@ class ModelJob : public llis::job::CoroutineJob {
     std::vector<int> group_end_;   // per kernel: index of the last kernel of the group it is issued with
     bool direct_ = true;
     bool pack_ = false;
+    bool stage_off_thread_ = false;
     bool timed_ = false;
     bool unfit_starts_ = false;
     bool input_resident_ = false, input_uploaded_ = false;

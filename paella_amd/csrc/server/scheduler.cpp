@@ -138,10 +138,7 @@ void StreamPoolScheduler::post_mem_completion(job::Job* job) {
 
 void StreamPoolScheduler::mem_notification_callback(void* job) {
     // Runs on a runtime thread; several streams may complete at once, so serialise whole messages.
-    ipc::ShmChannelCpuWriter* channel = job::Context::get_mem2sched_channel();
-    channel->acquire_writer_lock();
-    channel->write(job);
-    channel->release_writer_lock();
+    job::Context::post_mem_completion(static_cast<job::Job*>(job));
 }
 
 void StreamPoolScheduler::spin_sleep() const {

@@ -58,6 +58,7 @@ void SchedulerFifo2::schedule_job() {
         const unsigned stream = take_stream();
         job->set_running(stream_handle(stream));
         const bool is_mem = job->is_mem();
+        const bool posts_itself = is_mem && job->completes_itself();  // read before run_next declares the stage after
         long long notifier = -1;
         if (!is_mem) {
             notifier = take_notifier();
@@ -77,7 +78,7 @@ void SchedulerFifo2::schedule_job() {
         } else {
             job->run_next();
         }
-        if (is_mem) post_mem_completion(job);
+        if (is_mem && !posts_itself) post_mem_completion(job);
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);
     }
 }

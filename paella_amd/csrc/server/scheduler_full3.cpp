@@ -176,6 +176,7 @@ void SchedulerFull3::schedule_job() {
         spin_sleep();
 
         const bool is_mem = job->is_mem();
+        const bool posts_itself = is_mem && job->completes_itself();  // read before run_next declares the stage after
         bool unfit = false;
         if (!is_mem && !gpu_resources_.job_fits(job)) {
             if (num_outstanding_kernels_ >= (int)options_.extra_kernels) {
@@ -214,7 +215,7 @@ void SchedulerFull3::schedule_job() {
             } else {
                 job->run_next();
             }
-            if (is_mem) post_mem_completion(job);
+            if (is_mem && !posts_itself) post_mem_completion(job);
         }
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);
     }

@@ -4,13 +4,19 @@
 //   FAKE_VARIANT 1  fake_long  : 50 kernels of 5 x 256                                   (shape of dummy_long)
 //   FAKE_VARIANT 2  fake_mem3  : copy, kernels of 40 / 200 / 17 workgroups with distinct footprints, copy(pre-notify)
 //   FAKE_VARIANT 3  fake_big   : 3 kernels of 3000 x 256 x 64 regs -- never fits beside anything (over-subscription path)
+//   FAKE_VARIANT 4  fake_self  : a copy stage that reports its own completion (from a thread of its own after 300 us when
+//                                FAKE_SELF_THREAD=1, else before it returns), copy, kernel of 40, copy(pre-notify); output = input + 1
 
 #include <llis/job/context.h>
 #include <llis/job/coroutine_job.h>
 
 #include "paella_hip.h"
 
+#include <cstdlib>
 #include <cstring>
+#include <thread>
+
+#include <unistd.h>
 
 extern "C" int fake_hip_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks);
 
@@ -22,8 +28,8 @@ namespace {
 
 class FakeJob : public llis::job::CoroutineJob {
   public:
-    size_t get_input_size() override { return FAKE_VARIANT == 2 ? 100 : 5; }
-    size_t get_output_size() override { return FAKE_VARIANT == 2 ? 100 : 11; }
+    size_t get_input_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 ? 100 : 5; }
+    size_t get_output_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 ? 100 : 11; }
     size_t get_param_size() override { return 4; }
 
     void one_time_init() override {}
@@ -55,6 +61,34 @@ class FakeJob : public llis::job::CoroutineJob {
         set_pre_notify();
         yield();
         llis_hip_memcpy_async(reinterpret_cast<char*>(io_ptr) + 100, buf_, 100, LLIS_HIP_D2H, reinterpret_cast<void*>(get_cuda_stream()));
+#elif FAKE_VARIANT == 4
+        set_is_mem();
+        set_completes_itself();
+        yield();
+        {
+            const char* threaded = std::getenv("FAKE_SELF_THREAD");
+            llis::job::Job* self = this;
+            char* stage = stage_;
+            if (threaded && threaded[0] == '1') {
+                std::thread([self, stage, io_ptr] {
+                    usleep(300);
+                    std::memcpy(stage, io_ptr, 100);
+                    llis::job::Context::post_mem_completion(self);
+                }).detach();
+            } else {
+                std::memcpy(stage, io_ptr, 100);
+                llis::job::Context::post_mem_completion(self);
+            }
+        }
+        unset_completes_itself();
+        yield();
+        llis_hip_memcpy_async(buf_, stage_, 100, LLIS_HIP_H2D, reinterpret_cast<void*>(get_cuda_stream()));
+        kernel(40, 128, 1024, 64, false);
+        for (int i = 0; i < 100; ++i) buf_[i] = (char)(buf_[i] + 1);
+        set_is_mem();
+        set_pre_notify();
+        yield();
+        llis_hip_memcpy_async(reinterpret_cast<char*>(io_ptr) + 100, buf_, 100, LLIS_HIP_D2H, reinterpret_cast<void*>(get_cuda_stream()));
 #else
         for (int i = 0; i < 3; ++i) kernel(3000, 256, 0, 64, i == 2);
 #endif
@@ -63,6 +97,7 @@ class FakeJob : public llis::job::CoroutineJob {
 
   private:
     char buf_[100];
+    char stage_[100];
 };
 
 }  // namespace

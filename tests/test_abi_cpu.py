@@ -142,3 +142,46 @@ def test_reference_client_programs_compile_against_these_headers(source):
         pytest.skip(source + " is not in this copy of the reference")
     out = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I" + os.path.join(ROOT, "include"), path], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr[-3000:]
+
+
+def test_host_copy_helper_copies_in_order_and_declines_while_asleep():
+    """paella_host_copy_submit: copies land before done() runs, in submission order; after half a millisecond without work the
+    helper sleeps and the next call is declined (PAELLA_EBUSY, nothing copied, the caller copies by itself) but wakes it."""
+    import threading
+    import time
+    from paella_amd import _abi
+    lib = _abi.ops()
+    done_t = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+    order, lock = [], threading.Lock()
+
+    @done_t
+    def done(arg):
+        with lock:
+            order.append(arg)
+
+    def submit_until_taken(dst, src, tag):
+        for _ in range(2000):  # a declined call wakes the helper; it is up within microseconds
+            rc = lib.paella_host_copy_submit(dst.ctypes.data, src.ctypes.data, src.nbytes, done, tag)
+            if rc == 0:
+                return
+            assert rc == -5
+            time.sleep(0.0001)
+        raise AssertionError("the helper never woke up")
+
+    rng = np.random.default_rng(5)
+    srcs = [rng.integers(0, 255, 300000 + 7 * i, dtype=np.uint8) for i in range(6)]
+    dsts = [np.zeros_like(s) for s in srcs]
+    submit_until_taken(dsts[0], srcs[0], 1)
+    for i in range(1, 6):  # right behind: the helper is awake
+        assert lib.paella_host_copy_submit(dsts[i].ctypes.data, srcs[i].ctypes.data, srcs[i].nbytes, done, i + 1) == 0
+    deadline = time.time() + 10
+    while len(order) < 6 and time.time() < deadline:
+        time.sleep(0.001)
+    assert order == [1, 2, 3, 4, 5, 6]
+    assert all(np.array_equal(d, s) for d, s in zip(dsts, srcs))
+    time.sleep(0.05)  # a hundred times the helper's spin: asleep now
+    late = np.zeros_like(srcs[0])
+    assert lib.paella_host_copy_submit(late.ctypes.data, srcs[0].ctypes.data, srcs[0].nbytes, done, 7) == -5
+    time.sleep(0.01)
+    assert not late.any() and order == [1, 2, 3, 4, 5, 6]  # declined means untouched
+    assert lib.paella_host_copy_submit(None, srcs[0].ctypes.data, 1, done, 0) == -1

@@ -54,6 +54,21 @@ def test_request_bytes_travel_through_the_pool_slots():
     assert sorted(r for r in replies if r.startswith("done")) == ["done 1000", "done 1003"]
 
 
+@pytest.mark.parametrize("policy", ["fifo2", "full3"])
+def test_a_copy_stage_that_reports_its_own_completion(policy):
+    """fake_self: its first copy stage posts its completion itself (Job::set_completes_itself, Context::post_mem_completion):
+    the scheduler launches no marker behind it -- the device sees only the two real copies and the kernel -- and goes on to the
+    next stage when the message arrives; the bytes staged in that stage come back as input + 1."""
+    replies, log = run_harness(scenario(policy, 2, "put 4 0 9\nput 4 1 30\nlaunch 4 0\nlaunch 4 1\ndrain\nget 4 0\nget 4 1\n", types=TYPES + ["fake_self"]))
+    assert [r for r in replies if r.startswith("out")] == ["out 10 10 10 10 10 10 10 10", "out 31 31 31 31 31 31 31 31"]
+    assert sorted(r for r in replies if r.startswith("done")) == ["done 5000", "done 5001"]
+    events = sched.parse_log(log)
+    for job in (0, 1):
+        mine = [e for e in events if e[0] in ("D", "M") and e[1] == job]
+        # dispatch of the self-reporting stage, its completion, the host-to-device copy, its completion, the kernel, the last copy
+        assert [e[0] for e in mine[:5]] == ["D", "M", "D", "M", "D"] and [e[5] for e in mine if e[0] == "D"] == [1, 1, 0, 1]
+
+
 def test_oversubscription_credit_path():
     """fake_big (3000 x 256 x 64 regs) never fits a small budget: it is admitted as an 'unfit' kernel while
     credits last, the credit returns when its start messages are complete (or at its end), and the

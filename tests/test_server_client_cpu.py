@@ -145,6 +145,20 @@ def test_single_latency_client(tmp_path):
     assert srv.wait(timeout=30) == 0
 
 
+@pytest.mark.parametrize("sched_name", ["fifo2", "full3"])
+def test_a_copy_stage_completed_from_another_thread(sched_name):
+    """fake_self with FAKE_SELF_THREAD=1: the first copy stage is finished by a thread of the job's own, 300 us later, through
+    Context::post_mem_completion; the server binaries serve fifty such requests."""
+    name = "ptself%d%s" % (os.getpid(), sched_name)
+    srv = start_server(name, sched_name, 4, FAKE_SELF_THREAD="1")
+    out = subprocess.run([os.path.join(BIN, "llis_app_single_latency"), name, fake_job("fake_self"), "50", "--quiet"], env=fake_env(),
+                         capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    stats = json.loads(out.stdout.strip().splitlines()[-1])
+    assert stats["num_jobs"] == 50 and stats["min_us"] >= 300  # every request waited for its thread
+    assert srv.wait(timeout=30) == 0
+
+
 def test_in_process_serve_abi_on_the_scripted_device():
     """paella_server_start / paella_client_run / paella_client_single in a child interpreter that loads the
     scripted device first (same soname as the HIP layer)."""
