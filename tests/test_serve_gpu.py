@@ -73,6 +73,36 @@ def test_resident_input_mode_and_both_dispatch_paths_match_oracle(cuda, dispatch
     close(out, ref)
 
 
+@pytest.mark.parametrize("sched_name,helper", [("full3", "0"), ("full3", "1"), ("fifo2", "1"), ("fifo", "1")])
+def test_input_staging_on_and_off_the_serving_thread(cuda, sched_name, helper):
+    """The host-side copy of a request's input into the pinned staging buffer: on the serving thread (PAELLA_STAGE_THREAD=0,
+    and always under fifo, which issues every stage at once) or as a copy stage of its own that the operator library's helper
+    thread finishes and reports.  Requests in a burst (the helper is awake) and one at a time (it sleeps in between and the
+    adapter copies by itself) must both give the oracle's result for their own input."""
+    import time
+    from paella_amd import models, serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    desc = models.describe("resnet18")
+    xs = [om.make_input(desc, 40 + i, "normal") for i in range(2)]
+    refs = [om.run(desc, x, seed=1) for x in xs]
+    old = os.environ.get("PAELLA_STAGE_THREAD")
+    os.environ["PAELLA_STAGE_THREAD"] = helper
+    try:
+        with serve.Server(server_name("stage" + helper), sched_name, num_streams=8) as srv:
+            burst, _ = serve.client_single(srv.name, serve.job_path("tvm_resnet18"), xs[0], refs[0].size, n=6)
+            time.sleep(0.01)  # the helper has gone to sleep
+            lone, _ = serve.client_single(srv.name, serve.job_path("tvm_resnet18"), xs[1], refs[1].size, n=1)
+            load = serve.client_run(srv.name, [(serve.job_path("tvm_resnet18"), 1.0, 8)], 0.0, 8, 64)
+    finally:
+        if old is None:
+            os.environ.pop("PAELLA_STAGE_THREAD", None)
+        else:
+            os.environ["PAELLA_STAGE_THREAD"] = old
+    close(burst, refs[0])
+    close(lone, refs[1])
+    assert load["all"]["count"] == 64
+
+
 @pytest.mark.parametrize("mem_marker", [True, False])
 def test_both_copy_completion_paths_on_the_gpu(cuda, mem_marker):
     from paella_amd import serve
