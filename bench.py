@@ -117,6 +117,74 @@ def conv_roofline(models, hip, model, reps, back_to_back=200):
             "by_op": by_op, "direct_rps": direct_rps, "forward_us": sum(per_stage)}
 
 
+def full_device_pass(models, hip, model, images=16, reps=10, timed=True):
+    """The conv kernel with the device full: every distinct conv layer of the model (groups == 1) over `images` inputs stacked
+    along the height, i.e. with `images` times the pixel tiles -- what the compute units see on the serving path, where packed
+    launches on four queues keep 16 to 24 problems in flight -- on the 32 x 32 tile with the layer's own waves per workgroup and
+    no split of the reduction over workgroups, one launch at a time on a HIP stream.  timed: durations from the kernel's own
+    begin and end stamps; otherwise one launch per layer with a synchronize after each (for counter collection)."""
+    import numpy as np
+    import torch
+    from paella_amd import ops
+    desc = models.describe(model)
+    lib = models._abi.ops()
+    stream = ctypes.c_void_p()
+    hip.llis_hip_stream_create(ctypes.byref(stream))
+    ev = []
+    for _ in range(2):
+        e = ctypes.c_void_p()
+        hip.llis_hip_event_create(ctypes.byref(e))
+        ev.append(e)
+    rng = np.random.default_rng(1)
+    seen, rows = {}, []
+    for node in desc["nodes"]:
+        if node["op"] != "conv" or node["groups"] != 1:
+            continue
+        x = node["x"]
+        key = (x["C"], x["H"], x["W"], node["K"], node["R"], node["S"], tuple(node["stride"]), tuple(node["pad"]))
+        if key in seen:
+            rows[seen[key]]["count"] += 1
+            continue
+        c, h, w, k, r, q = x["C"], x["H"], x["W"], node["K"], node["R"], node["S"]
+        wt = (rng.standard_normal((k, c, r, q)) / np.sqrt(c * r * q)).astype(np.float32)
+        alone = ops.Conv2d(wt, None, stride=tuple(node["stride"]), pad=tuple(node["pad"]), dil=tuple(node["dil"]), act=ops.ACT_RELU, in_hw=(h, w))
+        hint = (1 << 8) | (1 << 4) | (alone.plan.kw.bit_length() - 1)
+        conv = ops.Conv2d(wt, np.zeros(k, np.float32), stride=tuple(node["stride"]), pad=tuple(node["pad"]), dil=tuple(node["dil"]), act=ops.ACT_RELU,
+                          in_hw=(h * images, w), tile_hint=hint)
+        xin = torch.randn((1, c, h * images, w), device="cuda:0")
+        y = torch.empty((1, k, conv.plan.P, conv.plan.Q), device="cuda:0")
+        torch.cuda.synchronize()  # the operands are written on torch's stream, the launches go to another
+        conv(xin, out=y, stream=stream.value)
+        hip.llis_hip_stream_synchronize(stream)
+        us = None
+        if timed:
+            lib.paella_ops_time_launches(ev[0], ev[1])
+            total = 0.0
+            for _ in range(reps):
+                conv(xin, out=y, stream=stream.value)
+                hip.llis_hip_stream_synchronize(stream)
+                ms = ctypes.c_float()
+                hip.llis_hip_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms))
+                total += ms.value
+            lib.paella_ops_time_launches(None, None)
+            us = total / reps * 1e3
+        seen[key] = len(rows)
+        rows.append({"layer": "%dx%d %d->%d %dx%d s%d" % (h, w, c, k, r, q, node["stride"][0]), "count": 1, "workgroups": conv.plan.dims.grid,
+                     "waves_per_workgroup": conv.plan.kw, "k_order": conv.plan.k_order, "flops": conv.plan.flops, "us": us})
+    for e in ev:
+        hip.llis_hip_event_destroy(e)
+    hip.llis_hip_stream_destroy(stream)
+    out = {"model": model, "images": images, "layers": rows}
+    if timed:
+        # weighted by how often a layer shape occurs in one forward pass
+        flops = sum(r["flops"] * r["count"] for r in rows)
+        us = sum(r["us"] * r["count"] for r in rows)
+        out.update({"achieved": flops / us / 1e6, "frac": flops / us / 1e6 / FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "how": "every conv layer of %s over %d inputs stacked along the height (%d times the pixel tiles), 32 x 32 tile, one launch at a time; "
+                           "layers weighted by their count in a forward pass" % (model, images, images)})
+    return out
+
+
 def multi_queue_rate(models, model, nq=4, reps=200):
     """Forward passes per second with nq requests in flight and no scheduler in between: nq executors, each on its own
     ordered direct-dispatch queue, kernels without hooks.  The GPU-side ceiling of the served path.  Four queues is
@@ -360,6 +428,9 @@ def main():
                     help="only: how many kernels run side by side and what sharing a launch gains (paella_queue_concurrency_probe), as a table on stderr")
     ap.add_argument("--roofline-only", default=None, metavar="MODEL",
                     help="only the isolated per-launch timing of one forward pass of MODEL (the leg roofline.achieved comes from)")
+    ap.add_argument("--full-device", default=None, metavar="MODEL",
+                    help="only: the conv kernel with the device full (every conv layer of MODEL over 16 stacked inputs, one launch at a time); "
+                         "under counter collection one untimed launch per layer")
     ap.add_argument("--counter-pass", default=None, metavar="MODEL",
                     help="only this: three forward passes of MODEL, one launch at a time with a synchronize after each (the leg to run "
                          "under `rocprofv3 --pmc`: nothing else is in flight and at most one dispatch is ever queued)")
@@ -382,6 +453,13 @@ def main():
             _abi.check(_abi.ops().paella_copy_launch(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(y.data_ptr()), n, None, 0, None), "copy")
             torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"launches": 5, "kib_read_per_launch": n * 4 / 1024, "kib_written_per_launch": n * 4 / 1024}}), flush=True)
+        return
+    if args.full_device:
+        fd = full_device_pass(models, hip, args.full_device, timed=not under_counter_collection())
+        for r in fd["layers"]:
+            log("[bench] %-26s x%d  %5d workgroups x %d waves  %8.1f MFLOP  %s" % (r["layer"], r["count"], r["workgroups"], r["waves_per_workgroup"], r["flops"] / 1e6,
+                "%7.2f us  %6.1f TFLOP/s" % (r["us"], r["flops"] / r["us"] / 1e6) if r["us"] else ""))
+        print(json.dumps({"full_device": fd}), flush=True)
         return
     if args.counter_pass:
         ex = models.Exec(args.counter_pass, seed=1)
@@ -603,6 +681,9 @@ def main():
 
     # ---- kernel-level figures
     lib = _abi.ops()
+    fd = full_device_pass(models, hip, "inception_v3")
+    roofline["full_device"] = {k: fd[k] for k in ("achieved", "frac", "unit", "how")}
+    log("[bench] conv kernel with the device full (Inception-v3's layers over 16 stacked inputs): %.1f TFLOP/s = %.1f%% of peak" % (fd["achieved"], 100 * fd["frac"]))
     if not args.no_side:
         try:
             mq = multi_queue_rate(models, "inception_v3", reps=60)
