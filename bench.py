@@ -424,6 +424,8 @@ def main():
     ap.add_argument("--zoo-ops", nargs="?", const="all", default=None, metavar="MODELS",
                     help="only this: per operator family of every zoo model (or of the comma-separated ones), launches, time and rates "
                          "of one forward pass, one launch at a time")
+    ap.add_argument("--overlap-probe", action="store_true",
+                    help="only: whether vector-ALU instructions hide behind matrix instructions on this device (a table on stderr)")
     ap.add_argument("--queue-probe", action="store_true",
                     help="only: how many kernels run side by side and what sharing a launch gains (paella_queue_concurrency_probe), as a table on stderr")
     ap.add_argument("--roofline-only", default=None, metavar="MODEL",
@@ -499,6 +501,18 @@ def main():
                     (op, row["launches"], row["us"], row["us_per_launch"], row["tflops"], 100 * row["frac_of_fp32_mfma_peak"],
                      row["gbytes_per_s"], 100 * row["frac_of_hbm_peak"]))
         print(json.dumps({"zoo_ops": table}), flush=True)
+        return
+    if args.overlap_probe:
+        lib = _abi.ops()
+        out = {}
+        log("[bench] four matrix instructions + N multiply-adds per iteration, eight waves per SIMD, register-resident (paella_mfma_valu_overlap_probe)")
+        log("[bench] %4s %12s %14s %10s" % ("N", "both, us", "vector alone", "TFLOP/s"))
+        for n in (0, 8, 16, 32, 64, 128):
+            both, alone, tf = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+            _abi.check(lib.paella_mfma_valu_overlap_probe(n, ctypes.byref(both), ctypes.byref(alone), ctypes.byref(tf)), "paella_mfma_valu_overlap_probe")
+            out[n] = {"us_both": both.value, "us_valu_alone": alone.value, "tflops": tf.value}
+            log("[bench] %4d %12.1f %14.1f %10.1f" % (n, both.value, alone.value, tf.value))
+        print(json.dumps({"mfma_valu_overlap": out}))
         return
     if args.queue_probe:
         from paella_amd._abi import ConvDesc

@@ -139,6 +139,7 @@ RING_SYMBOLS = {
     "paella_empty_kernel_probe": (c_int, [c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_echo": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "paella_mfma_peak_probe": (c_int, [ctypes.POINTER(c_double)]),
+    "paella_mfma_valu_overlap_probe": (c_int, [c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "paella_queue_concurrency_probe": (c_int, [ctypes.POINTER(ConvDesc), c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_double)]),
 }
 

@@ -83,6 +83,43 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(float* sink, int iters) 
     if (v == 123.456f) sink[0] = v;  // keeps the loop alive without a store in practice
 }
 
+// The same loop with V independent multiply-adds after every four matrix instructions (MFMA = false: the multiply-adds alone):
+// whether vector-ALU work of a SIMD's waves hides behind its matrix instructions or adds to them.
+template <int V, bool MFMA>
+__global__ __launch_bounds__(512) void mfma_valu_kernel(float* sink, int iters) {
+    probe_f32x16 acc = {0};
+    float a = 1.0f + threadIdx.x * 1e-6f, b = 1.0f - threadIdx.x * 1e-6f;
+    float v[8] = {a, b, a + 1.f, b + 1.f, a + 2.f, b + 2.f, a + 3.f, b + 3.f};
+    for (int i = 0; i < iters; ++i) {
+        if (MFMA) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[j & 7] = v[j & 7] * 1.0001f + 0.5f;
+        asm volatile("" ::: "memory");
+    }
+    float r = 0.f;
+    for (int e = 0; e < 16; ++e) r += acc[e];
+    for (int j = 0; j < 8; ++j) r += v[j];
+    if (r == 123.456f) sink[threadIdx.x] = r;
+}
+
+template <int V, bool MFMA>
+double mfma_valu_us(float* sink, int iters, unsigned blocks, hipEvent_t e0, hipEvent_t e1) {
+    float best = 0.f;
+    for (int rep = 0; rep < 3; ++rep) {
+        hipEventRecord(e0, nullptr);
+        hipLaunchKernelGGL((mfma_valu_kernel<V, MFMA>), dim3(blocks), dim3(512), 0, nullptr, sink, iters);
+        hipEventRecord(e1, nullptr);
+        hipEventSynchronize(e1);
+        float ms = 0;
+        hipEventElapsedTime(&ms, e0, e1);
+        if (rep == 0 || ms < best) best = ms;
+    }
+    return best * 1e3;
+}
+
 __global__ void flag_kernel(int* flag) { __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM); }
 
 // One lane answers `total` host pings: waits (bounded by a tick budget, and by a negative value of the flag) until
@@ -362,6 +399,34 @@ int paella_mfma_peak_probe(double* tflops) {
     hipFree(sink);
     *tflops = best;
     return 0;
+}
+
+int paella_mfma_valu_overlap_probe(int valu_per_four_mfma, double* us_both, double* us_valu_alone, double* tflops) {
+    if (!us_both || !us_valu_alone || !tflops) return -1;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, 0);
+    if (e != hipSuccess) return (int)e;
+    float* sink = nullptr;
+    e = hipMalloc(&sink, 4096);
+    if (e != hipSuccess) return (int)e;
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    const int iters = 2000;
+    const unsigned blocks = (unsigned)prop.multiProcessorCount * 4;  // 32 waves per CU: eight per SIMD
+    int rc = 0;
+    switch (valu_per_four_mfma) {
+#define PAELLA_PROBE_CASE(V) \
+    case V: *us_both = mfma_valu_us<V, true>(sink, iters, blocks, e0, e1); *us_valu_alone = mfma_valu_us<V, false>(sink, iters, blocks, e0, e1); break;
+        PAELLA_PROBE_CASE(0) PAELLA_PROBE_CASE(8) PAELLA_PROBE_CASE(16) PAELLA_PROBE_CASE(32) PAELLA_PROBE_CASE(64) PAELLA_PROBE_CASE(128)
+#undef PAELLA_PROBE_CASE
+        default: rc = -1;
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    hipFree(sink);
+    if (rc == 0) *tflops = (double)blocks * 8 /*waves*/ * iters * 4 /*mfma*/ * 4096.0 / (*us_both * 1e-6) / 1e12;
+    return rc;
 }
 
 int paella_queue_concurrency_probe(const paella_conv_desc* desc, int instances, int per_launch, int queues, int ordered, int reps,

@@ -124,3 +124,24 @@ def test_queue_concurrency_probe_runs_and_reports_a_time(cuda):
     four = us.value
     _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 4, 4, 1, 20, ctypes.byref(us)), "probe, four per launch")
     assert 0.1 < four <= one * 1.1 and 0.05 < us.value < one * 1.1, (one, four, us.value)
+
+
+def test_vector_alu_work_adds_to_matrix_instruction_time(cuda):
+    """paella_mfma_valu_overlap_probe: on this device a SIMD's vector-ALU instructions do not hide behind its matrix
+    instructions -- the loop with both takes the matrix loop's time plus the vector loop's time (which is why the conv
+    kernel keeps its per-chunk address arithmetic on the scalar unit)."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+
+    def probe(n):
+        both, alone, tf = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        _abi.check(lib.paella_mfma_valu_overlap_probe(n, ctypes.byref(both), ctypes.byref(alone), ctypes.byref(tf)), "paella_mfma_valu_overlap_probe")
+        return both.value, alone.value, tf.value
+
+    base, _, peak = probe(0)
+    assert 120.0 < peak < 165.0  # the matrix loop alone runs near the fp32 peak
+    for n in (32, 128):
+        both, alone, tf = probe(n)
+        assert alone > 0 and 0.9 * (base + alone) < both < 1.1 * (base + alone), (n, base, alone, both)
+        assert tf < peak
+    assert lib.paella_mfma_valu_overlap_probe(7, None, None, None) == -1
