@@ -79,8 +79,8 @@ class FinishedBlockNotifier {
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            if (measure_block_time_) send_block_time_first();
             announce<true>(&agg_counter_end_, 0, job_id);
-            if (measure_block_time_) send_block_time();
         }
     }
 
@@ -92,8 +92,8 @@ class FinishedBlockNotifier {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
+            if (measure_block_time_) send_block_time_first();
             announce<false>(&agg_counter_end_, 0, job_id);
-            if (measure_block_time_) send_block_time();
         }
     }
 
@@ -106,8 +106,8 @@ class FinishedBlockNotifier {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
+            if (timed && measure_block_time_) send_block_time_first();  // the member is looked at only when timing was asked for
             announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
-            if (timed && measure_block_time_) send_block_time();  // the member is looked at only when timing was asked for
         }
     }
 
@@ -118,8 +118,8 @@ class FinishedBlockNotifier {
         end_from_one_lane(job_id, timed, gridDim.x * gridDim.y * gridDim.z);
     }
     __device__ __forceinline__ void end_from_one_lane(JobId job_id, bool timed, unsigned num_blocks) {
+        if (timed && measure_block_time_) send_block_time_first();
         announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
-        if (timed && measure_block_time_) send_block_time();
     }
 #endif
 
@@ -147,6 +147,14 @@ class FinishedBlockNotifier {
         t.data[1] = (uint16_t)(((s & 0xFFu) << 8) | (e >> 16));
         t.data[2] = (uint16_t)(e & 0xFFFFu);
         block_time_channel_.write_relaxed(t);
+    }
+
+    // The workgroup's time sample goes out ahead of its end message, with a system-scope release between the two: once the
+    // host has seen a kernel's last end message, every sample of that kernel is in the timing ring (a recording that stops
+    // when the server is idle then holds whole kernels).  Only when per-workgroup timing is on.
+    __device__ __forceinline__ void send_block_time_first() {
+        send_block_time();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     }
 
     // ACQUIRE: the sender first acquires (device scope) what the other workgroups released before their bump.

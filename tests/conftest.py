@@ -40,6 +40,9 @@ def _two_process_run():
                     return res
                 time.sleep(0.05)
             prefix = os.path.join(out_dir, "two_process")
+            for suffix in (".txt", "_raw.txt", "_timeline.txt"):  # the client appends, as the reference's does: one session, one row
+                if os.path.exists(prefix + suffix):
+                    os.remove(prefix + suffix)
             cmd = [os.path.join(bin_dir, "llis_app_client"), "--server_name", name, "--iat", "100", "--dist", "exp", "--concurrency", "56",
                    "--num_jobs", "6000", "--start_record_num", "500", "--seed", "1", "--prefix", prefix,
                    os.path.join(lib_dir, "libjob_tvm_mnist.so"), "0.9", "48", os.path.join(lib_dir, "libjob_tvm_inception_v3.so"), "0.1", "8"]
