@@ -47,8 +47,13 @@ KEEP_UP = 0.95            # served rate / offered rate below which a point does 
 MIX = [("small_cnn", "tvm_mnist", "mnist", 0.9, 96), ("inception_v3", "tvm_inception_v3", "inception_v3", 0.1, 16)]
 
 
+SUMMARY = []  # the top-level progress lines, printed once more after the detail dump so that they end the stderr stream
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+    if len(a) == 1 and isinstance(a[0], str) and a[0].startswith("[bench] ") and not a[0].startswith("[bench]  ") and not a[0].startswith("[bench] detail"):
+        SUMMARY.append(a[0])
 
 
 # HBM-side bytes per conv launch (mean over the conv launches of one forward pass), from FETCH_SIZE / WRITE_SIZE
@@ -226,7 +231,7 @@ def cpu_baseline(model, budget_s, max_passes=64):
         if dt >= budget_s or n >= max_passes:
             break
     return {"value": n / dt, "unit": "requests/s", "cores": orc.num_threads(), "kind": "port",
-            "sample": "%d %s forward passes (batch 1, fp32, same graph and seeded weights) with the float-accumulate CPU oracle, %.1f s" % (n, model, dt)}
+            "sample": "%d %s passes in %.1f s" % (n, model, dt)}
 
 
 def torch_cpu_baseline(model, budget_s):
@@ -303,7 +308,7 @@ def torch_cpu_baseline(model, budget_s):
             if dt >= budget_s or n >= 2000:
                 break
     return {"value": n / dt, "unit": "requests/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "%d %s forward passes (batch 1, fp32, same graph and seeded weights) through torch's CPU operators, %.1f s" % (n, model, dt)}
+            "sample": "%d %s passes in %.1f s" % (n, model, dt)}
 
 
 class Arm:
@@ -753,14 +758,14 @@ def main():
         small = cpu_baseline("mnist", 1.0, max_passes=2000)
         per_request_s = 0.9 / small["value"] + 0.1 / big["value"]
         cpu = {"value": 1.0 / per_request_s, "unit": "requests/s", "cores": big["cores"], "kind": "port",
-               "sample": "CPU oracle forward passes, batch 1, fp32, same graphs and seeded weights: %s; %s; combined at 9 : 1 as 1 / (0.9 t_small + 0.1 t_inception)" %
+               "sample": "CPU oracle (float accumulate, OpenMP), same graphs and weights, batch 1: %s; %s; mix rate = 1/(0.9 t_small + 0.1 t_big)" %
                          (big["sample"], small["sample"]),
                "inception_v3_passes_per_s": big["value"], "small_cnn_passes_per_s": small["value"]}
         try:
             tb, ts = torch_cpu_baseline("inception_v3", min(args.cpu_seconds, 8.0)), torch_cpu_baseline("mnist", 1.0)
             if tb and ts:
                 cpu_torch = {"value": 1.0 / (0.9 / ts["value"] + 0.1 / tb["value"]), "unit": "requests/s", "cores": tb["cores"], "kind": "port",
-                             "sample": "the same two graphs through torch's CPU operators (oneDNN), combined the same way: %s; %s" % (tb["sample"], ts["sample"])}
+                             "sample": "torch CPU operators (oneDNN), same graphs and weights: %s; %s; combined the same way" % (tb["sample"], ts["sample"])}
         except Exception as ex:  # torch missing or an operator it lacks: the oracle figure stands alone
             log("[bench]   torch CPU baseline unavailable: %s" % ex)
         log("[bench] CPU: oracle %.2f req/s of the mix on %d threads%s" % (cpu["value"], cpu["cores"], "" if not cpu_torch else ", torch CPU operators %.1f req/s" % cpu_torch["value"]))
@@ -801,7 +806,82 @@ def main():
                           "gbytes_per_s": v["bytes"] / (v["us"] * 1e-6) / 1e9 if v["us"] else None} for k, v in rl["by_op"].items()},
         "notify_us": notify,
     }
-    print(json.dumps(out), flush=True)
+    emit(out)
+
+
+def _short(x, digits=6):
+    """Numbers to `digits` significant figures, recursively: the stdout line is read by a harness that keeps a few KB."""
+    if isinstance(x, bool) or x is None:
+        return x
+    if isinstance(x, float):
+        return float("%.*g" % (digits, x))
+    if isinstance(x, dict):
+        return {k: _short(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_short(v, digits) for v in x]
+    return x
+
+
+def headline(out):
+    """The one stdout line: the contract's keys, the roofline and CPU-baseline objects and a handful of headline figures.  Everything
+    else the run measured (the rate-search points, every arm at equal load, the side workloads, per-operator times) goes to
+    the detail file and to stderr; this line stays under 4 KB whatever the run produced."""
+    cfg, rf = out["config"], out.get("roofline") or {}
+    line = {k: out[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
+    line["config"] = {"workload": "small CNN : Inception-v3 (299x299) = 9 : 1, batch 1, fp32, open-loop Poisson, per-request H2D/D2H, full3 on direct dispatch",
+                      "slo_us": cfg.get("slo_us"), "slo_factor": cfg.get("slo_factor"), "timed_requests": cfg.get("timed_requests"),
+                      "timed_seconds": cfg.get("timed_seconds"), "pools": cfg.get("pools")}
+    for k in ("offered_rps", "slo_met", "latency_us", "verified_requests", "mismatches"):
+        if k in out:
+            line[k] = out[k]
+    r = {k: rf.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic") if k in rf}
+    r["kernel"] = "conv_mfma_kernel (+ grouped forms), Inception-v3's conv launches one at a time"
+    for k in ("flops_per_launch_avg", "us_per_launch_avg", "algorithmic_bytes_per_launch_avg", "peak_measured", "empty_kernel_us"):
+        if k in rf:
+            r[k] = rf[k]
+    for k in ("served", "under_load", "full_device"):
+        if isinstance(rf.get(k), dict):
+            r[k] = {"frac": rf[k].get("frac"), "tflops": rf[k].get("conv_tflops", rf[k].get("achieved"))}
+    line["roofline"] = r
+    for key in ("cpu_baseline", "cpu_baseline_torch"):
+        c = out.get(key)
+        if c:
+            line[key] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"], "kind": c["kind"], "sample": c["sample"][:200]}
+        else:
+            line[key] = None
+    arms = {}
+    for label, s in (out.get("rate_search") or {}).items():
+        arms[label] = {"rate_at_slo_rps": s.get("rate_at_slo_rps"), "saturation_rps": s.get("saturation_rps")}
+    line["arms"] = arms
+    n = out.get("notify_us") or {}
+    line["notify_us"] = {k: ({"p50": v["p50"], "p99": v["p99"]} if isinstance(v, dict) else v) for k, v in n.items()}
+    if out.get("policy"):
+        line["policy"] = out["policy"]
+    line["detail"] = "gpurun_out/bench_detail.json"
+    line = _short(line)
+    text = json.dumps(line, separators=(",", ":"))
+    # belt and braces: whatever a future key adds, the line that carries the metric is never the one that gets cut
+    for drop in ("policy", "arms", "notify_us", "cpu_baseline_torch", "latency_us"):
+        if len(text) < 4000:
+            break
+        line.pop(drop, None)
+        text = json.dumps(line, separators=(",", ":"))
+    return text
+
+
+def emit(out):
+    detail_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(detail_dir, exist_ok=True)
+        with open(os.path.join(detail_dir, "bench_detail.json"), "w") as f:
+            json.dump(out, f, indent=1)
+    except OSError as ex:
+        log("[bench] detail file not written: %s" % ex)
+    log("[bench] detail: " + json.dumps(_short(out)))
+    for ln in SUMMARY:
+        print(ln, file=sys.stderr)
+    sys.stderr.flush()
+    print(headline(out), flush=True)
 
 
 if __name__ == "__main__":
