@@ -315,6 +315,10 @@ class Arm:
     """One way of serving the mix: a scheduler behind the server (with a launch path for the model kernels), or the
     direct no-server multi-stream loop.  run() serves `n` requests at mean inter-arrival `iat_us` (0 = saturation)."""
 
+    verify = 4          # seeded inputs per tenant; every completion is compared with the idle server's answer for its input
+    verified = 0        # completions checked so far, over every arm and run of this process
+    mismatches = 0
+
     def __init__(self, serve, label, sched, dispatch, streams, tenants, extra_kernels, unfair=1e6):
         self.serve, self.label, self.sched, self.dispatch, self.streams = serve, label, sched, dispatch, streams
         self.tenants, self.extra_kernels, self.unfair = tenants, extra_kernels, unfair
@@ -342,7 +346,12 @@ class Arm:
                                               pin_threads=True)
         else:
             jobs = [(self.serve.job_path(t[1]), t[3], t[4]) for t in self.tenants]
-            r = self.serve.client_run(self.srv.name, jobs, iat_us, self.cap, n, warmup_jobs=warmup, seed=seed, pin_threads=True)
+            r = self.serve.client_run(self.srv.name, jobs, iat_us, self.cap, n, warmup_jobs=warmup, seed=seed, pin_threads=True, verify=Arm.verify)
+            if Arm.verify:
+                Arm.verified += r["verified_requests"]
+                Arm.mismatches += r["mismatches"]
+                if r["mismatches"]:
+                    log("[bench] %s: %d of %d checked completions DIFFER from the idle server's answer" % (self.label, r["mismatches"], r["verified_requests"]))
         return r
 
 
@@ -423,6 +432,7 @@ def main():
     ap.add_argument("--unfair", type=float, default=1e6, help="full3: deficit threshold of the headline arm (1e6 = shortest remaining work first only)")
     ap.add_argument("--no-arms", action="store_true", help="only the headline search and timed run (plus roofline and CPU baseline)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-verify", action="store_true", help="do not compare every completion with the idle server's answer for its input")
     ap.add_argument("--no-side", action="store_true", help="skip the side workloads (other configurations, fairness sweep, probes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel over a 64 MiB buffer five times (reference point for memory-traffic counters)")
@@ -550,6 +560,8 @@ def main():
 
     os.environ.setdefault("LLIS_MODEL_SEED", "1")
     os.environ["PAELLA_INPUT_RESIDENT"] = "0"   # every request's input crosses PCIe
+    if args.no_verify:
+        Arm.verify = 0
     ek, streams = args.extra_kernels, args.num_streams
     tenants = MIX
     cap = sum(t[4] for t in tenants)
@@ -591,7 +603,8 @@ def main():
                 break
             rate *= 0.97  # the longer run saw a tail the search point did not: back off and measure again
         main_run, main_point = final
-    value = main_run["throughput_rps"] if main_point["meets_slo"] else None
+    # a rate at which a single answer was wrong is not a rate at which the SLO was met
+    value = main_run["throughput_rps"] if main_point["meets_slo"] and not main_run.get("mismatches") else None
 
     # ---- the same search for plain multi-stream serving, served (fifo, job by job on HIP streams) and without a server
     arms_at_equal_load, equal_rate = {}, None
@@ -749,6 +762,14 @@ def main():
             notify["echo_round_trip_us"] = {"p50": float(rtt[n_echo // 2]), "p99": float(rtt[int(n_echo * 0.99)]),
                                             "what": "host flag store -> resident lane sees it -> ring message readable on the host"}
             log("[bench] notification: echo round trip p50 %.2f / p99 %.2f us" % (rtt[n_echo // 2], rtt[int(n_echo * 0.99)]))
+            ow = np.sort(one_way[one_way > -1e29])
+            if len(ow) >= n_echo // 2:
+                # the lane's clock sample just before its ring store, converted to the host's clock domain, against the host's
+                # sample when the message became readable (reference tests/ipc/shm_channel/latency/shmpc_latency_gpu.cu measures
+                # the same hop including a kernel launch)
+                notify["gpu_to_host_us"] = {"p50": float(ow[len(ow) // 2]), "p99": float(ow[int(len(ow) * 0.99)]), "samples": int(len(ow)),
+                                            "what": "device clock at the lane's ring store -> message readable on the host (one way)"}
+                log("[bench] notification: GPU -> host one way p50 %.2f / p99 %.2f us" % (notify["gpu_to_host_us"]["p50"], notify["gpu_to_host_us"]["p99"]))
         lib.paella_ring_destroy(ring)
 
     # ---- the CPU path beside it: the oracle's forward pass of both tenants on the host cores, combined at the mix's ratio
@@ -793,6 +814,9 @@ def main():
         "offered_rps": main_point["offered_rps"],
         "latency_us": {k: main_point[k] for k in main_point if k.endswith("_us")},
         "slo_met": main_point["meets_slo"],
+        "verified_requests": main_run.get("verified_requests"),  # of the timed run: warm-up and measured completions, each compared
+        "mismatches": main_run.get("mismatches"),                # byte for byte with the idle server's answer for the same input
+        "verified_requests_all_runs": Arm.verified, "mismatches_all_runs": Arm.mismatches,
         "timed_run_attempts": attempts,
         "rate_search": searches,
         "arms_at_equal_offered_load": {"offered_rps": equal_rate, "arms": arms_at_equal_load},

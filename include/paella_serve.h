@@ -65,6 +65,12 @@ typedef struct paella_load_options {
     const char* profile_prefix; /* non-NULL: server-side recording around the measured phase, saved to this prefix */
     const char* trace_path;    /* non-NULL: replay this "<type> <submit time us>" trace (paella_workload_pregen,
                                   llis_app_workload_pregen; reference tests/utils/workload_pregen.cpp:107) instead of drawing */
+    int verify;                /* > 0: verify mode with this many seeded inputs per job type (paella_verify_input): the warm-up runs
+                                  every pooled instance alone on the idle server and keeps the first output of every (type, input) pair;
+                                  every later completion is compared with it byte for byte before its slot is reused (the reference's
+                                  client, app/client.cpp:62-121, checks no output).  0 = off */
+    void* verify_expected;     /* optional: receives those expected outputs, [type][input] one after the other */
+    size_t verify_expected_bytes; /* capacity of verify_expected */
 } paella_load_options;
 
 typedef struct paella_latency_stats {
@@ -78,7 +84,13 @@ typedef struct paella_load_result {
     paella_latency_stats all;
     paella_latency_stats per_type[PAELLA_MAX_JOB_TYPES];
     unsigned queue_full_events, type_full_events;
+    uint64_t verified_requests; /* verify mode: completions compared with their expectation (warm-up included) */
+    uint64_t mismatches;        /* ... and how many differed */
 } paella_load_result;
+
+/* Element i of input `variant` of job type `type` under arrival seed `seed`, as verify mode writes it into a request slot:
+ * floats in [-1, 1).  0 on success. */
+int paella_verify_input(unsigned seed, unsigned type, unsigned variant, float* out, size_t n);
 
 /* Writes an arrival trace with the draws of the live generator (type first, then the gap), in the file set of the
  * reference's tool (reference tests/utils/workload_pregen.cpp:72-115): <prefix>_iat<I>_lns<S>_n<N>_seed<K>.txt plus one

@@ -15,6 +15,8 @@
 //   * <prefix>.txt gets one CSV row: x,num_jobs,elapsed_us, then mean,p50,p90,p95,p99,max,sd overall and
 //     per type; <prefix>_raw.txt all latencies; <prefix>_timeline.txt outstanding-per-type samples.
 // --iat 0 submits as fast as the caps allow (saturation).  A one-line JSON summary goes to stdout.
+// --verify N (no counterpart in the reference, whose client checks no output): N seeded inputs per job type, expected outputs learnt
+// from the idle server during the warm-up, every completion compared with its expectation byte for byte; exit code 3 on a mismatch.
 
 #include <llis/client/client.h>
 #include <llis/client/job_instance_ref.h>
@@ -64,7 +66,8 @@ int main(int argc, char** argv) {
                                      {"fairness", required_argument, nullptr, 'f'},    {"sched_sleep", required_argument, nullptr, 'h'},
                                      {"dist", required_argument, nullptr, 'd'},        {"warmup", required_argument, nullptr, 'w'},        {"no_pin", no_argument, nullptr, 'P'},
                                      {"profile", required_argument, nullptr, 'R'},
-                                     {"trace", required_argument, nullptr, 'T'}};
+                                     {"trace", required_argument, nullptr, 'T'},
+                                     {"verify", required_argument, nullptr, 'V'}};
     for (int i = 0; i < 16; ++i) long_opts.push_back(option{flag_names[i], no_argument, &flag_slot, i + 1});
     long_opts.push_back(option{nullptr, 0, nullptr, 0});
 
@@ -86,13 +89,14 @@ int main(int argc, char** argv) {
             case 'P': opt.pin_threads = false; break;
             case 'R': opt.profile_prefix = optarg; break;
             case 'T': opt.trace_path = optarg; break;
+            case 'V': opt.verify_variants = (unsigned)std::atoi(optarg); break;
             default: return 2;
         }
     }
     if (opt.server_name.empty() || opt.iat < 0 || opt.concurrency <= 0 || opt.num_jobs == 0 || (argc - optind) < 3 || (argc - optind) % 3 != 0 ||
         (opt.dist != "exp" && opt.dist != "ln")) {
         std::fprintf(stderr, "usage: %s --server_name S --iat US [--dist exp|ln] [--ln_sigma X] --concurrency C --num_jobs N [--start_record_num R]\n"
-                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] [--trace FILE] job.so proportion max_outstanding ...\n", argv[0]);
+                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] [--trace FILE] [--verify INPUTS_PER_TYPE] job.so proportion max_outstanding ...\n", argv[0]);
         return 2;
     }
 
@@ -136,19 +140,9 @@ int main(int argc, char** argv) {
 
     LoadGenerator gen(&client, opt, props_cum, max_outstanding);
 
-    // Warm-up: create every pooled instance and run it once.
+    // Warm-up: create every pooled instance and run it once (one at a time in verify mode, which also learns the expected outputs).
     const auto init_start = Clock::now();
-    unsigned total_instances = 0;
-    for (unsigned t = 0; t < job_refs.size(); ++t) {
-        for (unsigned i = 0; i < max_outstanding[t]; ++i) {
-            llis::client::JobInstanceRef* inst = job_refs[t].create_instance();
-            gen.add_instance(t, inst);
-            inst->launch();
-            ++total_instances;
-        }
-    }
-    for (unsigned i = 0; i < total_instances; ++i) client.wait();
-    gen.publish_free_counts();
+    gen.warm_up(job_refs);
     const double init_us = std::chrono::duration<double, std::micro>(Clock::now() - init_start).count();
 
     gen.run();
@@ -191,9 +185,15 @@ int main(int argc, char** argv) {
     for (size_t t = 0; t < per_type.size(); ++t) std::printf("%s%.3f", t ? ", " : "", per_type[t].p50);
     std::printf("], \"per_type_count\": [");
     for (size_t t = 0; t < gen.latencies_per_type().size(); ++t) std::printf("%s%zu", t ? ", " : "", gen.latencies_per_type()[t].size());
-    std::printf("]}\n");
+    std::printf("]");
+    if (opt.verify_variants) std::printf(", \"verified_requests\": %llu, \"mismatches\": %llu", (unsigned long long)gen.verified(), (unsigned long long)gen.mismatches());
+    std::printf("}\n");
     std::fflush(stdout);
+    for (const Mismatch& m : gen.first_mismatches())
+        std::fprintf(stderr, "llis_app_client: output mismatch at checked completion %llu: job type %u, input variant %u, first differing byte %zu\n",
+                     (unsigned long long)m.request, m.type, m.variant, m.offset);
 
     if (!std::getenv("LLIS_CLIENT_KEEP_SERVER")) client.kill_server();
+    if (gen.mismatches()) return 3;
     return 0;
 }

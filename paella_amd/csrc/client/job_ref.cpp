@@ -7,6 +7,8 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
+#include <cstdint>
 #include <stdexcept>
 
 namespace llis {
@@ -19,9 +21,14 @@ JobRef::JobRef(std::unique_ptr<job::Job> job, Client* client, std::string path) 
     c2s_channel_ = client_->get_c2s_channel();
     client_id_ = client_->get_client_id();
 
-    // The name only has to be unique per client; the address of this object is, at creation time.
-    shm_name_ = "llis:shm:" + std::to_string(client_id_) + ":" + std::to_string((intptr_t)this);
-    shm_fd_ = shm_open(shm_name_.c_str(), O_CREAT | O_RDWR, 0600);
+    // The name has to be unique among the live pools of this client.  The reference takes the address of this object
+    // (reference src/client/job_ref.cpp:24), but register_job() returns by value: two calls from one loop build their objects in
+    // the same stack slot, get the same name, and both job types' request slots then alias one shared-memory object (every
+    // answer of one type can be overwritten by the other's inputs).  A per-process counter under the process id cannot repeat.
+    static std::atomic<uint64_t> next_pool{0};
+    shm_name_ = "llis:shm:" + std::to_string(client_id_) + ":" + std::to_string(((uint64_t)getpid() << 24) + next_pool.fetch_add(1));
+    shm_unlink(shm_name_.c_str());  // a leftover of a killed process that had this pid
+    shm_fd_ = shm_open(shm_name_.c_str(), O_CREAT | O_EXCL | O_RDWR, 0600);
     LLIS_CHECK_POSIX(shm_fd_);
 
     register_job();

@@ -8,6 +8,13 @@
 //     when an instance of that type returns; a global cap `concurrency` blocks the submitter;
 //   * latency = completion time - scheduled arrival time; percentiles are sorted[size * q] (truncated).
 // iat == 0 submits as fast as the caps allow (saturation).
+//
+// Verify mode (Options::verify_variants > 0; the reference's client checks no output at all): every pooled instance carries one
+// of `verify_variants` seeded inputs of its job type (verify_input below), the warm-up runs the instances ONE AT A TIME on the
+// otherwise idle server and keeps the first output of every (type, variant) as that pair's expectation, and from then on every
+// completion -- warm-up, measured, whatever shared a launch with whatever -- is compared with its expectation byte for byte
+// before its slot is handed out again; the slot's output area is overwritten with 0xFF bytes before each launch, so a request
+// that was never answered cannot pass on its predecessor's bytes.
 
 #include <llis/client/client.h>
 #include <llis/client/job_instance_ref.h>
@@ -19,6 +26,9 @@
 #include <atomic>
 #include <chrono>
 #include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <map>
 #include <mutex>
 #include <queue>
 #include <random>
@@ -57,6 +67,26 @@ inline Stats summarize(std::vector<double>& v) {
     return s;
 }
 
+// Element i of the seeded input of (seed, job type, variant): 24 bits of splitmix64's output function over a counter, mapped
+// to [-1, 1).  paella_amd/serve.py restates it in numpy (tests compare the two bit for bit and derive the expected model outputs from it).
+inline uint64_t verify_mix(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+inline void verify_input(unsigned seed, unsigned type, unsigned variant, float* out, size_t n) {
+    const uint64_t base = ((uint64_t)seed << 40) ^ ((uint64_t)type << 32) ^ ((uint64_t)variant << 24);
+    for (size_t i = 0; i < n; ++i) out[i] = (float)(verify_mix(base + i) >> 40) * (1.0f / 8388608.0f) - 1.0f;
+}
+
+struct Mismatch {
+    unsigned type = 0, variant = 0;
+    size_t offset = 0;        // first differing byte of the output
+    uint64_t request = 0;     // how many completions had been checked before it
+};
+
 struct Options {
     std::string server_name, prefix = "llis_client", dist = "ln";
     double iat = -1, ln_sigma = 2.0, fairness = -1;
@@ -66,6 +96,7 @@ struct Options {
     bool pin_threads = true;
     std::string trace_path;      // non-empty: replay "<type> <submit time us>" lines (llis_app_workload_pregen) instead of drawing
     std::string profile_prefix;  // non-empty: the server records everything during the measured phase and saves to this prefix
+    unsigned verify_variants = 0;  // > 0: verify mode with this many distinct inputs per job type
     // name-shaping switches (which parameters appear in the output file names, which one is the x column)
     bool n_iat = false, n_lns = false, n_con = false, n_n = false, n_srn = false, n_seed = false, n_fair = false, n_scheds = false;
     bool g_iat = false, g_lns = false, g_con = false, g_n = false, g_srn = false, g_seed = false, g_fair = false, g_scheds = false;
@@ -90,6 +121,65 @@ class LoadGenerator {
         const unsigned ref = inst->get_job_ref_id();
         if (ref >= type_of_ref_.size()) type_of_ref_.resize(ref + 1, 0);
         type_of_ref_[ref] = type;
+    }
+
+    // Creates every pooled instance and runs it once before the clock starts (reference app/client.cpp:425-448 launches them
+    // all and then waits).  In verify mode the runs go one at a time, so the first output of every (type, variant) is what an
+    // idle server answers; the others of the same pair are already held against it.
+    void warm_up(std::vector<llis::client::JobRef>& job_refs) {
+        const unsigned variants = opt_.verify_variants;
+        if (variants) {
+            expected_.assign(job_refs.size(), std::vector<std::vector<char>>(variants));
+            in_size_.clear();
+            out_size_.clear();
+            for (auto& ref : job_refs) {
+                in_size_.push_back(ref.get_job()->get_input_size());
+                out_size_.push_back(ref.get_job()->get_output_size());
+            }
+        }
+        unsigned total = 0;
+        for (unsigned t = 0; t < job_refs.size(); ++t) {
+            for (unsigned i = 0; i < max_outstanding_[t]; ++i) {
+                llis::client::JobInstanceRef* inst = job_refs[t].create_instance();
+                const size_t in_bytes = job_refs[t].get_job()->get_input_size();
+                std::memset(inst->get_input_ptr(), 0, in_bytes);
+                add_instance(t, inst);
+                if (!variants) {
+                    inst->launch();
+                    ++total;
+                    continue;
+                }
+                const unsigned v = i % variants;
+                variant_of_[inst] = v;
+                verify_input(opt_.seed, t, v, static_cast<float*>(inst->get_input_ptr()), in_bytes / sizeof(float));
+                std::memset(inst->get_output_ptr(), 0xFF, out_size_[t]);
+                inst->launch();
+                if (client_->wait() != inst) throw std::runtime_error("verify warm-up: a completion for another instance");
+                std::vector<char>& want = expected_[t][v];
+                if (want.empty() && out_size_[t]) {
+                    want.assign(static_cast<char*>(inst->get_output_ptr()), static_cast<char*>(inst->get_output_ptr()) + out_size_[t]);
+                } else {
+                    check(inst, t);
+                }
+            }
+        }
+        for (unsigned i = 0; i < total; ++i) client_->wait();
+        publish_free_counts();
+    }
+
+    uint64_t verified() const { return verified_; }
+    uint64_t mismatches() const { return mismatches_; }
+    const std::vector<Mismatch>& first_mismatches() const { return first_mismatches_; }
+    // Expected outputs, [type][variant] one after the other (each type's output size); returns the bytes written.
+    size_t copy_expected(void* dst, size_t cap) const {
+        size_t at = 0;
+        for (const auto& type : expected_)
+            for (const auto& e : type) {
+                if (at + e.size() > cap) return at;
+                std::memcpy(static_cast<char*>(dst) + at, e.data(), e.size());
+                at += e.size();
+            }
+        return at;
     }
 
     void publish_free_counts() {
@@ -161,7 +251,25 @@ class LoadGenerator {
         free_instances_[type].pop_back();
         ++outstanding_per_type_[type];
         inst->set_start_time(scheduled_arrival_us);
+        if (opt_.verify_variants && out_size_[type]) std::memset(inst->get_output_ptr(), 0xFF, out_size_[type]);
         inst->launch();
+    }
+
+    // The monitor thread (or the warm-up) compares a completed instance's output with its expectation.
+    void check(llis::client::JobInstanceRef* inst, unsigned type) {
+        const std::vector<char>& want = expected_[type][variant_of_[inst]];
+        ++verified_;
+        if (want.empty() || std::memcmp(inst->get_output_ptr(), want.data(), want.size()) == 0) return;
+        ++mismatches_;
+        if (first_mismatches_.size() < 8) {
+            Mismatch m;
+            m.type = type;
+            m.variant = variant_of_[inst];
+            m.request = verified_ - 1;
+            const char* got = static_cast<const char*>(inst->get_output_ptr());
+            while (m.offset < want.size() && got[m.offset] == want[m.offset]) ++m.offset;
+            first_mismatches_.push_back(m);
+        }
     }
 
     void monitor() {
@@ -172,6 +280,7 @@ class LoadGenerator {
             const double latency = us_since_epoch(now) - inst->get_start_time();
             const double t = std::chrono::duration<double, std::micro>(now - very_start).count();
             const unsigned type = type_of_ref_[inst->get_job_ref_id()];
+            if (opt_.verify_variants) check(inst, type);
             {
                 std::lock_guard<std::mutex> lk(mtx_);
                 free_instances_[type].push_back(inst);
@@ -274,6 +383,13 @@ class LoadGenerator {
     unsigned num_queue_full_ = 0, num_type_full_ = 0;
     unsigned phase_jobs_ = 0;
     bool phase_record_ = true;
+
+    // verify mode
+    std::vector<std::vector<std::vector<char>>> expected_;  // [type][variant]
+    std::vector<size_t> in_size_, out_size_;
+    std::map<llis::client::JobInstanceRef*, unsigned> variant_of_;
+    uint64_t verified_ = 0, mismatches_ = 0;
+    std::vector<Mismatch> first_mismatches_;
 };
 
 

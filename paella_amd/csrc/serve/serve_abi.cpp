@@ -116,6 +116,7 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         opt.pin_threads = o->pin_threads != 0;
         if (o->profile_prefix) opt.profile_prefix = o->profile_prefix;
         if (o->trace_path) opt.trace_path = o->trace_path;
+        opt.verify_variants = o->verify > 0 ? (unsigned)o->verify : 0;
 
         std::vector<float> props_cum;
         std::vector<unsigned> max_outstanding;
@@ -130,17 +131,7 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         for (int t = 0; t < o->num_types; ++t) job_refs.push_back(client.register_job(o->job_paths[t]));
 
         llis::loadgen::LoadGenerator gen(&client, opt, props_cum, max_outstanding);
-        unsigned total = 0;
-        for (int t = 0; t < o->num_types; ++t)
-            for (unsigned i = 0; i < max_outstanding[t]; ++i) {
-                llis::client::JobInstanceRef* inst = job_refs[t].create_instance();
-                std::memset(inst->get_input_ptr(), 0, job_refs[t].get_job()->get_input_size());
-                gen.add_instance((unsigned)t, inst);
-                inst->launch();
-                ++total;
-            }
-        for (unsigned i = 0; i < total; ++i) client.wait();
-        gen.publish_free_counts();
+        gen.warm_up(job_refs);
         gen.run();
 
         std::memset(result, 0, sizeof(*result));
@@ -148,6 +139,12 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         result->throughput_rps = o->num_jobs / result->elapsed_us * 1e6;
         result->queue_full_events = gen.queue_full_events();
         result->type_full_events = gen.type_full_events();
+        result->verified_requests = gen.verified();
+        result->mismatches = gen.mismatches();
+        for (const llis::loadgen::Mismatch& m : gen.first_mismatches())
+            std::fprintf(stderr, "paella_client_run: output mismatch at checked completion %llu: job type %u, input variant %u, first differing byte %zu\n",
+                         (unsigned long long)m.request, m.type, m.variant, m.offset);
+        if (o->verify > 0 && o->verify_expected) gen.copy_expected(o->verify_expected, o->verify_expected_bytes);
         if (latencies_us) std::copy(gen.latencies().begin(), gen.latencies().end(), latencies_us);
         fill(&result->all, gen.latencies());
         for (int t = 0; t < o->num_types; ++t) fill(&result->per_type[t], gen.latencies_per_type()[t]);
@@ -156,6 +153,12 @@ int paella_client_run(const paella_load_options* o, paella_load_result* result, 
         std::fprintf(stderr, "paella_client_run: %s\n", e.what());
         return -1;
     }
+}
+
+int paella_verify_input(unsigned seed, unsigned type, unsigned variant, float* out, size_t n) {
+    if (!out) return -1;
+    llis::loadgen::verify_input(seed, type, variant, out, n);
+    return 0;
 }
 
 int paella_workload_pregen(double iat_us, int dist_exp, double ln_sigma, unsigned num_jobs, unsigned seed, const char* prefix,

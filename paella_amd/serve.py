@@ -18,7 +18,8 @@ class LoadOptions(ctypes.Structure):
     _fields_ = [("server_name", c_char_p), ("num_types", c_int), ("job_paths", c_char_p * MAX_TYPES), ("proportions", c_float * MAX_TYPES),
                 ("max_outstanding", c_uint * MAX_TYPES), ("iat_us", c_double), ("dist_exp", c_int), ("ln_sigma", c_double),
                 ("concurrency", c_int), ("num_jobs", c_uint), ("warmup_jobs", c_uint), ("seed", c_uint), ("pin_threads", c_int),
-                ("profile_prefix", c_char_p), ("trace_path", c_char_p)]
+                ("profile_prefix", c_char_p), ("trace_path", c_char_p), ("verify", c_int), ("verify_expected", c_void_p),
+                ("verify_expected_bytes", c_size_t)]
 
 
 class LatencyStats(ctypes.Structure):
@@ -31,7 +32,7 @@ class LatencyStats(ctypes.Structure):
 
 class LoadResult(ctypes.Structure):
     _fields_ = [("elapsed_us", c_double), ("throughput_rps", c_double), ("all", LatencyStats), ("per_type", LatencyStats * MAX_TYPES),
-                ("queue_full_events", c_uint), ("type_full_events", c_uint)]
+                ("queue_full_events", c_uint), ("type_full_events", c_uint), ("verified_requests", ctypes.c_uint64), ("mismatches", ctypes.c_uint64)]
 
 
 class DirectOptions(ctypes.Structure):
@@ -48,6 +49,7 @@ SERVE_SYMBOLS = {
     "paella_client_run": (c_int, [ctypes.POINTER(LoadOptions), ctypes.POINTER(LoadResult), c_void_p]),
     "paella_direct_multistream_run": (c_int, [ctypes.POINTER(DirectOptions), ctypes.POINTER(LoadResult)]),
     "paella_workload_pregen": (c_int, [c_double, c_int, c_double, c_uint, c_uint, c_char_p, ctypes.POINTER(c_float), c_int, c_char_p, c_size_t]),
+    "paella_verify_input": (c_int, [c_uint, c_uint, c_uint, c_void_p, c_size_t]),
     "paella_client_single": (c_int, [c_char_p, c_char_p, c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p]),
 }
 
@@ -103,8 +105,11 @@ class Server:
 
 
 def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, seed=1, dist="exp", ln_sigma=2.0, pin_threads=False,
-               want_latencies=False, profile_prefix=None, trace_path=None):
-    """jobs = [(path, proportion, max_outstanding), ...].  Returns a dict of the run's statistics."""
+               want_latencies=False, profile_prefix=None, trace_path=None, verify=0, expected_bytes=0):
+    """jobs = [(path, proportion, max_outstanding), ...].  Returns a dict of the run's statistics.
+    verify > 0: verify mode with that many seeded inputs per job type (verify_input); the dict then carries `verified_requests`
+    and `mismatches`, and, when expected_bytes is given, `expected` = the outputs the idle server gave, [type][input] one after
+    the other as bytes."""
     import numpy as np
     o = LoadOptions()
     o.server_name = server_name.encode()
@@ -119,6 +124,10 @@ def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, 
     o.concurrency, o.num_jobs, o.warmup_jobs, o.seed, o.pin_threads = concurrency, num_jobs, warmup_jobs, seed, int(pin_threads)
     o.profile_prefix = profile_prefix.encode() if profile_prefix else None
     o.trace_path = trace_path.encode() if trace_path else None
+    o.verify = verify
+    expected = np.zeros(expected_bytes, np.uint8) if verify and expected_bytes else None
+    if expected is not None:
+        o.verify_expected, o.verify_expected_bytes = expected.ctypes.data, expected.nbytes
     res = LoadResult()
     lat = np.zeros(num_jobs, np.float64) if want_latencies else None
     if lib().paella_client_run(ctypes.byref(o), ctypes.byref(res), lat.ctypes.data if want_latencies else None) != 0:
@@ -128,7 +137,23 @@ def client_run(server_name, jobs, iat_us, concurrency, num_jobs, warmup_jobs=0, 
            "type_full": res.type_full_events}
     if want_latencies:
         out["latencies_us"] = lat
+    if verify:
+        out["verified_requests"], out["mismatches"] = res.verified_requests, res.mismatches
+        if expected is not None:
+            out["expected"] = expected
     return out
+
+
+def verify_input(seed, job_type, variant, n):
+    """numpy restatement of verify mode's seeded input (csrc/serve/load_generator.h): n floats in [-1, 1)."""
+    import numpy as np
+    with np.errstate(over="ignore"):
+        z = np.uint64((seed << 40) ^ (job_type << 32) ^ (variant << 24)) + np.arange(n, dtype=np.uint64)
+        z = z + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    return ((z >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / 8388608.0) - np.float32(1.0)).astype(np.float32)
 
 
 def client_single(server_name, path, x, out_floats, n=1):
@@ -147,6 +172,7 @@ def _result_dict(r, n_types):
     return {"elapsed_us": r.elapsed_us, "throughput_rps": r.throughput_rps, "all": r.all.as_dict(),
             "per_type": [r.per_type[i].as_dict() for i in range(n_types)],
             "queue_full_events": r.queue_full_events, "type_full_events": r.type_full_events}
+
 
 
 def direct_multistream(tenants, iat_us, num_streams, num_jobs, warmup_jobs=0, seed=1, dist="exp", ln_sigma=2.0, pin_threads=False,

@@ -6,6 +6,7 @@
 //   FAKE_VARIANT 3  fake_big   : 3 kernels of 3000 x 256 x 64 regs -- never fits beside anything (over-subscription path)
 //   FAKE_VARIANT 4  fake_self  : a copy stage that reports its own completion (from a thread of its own after 300 us when
 //                                FAKE_SELF_THREAD=1, else before it returns), copy, kernel of 40, copy(pre-notify); output = input + 1
+//   FAKE_VARIANT 5  fake_flaky : fake_mem3 whose every FAKE_FLAKY_EVERY-th run (counted over the process) answers with one wrong byte
 
 #include <llis/job/context.h>
 #include <llis/job/coroutine_job.h>
@@ -28,8 +29,8 @@ namespace {
 
 class FakeJob : public llis::job::CoroutineJob {
   public:
-    size_t get_input_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 ? 100 : 5; }
-    size_t get_output_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 ? 100 : 11; }
+    size_t get_input_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 || FAKE_VARIANT == 5 ? 100 : 5; }
+    size_t get_output_size() override { return FAKE_VARIANT == 2 || FAKE_VARIANT == 4 || FAKE_VARIANT == 5 ? 100 : 11; }
     size_t get_param_size() override { return 4; }
 
     void one_time_init() override {}
@@ -49,7 +50,7 @@ class FakeJob : public llis::job::CoroutineJob {
 #if FAKE_VARIANT == 0 || FAKE_VARIANT == 1
         const int n = FAKE_VARIANT == 0 ? 10 : 50;
         for (int i = 0; i < n; ++i) kernel(5, 256, 0, 32, i == n - 1);
-#elif FAKE_VARIANT == 2
+#elif FAKE_VARIANT == 2 || FAKE_VARIANT == 5
         set_is_mem();
         yield();
         llis_hip_memcpy_async(buf_, io_ptr, 100, LLIS_HIP_H2D, reinterpret_cast<void*>(get_cuda_stream()));
@@ -57,6 +58,14 @@ class FakeJob : public llis::job::CoroutineJob {
         kernel(200, 64, 0, 32, false);
         kernel(17, 256, 8192, 128, false);
         for (int i = 0; i < 100; ++i) buf_[i] = (char)(buf_[i] + 1);
+#if FAKE_VARIANT == 5
+        {
+            static unsigned runs = 0;
+            const char* every = std::getenv("FAKE_FLAKY_EVERY");
+            const unsigned n = every ? (unsigned)std::atoi(every) : 0;
+            if (n && ++runs % n == 0) buf_[7] = (char)(buf_[7] + 1);
+        }
+#endif
         set_is_mem();
         set_pre_notify();
         yield();

@@ -174,15 +174,22 @@ def test_plain_job_with_raw_hooks(cuda):
     assert starts == ends == 3 * (1 + 2 + 3 + 4 + 5)
 
 
-@pytest.mark.parametrize("sched_name", ["fifo", "fifo2", "full3"])
-def test_dummy_job_event_log_is_bit_exact_closed_form(cuda, sched_name):
-    """dummy_short alone, three requests back to back: per stage exactly one dispatch, one start message and
+DUMMY_STAGES = {"dummy_short": 10, "dummy_long": 50, "dummy_10": 10, "dummy_11": 11, "dummy_20": 20, "dummy_21": 21}
+
+
+@pytest.mark.parametrize("job,sched_name", [("dummy_short", "fifo"), ("dummy_short", "fifo2"), ("dummy_short", "full3"),
+                                            ("dummy_long", "fifo"), ("dummy_long", "fifo2"), ("dummy_long", "full3"),
+                                            ("dummy_11", "full3"), ("dummy_20", "full3"), ("dummy_10", "fifo2"), ("dummy_21", "fifo")])
+def test_dummy_job_event_log_is_bit_exact_closed_form(cuda, job, sched_name):
+    """One dummy job alone, three requests back to back: per stage exactly one dispatch, one start message and
     one end message with num=5; stream, notifier and job id come from LIFO pools; the wake-up is sent when the
-    last stage is dispatched (fifo: when the work up to the pre-notify stage has finished)."""
+    last stage is dispatched (fifo: when the work up to the pre-notify stage has finished).  Stage counts follow
+    reference jobs/dummy_long/dummy_long.cu:29-78 (50) and jobs/dummy_{10,11,20,21}/dummy.cu; the 50-stage form is the
+    one that would show a job id, stream or notifier that does not return to its pool."""
     from paella_amd import serve
-    streams = 6
+    streams, stages = 6, DUMMY_STAGES[job]
     with serve.Server(server_name("dummy"), sched_name, num_streams=streams, event_log=True) as srv:
-        serve.client_single(srv.name, serve.job_path("dummy_short"), np.zeros(5, np.uint8), 0, n=3)
+        serve.client_single(srv.name, serve.job_path(job), np.zeros(5, np.uint8), 0, n=3)
     ev = [e for e in sched.parse_log(srv.event_log()) if e[0] != "L"]
     top = streams - 1
     expect = []
@@ -190,14 +197,14 @@ def test_dummy_job_event_log_is_bit_exact_closed_form(cuda, sched_name):
     for req in range(3):
         expect.append(("J", 0, 0, base + req, 0))
         if sched_name == "fifo":
-            expect += [("D", 0, s, top, top, 0, 0) for s in range(10)]
-            for s in range(10):
+            expect += [("D", 0, s, top, top, 0, 0) for s in range(stages)]
+            for s in range(stages):
                 expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
             expect += [("S", 0), ("E", 0)]
         else:
-            for s in range(10):
+            for s in range(stages):
                 expect.append(("D", 0, s, top, top, 0, 0))
-                if s == 9:
+                if s == stages - 1:
                     expect.append(("S", 0))
                 expect += [("B", 0, 1, 5), ("B", 0, 0, 5)]
             expect.append(("E", 0))

@@ -214,3 +214,57 @@ def test_server_outlives_a_client_killed_mid_run(tmp_path):
         for f in os.listdir("/dev/shm"):
             if name in f:
                 os.unlink(os.path.join("/dev/shm", f))
+
+
+def test_verify_mode_checks_every_completion(tmp_path):
+    """llis_app_client --verify: seeded inputs per job type, expectations learnt one request at a time during the warm-up,
+    every completion of the loaded run compared byte for byte: all equal for jobs that answer input + 1."""
+    name = "ptver%d" % os.getpid()
+    srv = start_server(name, "full3", FAKE_HIP_OP_US="20")
+    out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "200", "--dist", "exp", "--concurrency", "24",
+                          "--num_jobs", "500", "--warmup", "60", "--seed", "4", "--prefix", str(tmp_path / "v"), "--no_pin", "--verify", "3",
+                          fake_job("fake_mem3"), "0.6", "12", fake_job("fake_self"), "0.4", "12"],
+                         env=fake_env(), capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    stats = json.loads(out.stdout.strip().splitlines()[-1])
+    # 24 warm-up runs of which 2 x 3 taught the expectations, 60 extra warm-up requests, 500 measured
+    assert stats["verified_requests"] == 24 - 6 + 60 + 500 and stats["mismatches"] == 0
+    assert srv.wait(timeout=30) == 0
+
+
+def test_verify_mode_counts_wrong_answers(tmp_path):
+    """A job whose every 50th run answers with one wrong byte: verify mode counts exactly those, names the byte and the
+    client exits with code 3."""
+    name = "ptflaky%d" % os.getpid()
+    srv = start_server(name, "fifo2", FAKE_HIP_OP_US="20", FAKE_FLAKY_EVERY="50")
+    out = subprocess.run([os.path.join(BIN, "llis_app_client"), "--server_name", name, "--iat", "0", "--dist", "exp", "--concurrency", "8",
+                          "--num_jobs", "400", "--seed", "2", "--prefix", str(tmp_path / "f"), "--no_pin", "--verify", "2",
+                          fake_job("fake_flaky"), "1.0", "8"],
+                         env=fake_env(), capture_output=True, text=True, timeout=120)
+    stats = json.loads(out.stdout.strip().splitlines()[-1])
+    assert stats["verified_requests"] == 8 - 2 + 400
+    assert stats["mismatches"] == (8 + 400) // 50 and out.returncode == 3
+    assert "first differing byte 7" in out.stderr
+    assert srv.wait(timeout=30) == 0
+
+
+def test_verify_input_restated_in_numpy_is_the_generator_bit_for_bit():
+    code = r"""
+import ctypes, os, sys
+sys.path.insert(0, %r)
+ctypes.CDLL(%r, mode=ctypes.RTLD_GLOBAL)
+from paella_amd import serve, _abi
+_abi._cache["llis_hip"] = True
+import numpy as np
+for seed, t, v, n in [(1, 0, 0, 1000), (7, 3, 2, 268203), (123456, 15, 7, 5)]:
+    want = np.zeros(n, np.float32)
+    assert serve.lib().paella_verify_input(seed, t, v, want.ctypes.data, n) == 0
+    got = serve.verify_input(seed, t, v, n)
+    assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32)), (seed, t, v)
+    assert -1.0 <= got.min() and got.max() < 1.0 and (n < 100 or abs(got.mean()) < 0.1)
+a, b = serve.verify_input(1, 0, 0, 64), serve.verify_input(1, 0, 1, 64)
+assert not np.array_equal(a, b)
+print("ok")
+""" % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.join(FAKE_LIB, "libllis_hip.so"))
+    out = subprocess.run(["python3", "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stderr
