@@ -122,7 +122,7 @@ def conv_roofline(models, hip, model, reps, back_to_back=200):
             "by_op": by_op, "direct_rps": direct_rps, "forward_us": sum(per_stage)}
 
 
-def full_device_pass(models, hip, model, images=16, reps=10, timed=True):
+def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None, depth=0, only=None):
     """The conv kernel with the device full: every distinct conv layer of the model (groups == 1) over `images` inputs stacked
     along the height, i.e. with `images` times the pixel tiles -- what the compute units see on the serving path, where packed
     launches on four queues keep 16 to 24 problems in flight -- on the 32 x 32 tile with the layer's own waves per workgroup and
@@ -153,7 +153,12 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True):
         c, h, w, k, r, q = x["C"], x["H"], x["W"], node["K"], node["R"], node["S"]
         wt = (rng.standard_normal((k, c, r, q)) / np.sqrt(c * r * q)).astype(np.float32)
         alone = ops.Conv2d(wt, None, stride=tuple(node["stride"]), pad=tuple(node["pad"]), dil=tuple(node["dil"]), act=ops.ACT_RELU, in_hw=(h, w))
-        hint = (1 << 8) | (1 << 4) | (alone.plan.kw.bit_length() - 1)
+        if only and not any(o in "%dx%d %d->%d %dx%d" % (h, w, c, k, r, q) for o in only):
+            continue
+        # forced shape: waves per workgroup (the layer's own unless given) and chunks of operands in flight per wave (0: default)
+        use_kw = kw if kw and c % 8 == 0 else alone.plan.kw
+        use_depth = depth if c % 8 == 0 else 0
+        hint = (use_depth << 16) | (1 << 8) | (1 << 4) | (use_kw.bit_length() - 1)
         conv = ops.Conv2d(wt, np.zeros(k, np.float32), stride=tuple(node["stride"]), pad=tuple(node["pad"]), dil=tuple(node["dil"]), act=ops.ACT_RELU,
                           in_hw=(h * images, w), tile_hint=hint)
         xin = torch.randn((1, c, h * images, w), device="cuda:0")
@@ -448,6 +453,10 @@ def main():
     ap.add_argument("--full-device", default=None, metavar="MODEL",
                     help="only: the conv kernel with the device full (every conv layer of MODEL over 16 stacked inputs, one launch at a time); "
                          "under counter collection one untimed launch per layer")
+    ap.add_argument("--fd-kw", type=int, default=0, help="with --full-device: waves per workgroup of every tap-major layer (default: the layer's own)")
+    ap.add_argument("--fd-depth", type=int, default=0, help="with --full-device: chunks of operands in flight per wave (3, 4, 6, 8, 12; default 2)")
+    ap.add_argument("--fd-only", default=None, help="with --full-device: comma-separated substrings of the layers to run, e.g. '17x17 768->192'")
+    ap.add_argument("--fd-images", type=int, default=16)
     ap.add_argument("--counter-pass", default=None, metavar="MODEL",
                     help="only this: three forward passes of MODEL, one launch at a time with a synchronize after each (the leg to run "
                          "under `rocprofv3 --pmc`: nothing else is in flight and at most one dispatch is ever queued)")
@@ -459,7 +468,6 @@ def main():
     from paella_amd import _abi, models, serve
     hip = _abi.hip()
     _abi.ops()
-    serve.lib()
     if args.copy_calibration:
         import torch
         n = 16 << 20  # floats: 64 MiB read + 64 MiB written per launch
@@ -472,7 +480,8 @@ def main():
         print(json.dumps({"copy_calibration": {"launches": 5, "kib_read_per_launch": n * 4 / 1024, "kib_written_per_launch": n * 4 / 1024}}), flush=True)
         return
     if args.full_device:
-        fd = full_device_pass(models, hip, args.full_device, timed=not under_counter_collection())
+        fd = full_device_pass(models, hip, args.full_device, images=args.fd_images, timed=not under_counter_collection(), kw=args.fd_kw, depth=args.fd_depth,
+                              only=args.fd_only.split(",") if args.fd_only else None)
         for r in fd["layers"]:
             log("[bench] %-26s x%d  %5d workgroups x %d waves  %8.1f MFLOP  %s" % (r["layer"], r["count"], r["workgroups"], r["waves_per_workgroup"], r["flops"] / 1e6,
                 "%7.2f us  %6.1f TFLOP/s" % (r["us"], r["flops"] / r["us"] / 1e6) if r["us"] else ""))
@@ -558,6 +567,7 @@ def main():
         print(json.dumps(out), flush=True)
         return
 
+    serve.lib()
     os.environ.setdefault("LLIS_MODEL_SEED", "1")
     os.environ["PAELLA_INPUT_RESIDENT"] = "0"   # every request's input crosses PCIe
     if args.no_verify:

@@ -78,6 +78,8 @@ typedef struct paella_conv_plan {
     paella_launch_dims dims;
     double flops;                /* algorithmic: 2*K*(C/g)*R*S*P*Q */
     double bytes;                /* algorithmic: 4*(C*H*W + K*(C/g)*R*S + K + K*P*Q [+K*P*Q residual]) */
+    int depth;                   /* chunks of operands a wave keeps in flight; 0 = the tile's default */
+    int reserved;
 } paella_conv_plan;
 
 /* Pure host arithmetic: picks the kernel variant and launch shape.  tile_hint = 0 lets the library

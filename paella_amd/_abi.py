@@ -3,7 +3,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_DIR = os.path.join(_HERE, "lib")
+LIB_DIR = os.environ.get("PAELLA_LIB_DIR") or os.path.join(_HERE, "lib")  # PAELLA_LIB_DIR: the libraries of another build
 BIN_DIR = os.path.join(_HERE, "bin")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
@@ -23,7 +23,7 @@ class ConvDesc(ctypes.Structure):
 class ConvPlan(ctypes.Structure):
     _fields_ = [("d", ConvDesc), ("P", c_int), ("Q", c_int), ("kind", c_int), ("mi", c_int), ("ni", c_int),
                 ("kw", c_int), ("splits", c_int), ("m_pad", c_int), ("k_pad", c_int), ("k_order", c_int), ("wg_order", c_int), ("fast_div", c_int), ("blob_bytes", c_size_t), ("workspace_bytes", c_size_t), ("dims", LaunchDims),
-                ("flops", c_double), ("bytes", c_double)]
+                ("flops", c_double), ("bytes", c_double), ("depth", c_int), ("reserved", c_int)]
 
 
 class ConvOperands(ctypes.Structure):

@@ -24,6 +24,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <type_traits>
 #include <mutex>
 #include <vector>
 
@@ -40,6 +41,19 @@
 #include "pool_body.h"
 #include "dense_body.h"
 #include "pack.h"
+
+#ifdef PAELLA_CONV_TIMELINE
+// Measurement build only: every wave of a conv leaves eight realtime-counter samples (100 MHz) in this buffer.
+__device__ unsigned long long* g_tl_buf = nullptr;
+__device__ unsigned g_tl_cap = 0;
+#define TL_STAMP(i) tl[i] = wall_clock64()
+extern "C" int paella_conv_timeline_set(void* buf, unsigned waves) {
+    if (hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_tl_buf), &buf, sizeof(buf))) return (int)e;
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_tl_cap), &waves, sizeof(waves));
+}
+#else
+#define TL_STAMP(i)
+#endif
 
 namespace {
 
@@ -113,11 +127,15 @@ struct PreOp {
 };
 
 // One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
-template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false>
+template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false, int DEPTH = 0>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
     // A grouped launch starts every conv at a multiple of eight workgroups (see align_start): the ids between the end of one
     // problem and the start of the next belong to no tile and report to nobody.
+#ifdef PAELLA_CONV_TIMELINE
+    unsigned long long tl[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    TL_STAMP(0);
     if (bid >= (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
@@ -181,13 +199,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const int c_begin = g_begin + wave * cpw;
     const int c_end = min(g_end, c_begin + cpw);
 
+    // Not zeroed here: the first matrix instruction of a wave's first chunk takes a constant zero as its addend (sixteen vector
+    // moves per wave less; a vector instruction costs matrix-pipe time, and a wave that sits in its prologue while others are in
+    // their loops waits for the pipe once per vector instruction).  Only a wave without any chunk zeroes them explicitly.
     f32x16 acc[MI][NI];
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
     // Chunks outside [c_begin, c_end) are requested at an out-of-range offset: the loads keep their place in
     // the (static) issue order, return zeros and touch no memory.
@@ -304,28 +319,52 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // the pipelined loop below a full vmcnt(0).
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
 
-    // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
-    // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
     constexpr int NACC = MI * NI * 16;
     constexpr int RPW = NACC / KW;
-    constexpr bool kPrefetchEpilogue = RPW <= 16;
-    float bias_v[RPW], res_v[RPW];
-    auto out_coords = [&](int r, int& m, int& pix) {
-        const int tile = r >> 4;
+    // (a variant with a deeper operand pipeline keeps its registers for the chunks in flight)
+    constexpr bool kPrefetchEpilogue = DEPTH ? RPW <= 4 : RPW <= 16;
+    // Output addressing.  Register r of the tile (r = wave * RPW + rr for this wave) holds, in lane (j, kk), output channel
+    // m0 + row(r) + 4 * kk at pixel n0 + 32 * ni(r) + j.  Everything that depends on the tile, the wave or r is wave-uniform and
+    // goes into buffer descriptors and scalar offsets built on the scalar unit: per tensor a descriptor at the tile's first
+    // channel that ends at channel K, per register the row's byte offset as the access's scalar offset.  A lane contributes one
+    // byte offset per pixel tile -- its pixel within a channel plane plus the four planes of its half wave, or an offset beyond
+    // any length for a pixel past P*Q -- and the hardware holds the sum against the descriptor's length: rows at or past K and
+    // pixels past P*Q read as zero and their stores are dropped, without a compare on the vector unit.
+    // (K * P * Q * 4 < 2^31 is a condition of the plan.)
+    const unsigned plane = (unsigned)p.PQ * 4u;
+    auto row_of = [&](int rr) {
+        const int r = wave * RPW + rr;
         const int e = r & 15;
-        const int mi = tile / NI;
-        const int ni = tile - mi * NI;
-        m = m0 + mi * 32 + (e >> 2) * 8 + kk * 4 + (e & 3);
-        pix = n0 + ni * 32 + j;
+        return ((r >> 4) / NI) * 32 + (e >> 2) * 8 + (e & 3);
     };
+    auto lane_off = [&](int rr) {  // the same registers for every rr of one pixel tile (one tile unless the wave owns several)
+        const int ni = ((wave * RPW + rr) >> 4) % NI;
+        const int pix = n0 + ni * 32 + j;
+        return pix < p.PQ ? (int)((unsigned)kk * 4u * plane + (unsigned)pix * 4u) : (int)0x80000000u;
+    };
+    const int rows_tile = max(p.K - m0, 0);  // channels from this tile's first one to the last that exists (may exceed the tile)
+    const float* const res_tile = p.residual ? p.residual + (size_t)m0 * p.PQ : nullptr;
+    float* const y_tile = p.y + (size_t)m0 * p.PQ;
+    // The hardware holds lane offset + scalar offset against the length, so the length is that of all the tile's channels; a
+    // row that does not exist gets length zero and scalar offset zero (no sum that could pass a wrapped comparison).
+    auto row_exists = [&](int rr) { return row_of(rr) < rows_tile; };
+    auto plane_rsrc = [&](const float* tile_base, int rr) {
+        return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, row_exists(rr) ? (unsigned)rows_tile * plane : 0u, 0x00027000);
+    };
+    auto chan_rsrc = [&](const float* per_channel, int rr) {  // bias, slope: one float per channel
+        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, row_exists(rr) ? (unsigned)rows_tile * 4u : 0u, 0x00027000);
+    };
+    auto plane_soff = [&](int rr) { return row_exists(rr) ? (int)((unsigned)row_of(rr) * plane) : 0; };
+    auto chan_soff = [&](int rr) { return row_exists(rr) ? row_of(rr) * 4 : 0; };
+    const int chan_voff = kk * 16;
+    // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
+    // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
+    float bias_v[RPW], res_v[RPW];
     if (kPrefetchEpilogue) {
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            int m, pix;
-            out_coords(wave * RPW + rr, m, pix);
-            const bool ok = m < p.K && pix < p.PQ;
-            bias_v[rr] = (ok && p.bias) ? p.bias[m] : 0.f;
-            res_v[rr] = (ok && p.residual) ? p.residual[(size_t)m * p.PQ + pix] : 0.f;
+            bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
+            res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), plane_soff(rr), 0)) : 0.f;
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -338,8 +377,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // chunk's matrix instructions were no better either (23.8 against 24.9 TFLOP/s over a ResNet-18 pass): the loop is
     // bound by what the compute unit's vector cache can take in -- each wave fetches its own 32 x 8 operand
     // fragments, 147 KB per workgroup for a 64-channel 3x3 layer -- not by exposed latency.
-    constexpr int D = (MI * NI == 1) ? 2 : 4;
-    auto compute = [&](const Frag<MI, NI>& f) {
+    constexpr int D = DEPTH ? DEPTH : (MI * NI == 1) ? 2 : 4;
+    // first: the accumulators hold nothing yet, the first matrix instruction into each takes zero as its addend
+    auto compute = [&](const Frag<MI, NI>& f, auto first) {
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -353,13 +394,20 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                         const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
                         bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
                     }
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
+                    if (decltype(first)::value && t == 0) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zero, 0, 0, 0);
+                    else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
                 }
             }
         }
     };
-    // (Raising the wave's priority for the loop, s_setprio 2, or from here to the end of the kernel, s_setprio 3, changed
-    // nothing alone and nothing or -10 % with four passes in flight: 15.8 / 14.2 / 15.8 thousand ResNet-18 passes per second.)
+    constexpr std::true_type kFirst{};
+    constexpr std::false_type kLater{};
+    // (Raising the wave's priority for the loop, s_setprio 2, or from the loop to the end of the kernel, s_setprio 3, changed
+    // nothing alone and nothing or -10 % with four passes in flight: 15.8 / 14.2 / 15.8 thousand ResNet-18 passes per second.
+    // The opposite, priority 3 outside the loop so that prologues and epilogues get their few vector instructions in between
+    // other waves' matrix instructions: +2 % with the device full while a wave still executed some 130 vector instructions
+    // around its loop, -1 % everywhere once those were down to about 70.)
+    TL_STAMP(1);
     if (c_begin < c_end) {
         Frag<MI, NI> frag[D];
 #pragma unroll
@@ -367,56 +415,79 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
         }
+        TL_STAMP(2);
         const int n = c_end - c_begin;
         const int c_main_end = c_begin + (n / D) * D;
-        // Branch-free steady state: whole groups of D chunks.
-        for (int c = c_begin; c < c_main_end; c += D) {
+        // One group of D chunks: each slot is consumed and refilled with the chunk D ahead.
+        auto group = [&](int c, auto first) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
-                compute(frag[d]);
+                if (d == 0) compute(frag[d], first);
+                else compute(frag[d], kLater);
+#ifdef PAELLA_CONV_TIMELINE
+                if (d == 0 && decltype(first)::value) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    TL_STAMP(3);
+                }
+#endif
                 // keep the refill of this slot right here: hoisting all loads to one place would make every
                 // iteration wait for the whole memory latency
                 __builtin_amdgcn_sched_barrier(0);
                 load_frag(c + D + d, c + D + d < c_end, frag[d]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-        }
-        // Up to D-1 leftover chunks are already sitting in the first slots.
-        const int rest = n - (n / D) * D;
+        };
+        if (n >= D) {
+            // Branch-free steady state: whole groups of D chunks, the first one apart (it starts the accumulators).
+            group(c_begin, kFirst);
+            for (int c = c_begin + D; c < c_main_end; c += D) group(c, kLater);
+            // Up to D-1 leftover chunks are already sitting in the first slots.
+            const int rest = n - (n / D) * D;
 #pragma unroll
-        for (int d = 0; d < D - 1; ++d)
-            if (d < rest) compute(frag[d]);
+            for (int d = 0; d < D - 1; ++d)
+                if (d < rest) compute(frag[d], kLater);
+        } else {
+            // fewer chunks than slots: all of them are sitting in the first slots
+            compute(frag[0], kFirst);
+#pragma unroll
+            for (int d = 1; d < D - 1; ++d)
+                if (d < n) compute(frag[d], kLater);
+        }
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
     }
 
     // Finishes the wave's RPW outputs.  Every operand load comes first, then the arithmetic, then the stores back
     // to back: a load between two stores would make the compiler wait for the earlier store as well (one counter
     // covers both), and a write-through store takes about 0.3 us to be acknowledged.
     auto epilogue_all = [&](float (&v)[RPW]) {
-        size_t o[RPW];
-        bool ok[RPW];
         float sl[RPW];
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            int m, pix;
-            out_coords(wave * RPW + rr, m, pix);
-            ok[rr] = m < p.K && pix < p.PQ;
-            o[rr] = (size_t)m * p.PQ + pix;
-            sl[rr] = (ok[rr] && p.act == PAELLA_ACT_PRELU) ? p.slope[m] : 0.f;
-            if (kPrefetchEpilogue) {
-                v[rr] += bias_v[rr];
-                v[rr] += res_v[rr];
-            } else if (ok[rr]) {
-                if (p.bias) v[rr] += p.bias[m];
-                if (p.residual) v[rr] += p.residual[o[rr]];
+            sl[rr] = p.act == PAELLA_ACT_PRELU ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.slope, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
+            if (!kPrefetchEpilogue) {
+                bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
+                res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), plane_soff(rr), 0)) : 0.f;
             }
+        }
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {
+            v[rr] += bias_v[rr];
+            v[rr] += res_v[rr];
         }
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) v[rr] = apply_act(v[rr], p.act, sl[rr], p.lo, p.hi);
 #pragma unroll
-        for (int rr = 0; rr < RPW; ++rr)
-            if (ok[rr]) store_out(p.y + o[rr], v[rr]);
+        for (int rr = 0; rr < RPW; ++rr)  // write-through (sc1), like store_out
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[rr]), plane_rsrc(y_tile, rr), lane_off(rr), plane_soff(rr), 16);
     };
 
+    TL_STAMP(4);
     float mine[RPW];
     if (KW == 1) {
 #pragma unroll
@@ -445,6 +516,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
     }
 
+    TL_STAMP(5);
     if (p.splits == 1) {
         epilogue_all(mine);
     } else {
@@ -456,16 +528,19 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         // partials with device-scope atomic loads, which do not hit in its own caches.  A release on the bump and an acquire
         // after it would add a cache write-back and an invalidate per workgroup for data that never sat in a cache.
         const int tile = tile_m * p.n_tiles_n + tile_n;
-        float* part = p.ws_partials + ((size_t)tile * p.splits + split) * (NACC * 64);
+        // the tile's partial tiles, [split][NACC][64 lanes]: one descriptor, a lane's offset is its lane number
+        const __amdgpu_buffer_rsrc_t pres = __builtin_amdgcn_make_buffer_rsrc((void*)(p.ws_partials + (size_t)tile * p.splits * (NACC * 64)), 0,
+                                                                               (unsigned)p.splits * (NACC * 256u), 0x00027000);
+        const int lane4 = lane * 4;
 #pragma unroll
-        for (int rr = 0; rr < RPW; ++rr) store_out(part + (wave * RPW + rr) * 64 + lane, mine[rr]);
+        for (int rr = 0; rr < RPW; ++rr)
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, mine[rr]), pres, lane4, (split * NACC + wave * RPW + rr) * 256, 16);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         __shared__ unsigned arrived;
         if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(p.ws_counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (arrived == (unsigned)p.splits - 1) {
-            const float* all = p.ws_partials + (size_t)tile * p.splits * (NACC * 64) + (size_t)(wave * RPW) * 64 + lane;
             float v[RPW];
 #pragma unroll
             for (int rr = 0; rr < RPW; ++rr) v[rr] = 0.f;
@@ -473,12 +548,14 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             for (int z0 = 0; z0 < p.splits; z0 += ZB) {
                 float t[ZB][RPW];
 #pragma unroll
-                for (int u = 0; u < ZB; ++u)
+                for (int u = 0; u < ZB; ++u) {
+                    // a split past the last one reads through a descriptor of zero length (zeros, no memory touched); device
+                    // scope (sc1): the partial tiles were written by other workgroups and must not come from this one's caches
+                    const __amdgpu_buffer_rsrc_t zr = z0 + u < p.splits ? pres : __builtin_amdgcn_make_buffer_rsrc((void*)p.ws_partials, 0, 0, 0x00027000);
 #pragma unroll
                     for (int rr = 0; rr < RPW; ++rr)
-                        t[u][rr] = (z0 + u < p.splits)
-                                       ? __hip_atomic_load(all + (size_t)(z0 + u) * (NACC * 64) + rr * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                       : 0.f;
+                        t[u][rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(zr, lane4, ((z0 + u) * NACC + wave * RPW + rr) * 256, 16));
+                }
 #pragma unroll
                 for (int u = 0; u < ZB; ++u)  // split order: the sum does not depend on which workgroup came last
 #pragma unroll
@@ -489,6 +566,18 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
     }
 
+#ifdef PAELLA_CONV_TIMELINE
+    TL_STAMP(6);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    TL_STAMP(7);
+    {
+        const unsigned widx = bid * KW + (unsigned)wave;
+        if (lane == 0 && g_tl_buf && widx < g_tl_cap) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) g_tl_buf[(size_t)widx * 8 + i] = tl[i];
+        }
+    }
+#endif
     // End hook without a barrier: every wave waits for its own write-through stores, then counts itself in LDS; the wave that
     // completes the count reports the workgroup, the others leave the compute unit at once instead of waiting for the report's
     // round trip to the counter in memory (the wave slots they hold are what other workgroups are waiting for).
@@ -504,9 +593,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     }
 }
 
-template <int MI, int NI, int KW, bool TAP_MAJOR>
+template <int MI, int NI, int KW, bool TAP_MAJOR, int DEPTH = 0>
 __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? 1 : 1) void conv_mfma_kernel(ConvArgs p) {
-    conv_tile<MI, NI, KW, TAP_MAJOR>(p, blockIdx.x);
+    conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH>(p, blockIdx.x);
 }
 
 // A conv that applies a per-channel transform to its input on the way (smallest tile, tap-major order).
@@ -687,7 +776,33 @@ ConvKernel pick_tile(int mi, int ni, int kw) {
     return nullptr;
 }
 
-ConvKernel pick_kernel(int mi, int ni, int kw, int k_order = 0) { return k_order ? pick_tile<true>(mi, ni, kw) : pick_tile<false>(mi, ni, kw); }
+// Variants of the 32 x 32 tap-major kernel with fewer waves per tile and more chunks of operands in flight per wave.
+template <int KW>
+ConvKernel pick_depth(int depth) {
+    switch (depth) {
+        case 3: return conv_mfma_kernel<1, 1, KW, true, 3>;
+        case 4: return conv_mfma_kernel<1, 1, KW, true, 4>;
+        case 6: return conv_mfma_kernel<1, 1, KW, true, 6>;
+        case 8: return conv_mfma_kernel<1, 1, KW, true, 8>;
+        case 12: return conv_mfma_kernel<1, 1, KW, true, 12>;
+        default: return nullptr;
+    }
+}
+
+ConvKernel pick_deep_kernel(int kw, int depth) {
+    switch (kw) {
+        case 1: return pick_depth<1>(depth);
+        case 2: return pick_depth<2>(depth);
+        case 4: return pick_depth<4>(depth);
+        case 8: return pick_depth<8>(depth);
+        default: return nullptr;
+    }
+}
+
+ConvKernel pick_kernel(int mi, int ni, int kw, int k_order = 0, int depth = 0) {
+    if (depth) return (mi == 1 && ni == 1 && k_order) ? pick_deep_kernel(kw, depth) : nullptr;
+    return k_order ? pick_tile<true>(mi, ni, kw) : pick_tile<false>(mi, ni, kw);
+}
 
 constexpr size_t kMaxSplitTiles = 16384;  // counters at the head of a split-k workspace
 
@@ -714,6 +829,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
     // Offsets are 32-bit byte offsets and (r*dil, s*dil) are packed into 16 bits each.
     if ((double)d->C * d->H * d->W * 4 >= 2147483648.0 || (d->R - 1) * d->dil_h >= 0x7000 || (d->S - 1) * d->dil_w >= 0x7000)
         return PAELLA_ENOSUP;
+    // ... and so are the output's (a lane's offset within its tile's channels is held against the tensor's length in bytes)
+    if ((double)(d->K + 64) * P * Q * 4 >= 2147483648.0) return PAELLA_ENOSUP;
 
     std::memset(plan, 0, sizeof(*plan));
     plan->d = *d;
@@ -736,6 +853,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             ni = (tile_hint >> 4) & 0xF;
             kw = 1 << (tile_hint & 0xF);
             if (!pick_kernel(mi, ni, kw)) return PAELLA_EINVAL;
+            plan->depth = (tile_hint >> 16) & 0xF;
+            if (plan->depth && !pick_kernel(mi, ni, kw, d->C % 8 == 0 ? 1 : 0, plan->depth)) return PAELLA_EINVAL;
         } else {
             // The 32 x 32 tile unless it would make thousands of workgroups: measured on the layers of the model zoo
             // (one launch at a time) it is the fastest or within 3 % of the fastest everywhere, and up to twice as fast
@@ -749,7 +868,8 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             // reuse (ResNet-18, thousand passes per second, four queues / one): 32 x 32 everywhere 15.8 / 7.0; 64 x 32 where
             // K is a multiple of 64: 12.1 / 4.9, only from K = 256: 13.2 / 5.6; 32 x 64 on the 56 x 56 layers: 14.4 / 6.4.
             // (at most 4 where the reduction goes through the offset table -- stems: 7.8 against 7.9 us, 4.4 against 4.7)
-            const int kw_max = d->C % 8 == 0 ? 8 : 4;
+            static const int kw_cap = [] { const char* e = std::getenv("PAELLA_CONV_KW_MAX"); const int v = e ? std::atoi(e) : 8; return v == 1 || v == 2 || v == 4 ? v : 8; }();
+            const int kw_max = std::min(d->C % 8 == 0 ? 8 : 4, kw_cap);
             kw = 2;
             while (kw < kw_max && kw < nchunks) kw <<= 1;
         }
@@ -1458,11 +1578,11 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     auto* nf = reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier);
     const int PQ = plan->P * plan->Q;
     if (plan->kind == 0) {
-        ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order);
+        ConvKernel kern = pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order, plan->depth);
         if (!kern) return PAELLA_EINVAL;
         ConvArgs a;
         if (int rc = fill_args(plan, x, blob_dev, bias, residual, slope, y, workspace, job_id, nf, a)) return rc;
-        if (plan->mi == 1 && plan->ni == 1 && pack_hold(&plan, &a, 1, stream)) return 0;
+        if (plan->mi == 1 && plan->ni == 1 && !plan->depth && pack_hold(&plan, &a, 1, stream)) return 0;
         if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
         paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, st, a);
         return (int)hipGetLastError();
@@ -1647,7 +1767,7 @@ extern "C" int paella_conv2d_dims(const paella_conv_plan* plan, paella_launch_di
     if (!plan || !dims) return PAELLA_EINVAL;
     *dims = plan->dims;
     add_kernel_resources(plan->kind == 1 ? reinterpret_cast<const void*>(dwconv_kernel)
-                                         : reinterpret_cast<const void*>(pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order)), dims);
+                                         : reinterpret_cast<const void*>(pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order, plan->depth)), dims);
     return 0;
 }
 
