@@ -1,0 +1,3 @@
+build_tl3/hip/hip_layer.hsaco: hip/hip_layer.hip \
+  ../../include/paella_hip.h
+../../include/paella_hip.h:

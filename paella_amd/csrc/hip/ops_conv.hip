@@ -94,11 +94,16 @@ struct ConvArgs {
     // chunks per filter tap, filter width; fast_div = 0: operands too large for the shortcut, divide
     FastDiv div_w, div_tm, div_q, div_cb, div_s;
     int fast_div;
+    int pointwise;                  // tap-major only: 1x1 filter, stride 1, no padding
 };
 
 __device__ __forceinline__ unsigned quot(unsigned a, unsigned d, const FastDiv& f, int fast) {
     return fast ? __umulhi(a, f.mul) + (a & f.one) : a / d;
 }
+
+// The same without the fallback, for dividends and divisors the host has checked (chunk numbers by chunks per tap, taps by
+// filter width).
+__device__ __forceinline__ unsigned quot_fast(unsigned a, const FastDiv& f) { return __umulhi(a, f.mul) + (a & f.one); }
 
 __device__ __forceinline__ float apply_act(float v, int act, float slope, float lo, float hi) {
     switch (act) {
@@ -127,9 +132,12 @@ struct PreOp {
 };
 
 // One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
-template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false, int DEPTH = 0>
+// PW ("pointwise"): a 1x1 filter with stride 1 and no padding in tap-major order -- an input pixel is its output pixel, there
+// are no taps to step through and nothing to test per tap.
+template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false, int DEPTH = 0, bool PW = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
+    static_assert(!PW || TAP_MAJOR, "the pointwise shortcut belongs to the tap-major order");
     // A grouped launch starts every conv at a multiple of eight workgroups (see align_start): the ids between the end of one
     // problem and the start of the next belong to no tile and report to nobody.
 #ifdef PAELLA_CONV_TIMELINE
@@ -179,17 +187,28 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const int m0 = tile_m * (32 * MI);
     const int n0 = tile_n * (32 * NI);
 
-    __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, p.x_bytes, 0x00027000);
+    // The input through a descriptor that starts pad_off bytes in front of the tensor, pad_off = (pad_h * W + pad_w) * 4: a lane's
+    // offset is then that of input element (ho * stride_h, wo * stride_w) -- never negative, so a filter tap's offset
+    // (r * dil_h * W + s * dil_w) * 4 can ride in the loads' scalar offset and the lane's part need not change with the tap.
+    const unsigned pad_off = TAP_MAJOR ? (unsigned)(p.ph * p.W + p.pw) * 4u : 0u;
+    __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(p.x) - pad_off), 0, p.x_bytes + pad_off, 0x00027000);
 
+    const int HW4 = p.H * p.W * 4;
+    const int kk4hw = kk * 4 * HW4;
     int hb[NI], wb[NI], base[NI];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int pix = n0 + ni * 32 + j;
+        if (PW) {  // input pixel = output pixel
+            hb[ni] = wb[ni] = 0;
+            base[ni] = pix < p.PQ ? pix * 4 + kk4hw : -1;
+            continue;
+        }
         const int ho = (int)quot((unsigned)pix, (unsigned)p.Q, p.div_q, p.fast_div);
-        const int wo = pix - ho * p.Q;
-        hb[ni] = (pix < p.PQ) ? ho * p.sh - p.ph : -0x10000000;
-        wb[ni] = wo * p.sw - p.pw;
-        base[ni] = (hb[ni] * p.W + wb[ni]) * 4;
+        const int wo = pix - __mul24(ho, p.Q);  // every factor here is a pixel coordinate or an extent: far below 2^23
+        hb[ni] = (pix < p.PQ) ? __mul24(ho, p.sh) - p.ph : -0x100000;
+        wb[ni] = __mul24(wo, p.sw) - p.pw;
+        base[ni] = (__mul24(hb[ni], p.W) + wb[ni]) * 4 + (TAP_MAJOR ? (int)pad_off + kk4hw : 0);
     }
 
     // Reduction range of this workgroup (grid-level split), then of this wave inside it.
@@ -207,21 +226,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // Chunks outside [c_begin, c_end) are requested at an out-of-range offset: the loads keep their place in
     // the (static) issue order, return zeros and touch no memory.
     __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, p.w_bytes, 0x00027000);
-    // Tap-major order: running, wave-uniform position of the next chunk to request (load_frag is always called
-    // with consecutive chunk indices): channel block within the tap, filter row, filter column.
-    const int HW4 = p.H * p.W * 4;
-    const int kk4hw = kk * 4 * HW4;
     __amdgpu_buffer_rsrc_t sres, hres;
     if (PRE) {
         sres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, (unsigned)(p.CB * 32), 0x00027000);
         hres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, (unsigned)(p.CB * 32), 0x00027000);
-    }
-    int st_cb = 0, st_r = 0, st_s = 0;
-    if (TAP_MAJOR) {
-        const int tap = (int)quot((unsigned)c_begin, (unsigned)p.CB, p.div_cb, p.fast_div);
-        st_cb = c_begin - tap * p.CB;
-        st_r = (int)quot((unsigned)tap, (unsigned)p.S, p.div_s, p.fast_div);
-        st_s = tap - st_r * p.S;
     }
     // Vector instructions take their four cycles out of the matrix pipe's time on this part (a matrix instruction and a vector
     // instruction of any wave of the SIMD do not overlap), so the per-chunk address arithmetic is kept on the scalar unit:
@@ -234,7 +242,14 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     int tap_voff[NI];
     bool tap_ok[NI];
     bool tap_stale = true;
+    int tap_off = 0;  // byte offset of the current filter tap, wave-uniform
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
+#if defined(PAELLA_CONV_ABLATE) && (PAELLA_CONV_ABLATE & 2)  // measurement build: no operand loads
+        for (int mi = 0; mi < MI; ++mi) f.a[mi] = make_float4((float)c, 1.f, 2.f, 3.f);
+        for (int ni = 0; ni < NI; ++ni)
+            for (int t = 0; t < 4; ++t) f.b[ni][t] = (float)(c + t);
+        return;
+#endif
         if (TAP_MAJOR) {
             const __amdgpu_buffer_rsrc_t wr = valid ? wres : nores;
 #pragma unroll
@@ -242,34 +257,37 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 const auto v = __builtin_amdgcn_raw_buffer_load_b128(wr, wlane, c * wstep + mi * 32 * 16, 0);
                 f.a[mi] = __builtin_bit_cast(float4, v);
             }
-            if (tap_stale | (st_cb == 0)) {  // wave-uniform: once per filter tap
-                const int dy = st_r * p.dh, dx = st_s * p.dw;
+            // Where chunk c lies: filter tap and channel block within it, all on the scalar unit (two multiply-highs; a running
+            // position with carries from block to column to row ended up in vector registers).
+            int cb = c, tap_soff = 0;
+            if (!PW) {
+                const int tap = (int)quot_fast((unsigned)c, p.div_cb);
+                cb = c - tap * p.CB;
+                if (tap_stale | (cb == 0)) {  // wave-uniform: once per filter tap
+                    const int r = (int)quot_fast((unsigned)tap, p.div_s);
+                    const int dy = r * p.dh, dx = (tap - r * p.S) * p.dw;
+                    tap_off = (dy * p.W + dx) * 4;
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    const int h = hb[ni] + dy;
-                    const int w = wb[ni] + dx;
-                    tap_ok[ni] = ((unsigned)h < (unsigned)p.H) & ((unsigned)w < (unsigned)p.W);
-                    tap_voff[ni] = tap_ok[ni] ? base[ni] + (dy * p.W + dx) * 4 + kk4hw : -1;
+                    for (int ni = 0; ni < NI; ++ni) {
+                        tap_ok[ni] = ((unsigned)(hb[ni] + dy) < (unsigned)p.H) & ((unsigned)(wb[ni] + dx) < (unsigned)p.W);
+                        tap_voff[ni] = tap_ok[ni] ? base[ni] : -1;
+                    }
+                    tap_stale = false;
                 }
-                tap_stale = false;
+                tap_soff = tap_off;
             }
             const __amdgpu_buffer_rsrc_t xr = valid ? xres : nores;
-            const int chunk_off = st_cb * 8 * HW4;
+            const int chunk_off = cb * 8 * HW4 + tap_soff;
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
+                const int voff = PW ? base[ni] : tap_voff[ni];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, tap_voff[ni], chunk_off + t * HW4, 0));
+                for (int t = 0; t < 4; ++t) f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, voff, chunk_off + t * HW4, 0));
                 if (PRE) {  // a tap outside the image gets scale = shift = 0, so it stays the zero the padding asks for
-                    const int soff = (valid & tap_ok[ni]) ? (st_cb * 8 + kk * 4) * 4 : -1;
+                    const bool inside = PW ? base[ni] != -1 : tap_ok[ni];
+                    const int soff = (valid & inside) ? (cb * 8 + kk * 4) * 4 : -1;
                     f.sc = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(sres, soff, 0, 0));
                     f.sh = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(hres, soff, 0, 0));
-                }
-            }
-            if (++st_cb == p.CB) {
-                st_cb = 0;
-                if (++st_s == p.S) {
-                    st_s = 0;
-                    ++st_r;
                 }
             }
             return;
@@ -359,15 +377,17 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const int chan_voff = kk * 16;
     // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
     // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
+    // (requested once the first chunks' operand loads are out: the loop cannot start before those arrive)
     float bias_v[RPW], res_v[RPW];
-    if (kPrefetchEpilogue) {
+    auto prefetch_epilogue = [&]() {
+        if (!kPrefetchEpilogue) return;
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
             bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
             res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), plane_soff(rr), 0)) : 0.f;
         }
         __builtin_amdgcn_sched_barrier(0);
-    }
+    };
 
     // Software pipeline of depth D: D chunks of operands are in flight per wave; each slot is refilled with
     // the chunk D ahead right after it has been consumed.  Shallow is better here: the small tile measured
@@ -394,8 +414,13 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                         const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
                         bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
                     }
+#if defined(PAELLA_CONV_ABLATE) && (PAELLA_CONV_ABLATE & 1)  // measurement build: no matrix instructions
+                    if (decltype(first)::value && t == 0) acc[mi][ni] = zero;
+                    acc[mi][ni][0] += av * bv;
+#else
                     if (decltype(first)::value && t == 0) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zero, 0, 0, 0);
                     else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
+#endif
                 }
             }
         }
@@ -415,6 +440,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
         }
+        prefetch_epilogue();
         TL_STAMP(2);
         const int n = c_end - c_begin;
         const int c_main_end = c_begin + (n / D) * D;
@@ -454,6 +480,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 if (d < n) compute(frag[d], kLater);
         }
     } else {
+        prefetch_epilogue();
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -593,9 +620,19 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     }
 }
 
+// The second launch bound is waves per SIMD: eight is what the eight-wave workgroups of the small tile are planned for (four
+// workgroups per compute unit), and the bound keeps the scalar registers within 96 as well -- a wave that takes more than 100
+// of a SIMD's 800 leaves room for seven (three workgroups per compute unit).
 template <int MI, int NI, int KW, bool TAP_MAJOR, int DEPTH = 0>
-__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8) ? 1 : 1) void conv_mfma_kernel(ConvArgs p) {
-    conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH>(p, blockIdx.x);
+__global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8 && DEPTH == 0) ? 8 : 1) void conv_mfma_kernel(ConvArgs args) {
+    // The arguments are read through an index the compiler cannot see through (always 0), as the grouped kernel reads its
+    // member's: a field is then fetched from the argument block where it is used instead of being held in a scalar register
+    // from the first instruction to the epilogue (106 scalar registers and seven waves per SIMD otherwise, or 57 spills).
+    int idx = 0;
+    asm volatile("" : "+s"(idx));
+    const ConvArgs& p = (&args)[idx];
+    if (TAP_MAJOR && p.pointwise) conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH, TAP_MAJOR>(p, blockIdx.x);
+    else conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH>(p, blockIdx.x);
 }
 
 // A conv that applies a per-channel transform to its input on the way (smallest tile, tap-major order).
@@ -605,8 +642,12 @@ struct ConvPreArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_kernel(ConvPreArgs a) {
-    conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
+__global__ __launch_bounds__(64 * KW) void conv_mfma_pre_kernel(ConvPreArgs args) {
+    int idx = 0;  // see conv_mfma_kernel
+    asm volatile("" : "+s"(idx));
+    const ConvPreArgs& a = (&args)[idx];
+    if (a.conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(a.conv, blockIdx.x, a.pre);
+    else conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
 }
 
 // The same for up to kPackMax such convs of different requests in one launch (launch packing).
@@ -616,12 +657,13 @@ struct ConvPreGroupArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
+__global__ __launch_bounds__(64 * KW) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
     int idx = 0;
 #pragma unroll
     for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
         if (blockIdx.x >= g.start[i]) idx = i;
-    conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
+    if (g.m[idx].conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
+    else conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
 }
 
 // Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
@@ -653,7 +695,7 @@ struct ConvGroupArgs {
 };
 
 template <int KW, bool TAP_MAJOR>
-__global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
     int idx = 0;
 #pragma unroll
     for (int i = 1; i < kPackMax; ++i)
@@ -676,7 +718,8 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 1 : 1) void conv_mfma_group_kern
         paella::hook_exit(d.notifier, d.job_id, blocks);
         return;
     }
-    conv_tile<1, 1, KW, TAP_MAJOR>(g.m[idx].conv, bid);
+    if (TAP_MAJOR && g.m[idx].conv.pointwise) conv_tile<1, 1, KW, TAP_MAJOR, false, 0, TAP_MAJOR>(g.m[idx].conv, bid);
+    else conv_tile<1, 1, KW, TAP_MAJOR>(g.m[idx].conv, bid);
 }
 
 constexpr int kMaxGroupWithPool = 3;  // convs of one call that also carries a pooling operator
@@ -1012,6 +1055,9 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     const uint64_t most = std::max<uint64_t>({total, (uint64_t)a.n_tiles_n * 32 * plan->ni, (uint64_t)a.nchunks + a.chunks_per_split});
     const uint64_t widest = std::max<uint64_t>({d_w, (uint64_t)a.n_tiles_m, (uint64_t)plan->Q, d_cb, (uint64_t)d.S});
     a.fast_div = (plan->fast_div && most * widest < ((uint64_t)1 << 32)) ? 1 : 0;
+    // The reduction loop locates its chunks with the multiply-high alone (chunk by chunks per tap, tap by filter width).
+    if (((uint64_t)a.nchunks + a.chunks_per_split + 64) * std::max<uint64_t>(d_cb, (uint64_t)d.S) >= ((uint64_t)1 << 32)) return PAELLA_ENOSUP;
+    a.pointwise = plan->k_order && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1 && d.pad_h == 0 && d.pad_w == 0 ? 1 : 0;
     return 0;
 }
 
