@@ -244,12 +244,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     bool tap_stale = true;
     int tap_off = 0;  // byte offset of the current filter tap, wave-uniform
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
-#if defined(PAELLA_CONV_ABLATE) && (PAELLA_CONV_ABLATE & 2)  // measurement build: no operand loads
-        for (int mi = 0; mi < MI; ++mi) f.a[mi] = make_float4((float)c, 1.f, 2.f, 3.f);
-        for (int ni = 0; ni < NI; ++ni)
-            for (int t = 0; t < 4; ++t) f.b[ni][t] = (float)(c + t);
-        return;
-#endif
         if (TAP_MAJOR) {
             const __amdgpu_buffer_rsrc_t wr = valid ? wres : nores;
 #pragma unroll
@@ -414,13 +408,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                         const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
                         bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
                     }
-#if defined(PAELLA_CONV_ABLATE) && (PAELLA_CONV_ABLATE & 1)  // measurement build: no matrix instructions
-                    if (decltype(first)::value && t == 0) acc[mi][ni] = zero;
-                    acc[mi][ni][0] += av * bv;
-#else
                     if (decltype(first)::value && t == 0) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zero, 0, 0, 0);
                     else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
-#endif
                 }
             }
         }
