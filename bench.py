@@ -699,6 +699,19 @@ def main():
             r = serve.client_run(arm.srv.name, jobs, 1e6 / half, cap, 8192, warmup_jobs=512, dist="ln", ln_sigma=1.5, pin_threads=True)
             side["lognormal_arrivals_sigma_1.5"] = point_of(r, tenants, half)
 
+        # The request ring's own latency (client -> server), the reference's PRINT_LAUNCH_JOB_IPC_LATENCY probe (reference
+        # src/server/server.cpp:121-141): LAUNCH_JOB carries its send time, the server averages now - sent; the headline mix at half
+        # its SLO rate, the first 1000 requests left out.
+        os.environ["LLIS_IPC_LATENCY_SKIP"] = "1000"
+        os.environ["PAELLA_DISPATCH"] = "direct"
+        with serve.Server("bench%d_ipc" % os.getpid(), "full3", num_streams=streams, cpu=4, extra_kernels=ek, print_ipc_latency=True) as srv:
+            half = 0.5 * (value or main_run["throughput_rps"])
+            serve.client_run(srv.name, [(serve.job_path(t[1]), t[3], t[4]) for t in tenants], 1e6 / half, cap, 8192, warmup_jobs=512, pin_threads=True)
+            mean_us, count = srv.ipc_latency()
+        os.environ.pop("PAELLA_DISPATCH", None)
+        side["launch_job_ipc_latency"] = {"mean_us": mean_us, "requests": count, "offered_rps": half}
+        log("[bench] request ring: LAUNCH_JOB reaches the server %.2f us after the client sent it (mean of %d requests at %.0f req/s)" % (mean_us, count, half))
+
         # Deficit-threshold sweep (reference sosp23_artifact/gen_data_fig13.sh:37-60): ResNet-18 : Inception-v3 = 0.952 : 0.048 at
         # saturation, latency of each model over its latency alone, Jain's index over those slowdowns.
         from paella_amd import fairness

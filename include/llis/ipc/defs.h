@@ -15,7 +15,7 @@ using JobId = uint32_t;
 enum class MsgType : uint32_t {
     REGISTER_CLIENT = 0,      // {u32 temporary id}                         -> u32 client id on the temporary reply ring
     REGISTER_JOB = 1,         // {u32 client, str library path, str pool}   -> u32 job reference id
-    LAUNCH_JOB = 2,           // {u32 job reference, i32 pool, size_t offset, void* client-side handle}
+    LAUNCH_JOB = 2,           // {[u64 send time,] u32 job reference, i32 pool, size_t offset, void* client-side handle}
     GROW_POOL = 3,            // {u32 job reference, size_t bytes}
     CUDA_PROFILER_START = 4,  // (names kept from the reference; they switch the device profiler range on / off)
     CUDA_PROFILER_STOP = 5,
@@ -38,6 +38,18 @@ enum class ProfilerMsgType : uint32_t {
 #undef LLIS_PROFILER_MSG
     SAVE = 12,
 };
+
+namespace ipc {
+// Whether LAUNCH_JOB carries the client's send time (std::chrono::steady_clock ticks, a u64 right behind the message type)
+// so that the server can report the mean client-to-server latency of the request ring.  The reference compiles this in or
+// out on both sides with -DPRINT_LAUNCH_JOB_IPC_LATENCY (reference CMakeLists.txt:27-45, src/client/job_instance_ref.cpp:35-38,
+// src/server/server.cpp:121-141); here it is a process-wide run-time switch with the same default rule -- on when this
+// library was built with that macro, else the environment variable LLIS_PRINT_LAUNCH_JOB_IPC_LATENCY=1, else off -- which
+// `llis_server --print_ipc_latency` and `llis_app_client --print_ipc_latency` set.  Client and server must agree (the two
+// encodings cannot be told apart on the ring), exactly as two reference builds must.
+bool launch_timestamps();
+void set_launch_timestamps(bool on);
+}  // namespace ipc
 
 static_assert((uint32_t)ProfilerMsgType::UNSET_RECORD_RESOURCE_EVENTS == 11 && (uint32_t)ProfilerMsgType::SET_RECORD_RUN_NEXT_TIMES == 6,
               "profiler sub-commands are wire values");

@@ -49,6 +49,9 @@ class Server {
     Profiler* get_profiler() { return &profiler_; }
     EventLog* get_event_log() { return &event_log_; }
     const std::string& get_name() const { return server_name_; }
+    // With ipc::launch_timestamps(): mean client-to-server latency of LAUNCH_JOB in microseconds and how many requests it covers.
+    double ipc_latency_mean_us() const { return ipc_latency_count_ ? ipc_latency_sum_ns_ / (double)ipc_latency_count_ / 1e3 : 0.0; }
+    uint64_t ipc_latency_count() const { return ipc_latency_count_; }
 
   private:
     void handle_c2s();
@@ -74,6 +77,10 @@ class Server {
     std::atomic<bool> stop_{false};
     unsigned total_owed_wakeups_ = 0;
     unsigned polls_since_retry_ = 0;
+
+    unsigned ipc_latency_skip_ = 10000, ipc_latency_skipped_ = 0;  // LLIS_IPC_LATENCY_SKIP overrides the reference's 10 000
+    uint64_t ipc_latency_count_ = 0;
+    double ipc_latency_sum_ns_ = 0;
 };
 
 }  // namespace server

@@ -37,6 +37,9 @@ typedef struct paella_server_options {
     int measure_block_time;    /* 1: --measure_block_time (per-workgroup entry/exit clocks for the profiler) */
     unsigned noti_batch;       /* --noti_batch: workgroups per aggregated notification, a power of two <= 128; 0 = default (64);
                                   16 = the reference's constant (reference include/llis/job/finished_block_notifier.h:118) */
+    int print_ipc_latency;     /* 1: --print_ipc_latency: LAUNCH_JOB carries its send time and the server reports the request ring's mean
+                                  latency (the reference's PRINT_LAUNCH_JOB_IPC_LATENCY build, reference src/server/server.cpp:121-141).  The
+                                  switch is process-wide: clients of this process send the time from then on; 0 leaves it as it is */
 } paella_server_options;
 
 int paella_server_start(const paella_server_options* options, paella_server** out);
@@ -45,6 +48,12 @@ int paella_server_stop(paella_server* server);
 /* Text of the event log recorded so far (call after paella_server_stop, or while the server is idle).
  * Copies at most cap bytes including the NUL; returns the full length. */
 size_t paella_server_event_log(paella_server* server, char* buf, size_t cap);
+/* With print_ipc_latency: mean client-to-server latency of LAUNCH_JOB in microseconds over `*count` requests (the first
+ * LLIS_IPC_LATENCY_SKIP requests, 10 000 unless the environment says otherwise, are left out as in the reference).
+ * Call while the server runs.  0 on success. */
+int paella_server_ipc_latency(paella_server* server, double* mean_us, uint64_t* count);
+/* Switches the send time in LAUNCH_JOB off again for this process (after the server that asked for it has stopped). */
+void paella_ipc_latency_off(void);
 
 #define PAELLA_MAX_JOB_TYPES 16
 

@@ -15,12 +15,15 @@
 //   * <prefix>.txt gets one CSV row: x,num_jobs,elapsed_us, then mean,p50,p90,p95,p99,max,sd overall and
 //     per type; <prefix>_raw.txt all latencies; <prefix>_timeline.txt outstanding-per-type samples.
 // --iat 0 submits as fast as the caps allow (saturation).  A one-line JSON summary goes to stdout.
+// --print_ipc_latency: LAUNCH_JOB carries its send time (the reference's PRINT_LAUNCH_JOB_IPC_LATENCY build); the server must
+// run with the same switch.
 // --verify N (no counterpart in the reference, whose client checks no output): N seeded inputs per job type, expected outputs learnt
 // from the idle server during the warm-up, every completion compared with its expectation byte for byte; exit code 3 on a mismatch.
 
 #include <llis/client/client.h>
 #include <llis/client/job_instance_ref.h>
 #include <llis/client/job_ref.h>
+#include <llis/ipc/defs.h>
 
 #include <getopt.h>
 #include <pthread.h>
@@ -67,7 +70,8 @@ int main(int argc, char** argv) {
                                      {"dist", required_argument, nullptr, 'd'},        {"warmup", required_argument, nullptr, 'w'},        {"no_pin", no_argument, nullptr, 'P'},
                                      {"profile", required_argument, nullptr, 'R'},
                                      {"trace", required_argument, nullptr, 'T'},
-                                     {"verify", required_argument, nullptr, 'V'}};
+                                     {"verify", required_argument, nullptr, 'V'},
+                                     {"print_ipc_latency", no_argument, nullptr, 'L'}};
     for (int i = 0; i < 16; ++i) long_opts.push_back(option{flag_names[i], no_argument, &flag_slot, i + 1});
     long_opts.push_back(option{nullptr, 0, nullptr, 0});
 
@@ -90,13 +94,14 @@ int main(int argc, char** argv) {
             case 'R': opt.profile_prefix = optarg; break;
             case 'T': opt.trace_path = optarg; break;
             case 'V': opt.verify_variants = (unsigned)std::atoi(optarg); break;
+            case 'L': llis::ipc::set_launch_timestamps(true); break;
             default: return 2;
         }
     }
     if (opt.server_name.empty() || opt.iat < 0 || opt.concurrency <= 0 || opt.num_jobs == 0 || (argc - optind) < 3 || (argc - optind) % 3 != 0 ||
         (opt.dist != "exp" && opt.dist != "ln")) {
         std::fprintf(stderr, "usage: %s --server_name S --iat US [--dist exp|ln] [--ln_sigma X] --concurrency C --num_jobs N [--start_record_num R]\n"
-                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] [--trace FILE] [--verify INPUTS_PER_TYPE] job.so proportion max_outstanding ...\n", argv[0]);
+                             "          [--seed S] [--prefix OUT] [--warmup N] [--no_pin] [--profile PREFIX] [--trace FILE] [--verify INPUTS_PER_TYPE] [--print_ipc_latency] job.so proportion max_outstanding ...\n", argv[0]);
         return 2;
     }
 

@@ -5,6 +5,7 @@
 #include "load_generator.h"
 #include "workload_pregen.h"
 
+#include <llis/ipc/defs.h>
 #include <llis/server/scheduler.h>
 #include <llis/server/server.h>
 
@@ -50,6 +51,7 @@ int paella_server_start(const paella_server_options* o, paella_server** out) {
         so.mem_marker = o->mem_marker != 0;
         so.measure_block_time = o->measure_block_time != 0;
         so.noti_batch = o->noti_batch;
+        if (o->print_ipc_latency) llis::ipc::set_launch_timestamps(true);
         auto s = std::make_unique<paella_server>();
         s->scheduler = llis::server::SchedulerFactory::create(o->sched, so);
         s->server = std::make_unique<llis::server::Server>(o->name, s->scheduler.get());
@@ -88,6 +90,15 @@ int paella_server_stop(paella_server* s) {
     }
     return 0;
 }
+
+int paella_server_ipc_latency(paella_server* s, double* mean_us, uint64_t* count) {
+    if (!s || s->stopped || !mean_us || !count) return -1;
+    *mean_us = s->server->ipc_latency_mean_us();
+    *count = s->server->ipc_latency_count();
+    return 0;
+}
+
+void paella_ipc_latency_off(void) { llis::ipc::set_launch_timestamps(false); }
 
 size_t paella_server_event_log(paella_server* s, char* buf, size_t cap) {
     if (!s) return 0;

@@ -1,8 +1,10 @@
 // llis_server --name NAME --sched {fifo,fifo2,full3} [--num_streams N] [--extra_kernels N] [--unfair X]
 //             [--sched_sleep N] [--mem_notify {marker,hostfunc}] [--device N] [--measure_block_time] [--noti_batch N]
+//             [--print_ipc_latency]
 // Same options and defaults as reference src/server/server.cpp:203-235; an unknown scheduler name is an
 // error with the list of known ones instead of a null dereference.
 
+#include <llis/ipc/defs.h>
 #include <llis/server/scheduler.h>
 #include <llis/server/server.h>
 
@@ -19,7 +21,7 @@
 static void usage(const char* argv0) {
     std::fprintf(stderr,
                  "usage: %s --name NAME --sched {fifo,fifo2,full3} [--num_streams 500] [--extra_kernels 2]\n"
-                 "          [--unfair 1000000] [--sched_sleep 0] [--mem_notify marker|hostfunc] [--device 0] [--measure_block_time] [--noti_batch 64]\n",
+                 "          [--unfair 1000000] [--sched_sleep 0] [--mem_notify marker|hostfunc] [--device 0] [--measure_block_time] [--noti_batch 64] [--print_ipc_latency]\n",
                  argv0);
 }
 
@@ -33,7 +35,8 @@ int main(int argc, char** argv) {
                                        {"extra_kernels", required_argument, nullptr, 'e'}, {"unfair", required_argument, nullptr, 'u'},
                                        {"sched_sleep", required_argument, nullptr, 'p'},   {"mem_notify", required_argument, nullptr, 'm'},
                                        {"device", required_argument, nullptr, 'd'},  {"measure_block_time", no_argument, nullptr, 'B'},
-                                       {"noti_batch", required_argument, nullptr, 'b'},  {nullptr, 0, nullptr, 0}};
+                                       {"noti_batch", required_argument, nullptr, 'b'},  {"print_ipc_latency", no_argument, nullptr, 'L'},
+                                       {nullptr, 0, nullptr, 0}};
     for (int c; (c = getopt_long(argc, argv, "h", long_opts, nullptr)) != -1;) {
         switch (c) {
             case 'n': name = optarg; break;
@@ -50,6 +53,7 @@ int main(int argc, char** argv) {
             case 'd': device = std::atoi(optarg); break;
             case 'B': opts.measure_block_time = true; break;
             case 'b': opts.noti_batch = (unsigned)std::strtoul(optarg, nullptr, 10); break;
+            case 'L': llis::ipc::set_launch_timestamps(true); break;
             default: usage(argv[0]); return c == 'h' ? 1 : 2;
         }
     }

@@ -7,6 +7,7 @@
 
 #include "paella_hip.h"
 
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <stdexcept>
@@ -22,10 +23,15 @@ Server::Server(std::string server_name, Scheduler* scheduler)
     if (const char* path = std::getenv("LLIS_EVENT_LOG")) {
         if (*path) event_log_.enable(true);
     }
+    if (const char* skip = std::getenv("LLIS_IPC_LATENCY_SKIP")) ipc_latency_skip_ = (unsigned)std::strtoul(skip, nullptr, 10);
     scheduler_->set_server(this);
 }
 
 Server::~Server() {
+    if (ipc_latency_count_) {
+        std::printf("Avg launch job IPC latency: %f us over %llu requests\n", ipc_latency_mean_us(), (unsigned long long)ipc_latency_count_);
+        std::fflush(stdout);
+    }
     LLIS_PHASE_REPORT();
     if (const char* path = std::getenv("LLIS_EVENT_LOG")) {
         if (*path && event_log_.enabled()) event_log_.save(path);
@@ -116,6 +122,22 @@ void Server::handle_register_job() {
 }
 
 void Server::handle_launch_job() {
+    if (ipc::launch_timestamps()) {
+        // Mean latency of the request ring (reference src/server/server.cpp:121-141): the first 10 000 requests are left out,
+        // then every 1000th prints the running mean.
+        unsigned long long sent;
+        c2s_channel_.read(&sent);
+        if (ipc_latency_skipped_ >= ipc_latency_skip_) {
+            const unsigned long long now = (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
+            ipc_latency_sum_ns_ += (double)(now - sent) * (1e9 * (double)std::chrono::steady_clock::period::num / (double)std::chrono::steady_clock::period::den);
+            if (++ipc_latency_count_ % 1000 == 0) {
+                std::printf("Avg launch job IPC latency: %f us\n", ipc_latency_mean_us());
+                std::fflush(stdout);
+            }
+        } else {
+            ++ipc_latency_skipped_;
+        }
+    }
     JobRefId id;
     c2s_channel_.read(&id);
     if (id >= registered_jobs_.size()) throw std::runtime_error("LAUNCH_JOB for an unknown job type");

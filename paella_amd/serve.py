@@ -11,7 +11,7 @@ c_int, c_uint, c_float, c_double, c_char_p, c_void_p, c_size_t = (ctypes.c_int, 
 
 class ServerOptions(ctypes.Structure):
     _fields_ = [("name", c_char_p), ("sched", c_char_p), ("num_streams", c_uint), ("extra_kernels", c_uint), ("unfair", c_float),
-                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int), ("noti_batch", c_uint)]
+                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int), ("noti_batch", c_uint), ("print_ipc_latency", c_int)]
 
 
 class LoadOptions(ctypes.Structure):
@@ -46,6 +46,8 @@ SERVE_SYMBOLS = {
     "paella_server_start": (c_int, [ctypes.POINTER(ServerOptions), ctypes.POINTER(c_void_p)]),
     "paella_server_stop": (c_int, [c_void_p]),
     "paella_server_event_log": (c_size_t, [c_void_p, c_void_p, c_size_t]),
+    "paella_server_ipc_latency": (c_int, [c_void_p, ctypes.POINTER(c_double), ctypes.POINTER(ctypes.c_uint64)]),
+    "paella_ipc_latency_off": (None, []),
     "paella_client_run": (c_int, [ctypes.POINTER(LoadOptions), ctypes.POINTER(LoadResult), c_void_p]),
     "paella_direct_multistream_run": (c_int, [ctypes.POINTER(DirectOptions), ctypes.POINTER(LoadResult)]),
     "paella_workload_pregen": (c_int, [c_double, c_int, c_double, c_uint, c_uint, c_char_p, ctypes.POINTER(c_float), c_int, c_char_p, c_size_t]),
@@ -79,9 +81,9 @@ class Server:
     """`with Server('name', 'full3', num_streams=64) as s: ...`; s.event_log() after the block."""
 
     def __init__(self, name, sched, num_streams=500, extra_kernels=2, unfair=1e6, sched_sleep=0, mem_marker=True, event_log=False,
-                 cpu=-1, measure_block_time=False, noti_batch=0):
+                 cpu=-1, measure_block_time=False, noti_batch=0, print_ipc_latency=False):
         self.opts = ServerOptions(name.encode(), sched.encode(), num_streams, extra_kernels, unfair, sched_sleep, int(mem_marker),
-                                  int(event_log), cpu, int(measure_block_time), noti_batch)
+                                  int(event_log), cpu, int(measure_block_time), noti_batch, int(print_ipc_latency))
         self.name = name
         self.handle = c_void_p()
 
@@ -92,6 +94,15 @@ class Server:
 
     def stop(self):
         lib().paella_server_stop(self.handle)
+        if self.opts.print_ipc_latency:
+            lib().paella_ipc_latency_off()
+
+    def ipc_latency(self):
+        """(mean client-to-server latency of LAUNCH_JOB in us, requests it covers); needs print_ipc_latency=True."""
+        mean, count = c_double(), ctypes.c_uint64()
+        if lib().paella_server_ipc_latency(self.handle, ctypes.byref(mean), ctypes.byref(count)) != 0:
+            raise RuntimeError("paella_server_ipc_latency failed")
+        return mean.value, count.value
 
     def __exit__(self, *exc):
         self.stop()
