@@ -18,7 +18,12 @@
 //  * request buffers in the client's shared-memory pool cannot be registered with the runtime on this
 //    platform, so both copies go through a per-instance pinned staging buffer (filled on the server
 //    thread just before the H2D copy is issued -- or, under a stage-by-stage scheduler, by a helper thread as a copy stage
-//    of its own -- and drained in on_complete()).
+//    of its own -- and drained in on_complete());
+//  * under a scheduler that issues a whole job at once (fifo), PAELLA_DISPATCH=direct puts the job's kernels, in order, on one
+//    of the operator library's direct-dispatch queues with the barrier bit set (a queue then behaves like a stream), the
+//    input upload being a copy kernel on the same queue: plain per-request stream serving on the same launch path as the
+//    stage-by-stage schedulers, so that a comparison with them is one of policy and not of launch cost.  Default there: HIP
+//    streams and launches.
 
 #include <llis/job/context.h>
 #include <llis/job/coroutine_job.h>
@@ -97,11 +102,15 @@ class ModelJob : public llis::job::CoroutineJob {
         unfit_starts_ = starts && std::strcmp(starts, "1") == 0;
         const char* dispatch = std::getenv("PAELLA_DISPATCH");
         direct_ = !(dispatch && std::strcmp(dispatch, "hip") == 0) && llis::job::Context::is_stage_by_stage();
-        if (direct_) {
+        // whole-job issue on an ordered direct queue: asked for by name, and only when no copy has to stay on the HIP stream
+        // behind the kernels (every model's output here is small enough to be written by its last kernel)
+        whole_job_direct_ = !llis::job::Context::is_stage_by_stage() && dispatch && std::strcmp(dispatch, "direct") == 0 && zero_out_ &&
+                            in_bytes_ % sizeof(float) == 0;
+        if (direct_ || whole_job_direct_) {
             void* probe = nullptr;
             if (paella_direct_queue_shared(&probe) != 0) {
                 std::fprintf(stderr, "[llis] model job: direct dispatch unavailable, using HIP launches\n");
-                direct_ = false;
+                direct_ = whole_job_direct_ = false;
             }
         }
         // Conv launches of different requests share launches (paella_pack_enable) unless PAELLA_PACK=0: the serving thread
@@ -139,7 +148,17 @@ class ModelJob : public llis::job::CoroutineJob {
                 yield();
                 std::memcpy(staging_, io_ptr, in_bytes_);
             }
-            check(llis_hip_memcpy_async(paella_exec_input(exec_), staging_, in_bytes_, LLIS_HIP_H2D, stream()), "H2D");
+            if (whole_job_direct_) {
+                // the upload as a kernel that reads the pinned staging buffer, first packet of this job on its queue (the
+                // scheduler's completion marker for the copy stage goes to the idle HIP stream and counts at once; the job
+                // ends when its last kernel's workgroups have reported)
+                check(paella_direct_queue_shared(&job_queue_), "direct queue");
+                paella_direct_queue_set_ordered(job_queue_, 1);
+                check(paella_copy_launch(reinterpret_cast<const float*>(staging_), reinterpret_cast<float*>(paella_exec_input(exec_)),
+                                         in_bytes_ / sizeof(float), job_queue_, 0, nullptr), "upload kernel");
+            } else {
+                check(llis_hip_memcpy_async(paella_exec_input(exec_), staging_, in_bytes_, LLIS_HIP_H2D, stream()), "H2D");
+            }
             unset_is_mem();
         } else if (!input_uploaded_) {
             // Measurement mode PAELLA_INPUT_RESIDENT=1: the instance's input is uploaded once, from its first
@@ -165,6 +184,13 @@ class ModelJob : public llis::job::CoroutineJob {
             const uint32_t id = get_id() | (is_unfit() && unfit_starts_ ? 0u : PAELLA_JOB_ID_NO_START) | (timed_ ? PAELLA_JOB_ID_TIME_BLOCKS : 0u);
             void* target = stream();
             if (direct_) check(paella_direct_queue_shared(&target), "direct queue");
+            if (whole_job_direct_) {
+                if (!job_queue_) {  // no upload stage came first
+                    check(paella_direct_queue_shared(&job_queue_), "direct queue");
+                    paella_direct_queue_set_ordered(job_queue_, 1);
+                }
+                target = job_queue_;
+            }
             if (pack_) enable_packing_on_this_thread();
             // members of a group wait for what is ahead of them in the queue (a stream orders by itself); the first one
             // too, so that it is not held back for packing while the others go out
@@ -178,6 +204,10 @@ class ModelJob : public llis::job::CoroutineJob {
             if (recording) check(paella_pack_sequence_end(), "end of the recorded launch sequence");
             if (direct_ && last > s) paella_direct_queue_set_ordered(target, 0);
             s = last + 1;
+        }
+        if (job_queue_) {  // the whole job is out (the scheduler drained this coroutine in one go): the queue is the next job's
+            paella_direct_queue_set_ordered(job_queue_, 0);
+            job_queue_ = nullptr;
         }
 
         if (zero_out_) return;
@@ -220,6 +250,8 @@ class ModelJob : public llis::job::CoroutineJob {
     int num_stages_ = 0;
     std::vector<int> group_end_;   // per kernel: index of the last kernel of the group it is issued with
     bool direct_ = true;
+    bool whole_job_direct_ = false;
+    void* job_queue_ = nullptr;    // whole-job issue: the ordered queue this request's kernels are going to
     bool pack_ = false;
     bool stage_off_thread_ = false;
     bool timed_ = false;

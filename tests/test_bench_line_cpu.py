@@ -37,11 +37,12 @@ def _full_result():
         "roofline": rf, "roofline_resnet18": dict(rf),
         "cpu_baseline": {"value": 19.13, "unit": "requests/s", "cores": 16, "kind": "port", "sample": "s" * 500},
         "cpu_baseline_torch": {"value": 380.4, "unit": "requests/s", "cores": 16, "kind": "port", "sample": "s" * 500},
-        "side_workloads": {"k%d" % i: {"points": [_point(j) for j in range(6)]} for i in range(8)},
+        "side_workloads": dict({"k%d" % i: {"points": [_point(j) for j in range(6)]} for i in range(8)},
+                               policy_reference_two_model_workload={"arms": {a: [dict(_point(j), resnet18_p99_us=1234.56789, inception_v3_p99_us=23456.789)
+                                                                                 for j in range(1, 4)] for a in arms[:4]}}),
         "per_op_us": {op: {"launches": 3, "us": 12.3, "gflop": 1.0, "mbytes": 2.0, "tflops": 3.0, "gbytes_per_s": 4.0} for op in ("conv", "pool", "dense", "gap")},
         "notify_us": {"ring_drain_64_blocks_us_per_kernel": 11.87, "launch_plus_flag_store_us": 6.25, "launch_plus_stream_sync_us": 9.5,
-                      "echo_round_trip_us": {"p50": 2.98, "p99": 3.29, "what": "q" * 200}, "gpu_to_host_us": {"p50": 1.4, "p99": 1.6, "what": "q" * 200}},
-        "policy": {"fig12": {a: {"resnet18_p99_us": 1234.5, "inception_v3_p99_us": 23456.7} for a in arms[:4]}},
+                      "echo_round_trip_us": {"p50": 2.98, "p99": 3.29, "what": "q" * 200}, "gpu_to_host_us": {"upper_bound_p50": 2.98, "upper_bound_p99": 3.29, "what": "q" * 200, "clock_translated": {"p50": -1.6, "p99": -1.4, "plausible": False}}},
     }
 
 
@@ -64,6 +65,5 @@ def test_headline_is_short_and_carries_the_contract():
 def test_headline_survives_an_unmet_slo_and_missing_parts():
     out = _full_result()
     out.update({"value": None, "slo_met": False, "cpu_baseline": None, "cpu_baseline_torch": None, "rate_search": {}, "notify_us": {}})
-    out.pop("policy")
     line = json.loads(bench.headline(out))
     assert line["value"] is None and line["cpu_baseline"] is None

@@ -76,10 +76,11 @@ def test_every_completion_at_saturation_is_its_own_models_answer(cuda, mix):
     expectations_match_the_oracle(models, types, r, out_bytes, seed=3)
 
 
-@pytest.mark.parametrize("sched_name,dispatch", [("fifo2", "direct"), ("fifo", "hip"), ("full3", "hip")])
+@pytest.mark.parametrize("sched_name,dispatch", [("fifo2", "direct"), ("fifo", "hip"), ("fifo", "direct"), ("full3", "hip")])
 def test_every_completion_is_checked_under_the_other_schedulers_and_launch_paths(cuda, sched_name, dispatch):
     """The two-tenant mix under open-loop Poisson arrivals near its knee through fifo2 (packed direct dispatch), fifo (whole
-    requests on HIP streams) and full3 on HIP launches."""
+    requests on HIP streams, and whole requests on ordered direct-dispatch queues with the upload as a kernel) and full3 on HIP
+    launches."""
     from paella_amd import models, serve
     os.environ["LLIS_MODEL_SEED"] = "1"
     os.environ["PAELLA_DISPATCH"] = dispatch
