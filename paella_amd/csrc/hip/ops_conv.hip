@@ -752,36 +752,54 @@ __device__ __forceinline__ float dw_window(const DwArgs& p, const float* xc, con
     return acc;
 }
 
+// One output element of a depthwise conv.
+__device__ __forceinline__ void dw_element(const DwArgs& p, int idx, int PQ) {
+    const int c = idx / PQ;
+    const int pix = idx - c * PQ;
+    const int ho = pix / p.Q;
+    const int wo = pix - ho * p.Q;
+    const float* xc = p.x + (size_t)c * p.H * p.W;
+    const float* wc = p.w + (size_t)c * p.R * p.S;
+    float acc = p.bias ? p.bias[c] : 0.f;
+    const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
+    if (p.R == 3 && p.S == 3) {
+        acc = dw_window<3, 3>(p, xc, wc, acc, h0, w0);
+    } else {
+        for (int r = 0; r < p.R; ++r) {
+            const int h = h0 + r * p.dh;
+            if ((unsigned)h >= (unsigned)p.H) continue;
+            for (int s = 0; s < p.S; ++s) {
+                const int w = w0 + s * p.dw;
+                if ((unsigned)w >= (unsigned)p.W) continue;
+                acc = fmaf(xc[(size_t)h * p.W + w], wc[r * p.S + s], acc);
+            }
+        }
+    }
+    const size_t o = (size_t)idx;
+    if (p.residual) acc += p.residual[o];
+    const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
+    store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
+}
+
+// A thread computes kDwPerThread output elements, a whole grid apart from each other (neighbouring threads still touch
+// neighbouring elements), when the launch was planned that way (grid * 256 < elements): a quarter of the workgroups for the
+// large layers, whose kernels are bound by latency and not by the arithmetic, and with them a quarter of the end messages
+// the serving thread has to read (MobileNetV2: 133 of its 254 messages per request came from seven depthwise layers).
+constexpr int kDwPerThread = 4;
+constexpr int kDwWideFrom = 65536;  // elements from which a thread takes several
+
 __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
     paella::hook_entry(p.notifier, p.job_id);
     const int PQ = p.P * p.Q;
-    const int idx = blockIdx.x * 256 + threadIdx.x;  // over (channel, pixel): small feature maps still fill their workgroups
-    if (idx < p.C * PQ) {
-        const int c = idx / PQ;
-        const int pix = idx - c * PQ;
-        const int ho = pix / p.Q;
-        const int wo = pix - ho * p.Q;
-        const float* xc = p.x + (size_t)c * p.H * p.W;
-        const float* wc = p.w + (size_t)c * p.R * p.S;
-        float acc = p.bias ? p.bias[c] : 0.f;
-        const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
-        if (p.R == 3 && p.S == 3) {
-            acc = dw_window<3, 3>(p, xc, wc, acc, h0, w0);
-        } else {
-            for (int r = 0; r < p.R; ++r) {
-                const int h = h0 + r * p.dh;
-                if ((unsigned)h >= (unsigned)p.H) continue;
-                for (int s = 0; s < p.S; ++s) {
-                    const int w = w0 + s * p.dw;
-                    if ((unsigned)w >= (unsigned)p.W) continue;
-                    acc = fmaf(xc[(size_t)h * p.W + w], wc[r * p.S + s], acc);
-                }
-            }
-        }
-        const size_t o = (size_t)idx;
-        if (p.residual) acc += p.residual[o];
-        const float sl = (p.act == PAELLA_ACT_PRELU) ? p.slope[c] : 0.f;
-        store_out(p.y + o, apply_act(acc, p.act, sl, p.lo, p.hi));
+    const int total = p.C * PQ;
+    const int stride = (int)gridDim.x * 256;
+    int idx = blockIdx.x * 256 + threadIdx.x;  // over (channel, pixel): small feature maps still fill their workgroups
+    if (stride >= total) {
+        if (idx < total) dw_element(p, idx, PQ);
+    } else {
+#pragma unroll
+        for (int k = 0; k < kDwPerThread; ++k, idx += stride)
+            if (idx < total) dw_element(p, idx, PQ);
     }
     paella::hook_exit(p.notifier, p.job_id);
 }
@@ -965,7 +983,11 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->kind = 1;
         plan->blob_bytes = (size_t)d->C * d->R * d->S * sizeof(float);
         if ((double)d->C * PQ >= 2147483648.0) return PAELLA_ENOSUP;  // output elements are indexed with 32 bits
-        plan->dims.grid = (unsigned)(((size_t)d->C * PQ + 255) / 256);
+        {
+            const size_t elements = (size_t)d->C * PQ;
+            const size_t per_group = elements >= (size_t)kDwWideFrom ? 256u * (size_t)kDwPerThread : 256u;
+            plan->dims.grid = (unsigned)((elements + per_group - 1) / per_group);
+        }
         plan->dims.block = 256;
         plan->dims.lds_bytes = 0;
         plan->dims.vgprs = 32;

@@ -227,8 +227,8 @@ def test_verify_mode_checks_every_completion(tmp_path):
                          env=fake_env(), capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr
     stats = json.loads(out.stdout.strip().splitlines()[-1])
-    # 24 warm-up runs of which 2 x 3 taught the expectations, 60 extra warm-up requests, 500 measured
-    assert stats["verified_requests"] == 24 - 6 + 60 + 500 and stats["mismatches"] == 0
+    # 24 warm-up runs one at a time, of which 2 x 3 taught the expectations, 24 more all at once, 60 extra warm-up requests, 500 measured
+    assert stats["verified_requests"] == 24 - 6 + 24 + 60 + 500 and stats["mismatches"] == 0
     assert srv.wait(timeout=30) == 0
 
 
@@ -242,8 +242,8 @@ def test_verify_mode_counts_wrong_answers(tmp_path):
                           fake_job("fake_flaky"), "1.0", "8"],
                          env=fake_env(), capture_output=True, text=True, timeout=120)
     stats = json.loads(out.stdout.strip().splitlines()[-1])
-    assert stats["verified_requests"] == 8 - 2 + 400
-    assert stats["mismatches"] == (8 + 400) // 50 and out.returncode == 3
+    assert stats["verified_requests"] == 8 - 2 + 8 + 400
+    assert stats["mismatches"] == (8 + 8 + 400) // 50 and out.returncode == 3
     assert "first differing byte 7" in out.stderr
     assert srv.wait(timeout=30) == 0
 
@@ -295,8 +295,8 @@ def test_launch_job_with_and_without_its_send_time(tmp_path, timed):
     if not timed:
         assert not lines
         return
-    # 8 warm-up runs + 2500 requests, the first 100 left out: the running mean at 1000 and 2000, the final figure on exit
-    assert len(lines) == 3 and lines[-1].endswith("over 2408 requests"), lines
+    # 8 + 8 warm-up runs + 2500 requests, the first 100 left out: the running mean at 1000 and 2000, the final figure on exit
+    assert len(lines) == 3 and lines[-1].endswith("over 2416 requests"), lines
     for l in lines:
         us = float(l.split()[5])
         assert 0.0 < us < 5000.0, l

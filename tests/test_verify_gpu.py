@@ -39,7 +39,7 @@ def run_verified(serve, models, srv, types, iat_us, n, seed, warmup=200):
                          warmup_jobs=warmup, seed=seed, verify=VARIANTS, expected_bytes=VARIANTS * sum(out_bytes))
     pools = sum(t[3] for t in types)
     assert r["all"]["count"] == n
-    assert r["verified_requests"] == pools - VARIANTS * len(types) + warmup + n, r["verified_requests"]
+    assert r["verified_requests"] == pools - VARIANTS * len(types) + pools + warmup + n, r["verified_requests"]
     return r, out_bytes
 
 
