@@ -135,8 +135,20 @@ class Job {
 
     StreamHandle get_cuda_stream() const { return cuda_stream_; }
 
-    void set_finished_block_notifier(FinishedBlockNotifier* notifier) { finished_block_notifier_ = notifier; }
-    FinishedBlockNotifier* get_finished_block_notifier() { return finished_block_notifier_; }
+    void set_finished_block_notifier(FinishedBlockNotifier* notifier) {
+        finished_block_notifier_ = notifier;
+        notifier_read_ = false;
+    }
+    FinishedBlockNotifier* get_finished_block_notifier() {
+        notifier_read_ = true;
+        return finished_block_notifier_;
+    }
+    // False after run_next() if the stage did not ask for its notifier: its kernel then reports through the un-aggregated hooks
+    // (llis/job/instrument.h), one message per workgroup that names the compute unit it ran on.  A scheduler that places
+    // workgroups per compute unit records that with set_reports_cu() and reads reports_cu() when the messages come in.
+    bool used_finished_block_notifier() const { return notifier_read_; }
+    bool reports_cu() const { return reports_cu_; }
+    void set_reports_cu(bool v) { reports_cu_ = v; }
 
     Clock::time_point get_stage_start_time() const { return stage_start_time_; }
 
@@ -168,7 +180,7 @@ class Job {
     void* get_remote_ptr() const { return remote_ptr_; }
     void set_remote_ptr(void* p) { remote_ptr_ = p; }
 
-    // Per-compute-unit placement prediction (kept for API compatibility; sized for the 8-bit cu id).
+    // Per-compute-unit placement prediction of the running stage (reference include/llis/job/job.h:179-199), sized for the 8-bit cu id.
     static constexpr unsigned kMaxCuIds = 256;
     void add_predicted_smid(unsigned smid) {
         ++predicted_smid_nums_[smid % kMaxCuIds];
@@ -217,6 +229,8 @@ class Job {
     bool has_started_ = false;
     bool is_unfit_ = false;
     bool any_predicted_ = true;
+    bool notifier_read_ = false;
+    bool reports_cu_ = false;
 
     StreamHandle cuda_stream_ = nullptr;
     FinishedBlockNotifier* finished_block_notifier_ = nullptr;

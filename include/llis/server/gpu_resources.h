@@ -49,13 +49,18 @@ class GpuResources {
     void choose_cus(job::Job* job);
 
     // A workgroup of the job's running stage reported compute unit `cu`.  Predicted there: the prediction is consumed;
-    // otherwise the compute unit is acquired now.
+    // otherwise the compute unit is acquired now.  An id beyond the topology is left out of the books (start and finish alike).
     void observe_block_start(job::Job* job, unsigned cu);
     // All workgroups of the stage have started: predictions that never came true are given back.  Returns the number
     // of mispredicted workgroups and stores the number of compute units they were predicted on; both go to the profiler.
     unsigned reconcile(job::Job* job, unsigned* wrong_cus);
     // A workgroup of the job's running stage finished on compute unit `cu`.
-    void observe_block_finish(job::Job* job, unsigned cu) { release(cu, job, 1); }
+    void observe_block_finish(job::Job* job, unsigned cu) {
+        if (cu < cus_.size()) release(cu, job, 1);
+    }
+    // `num` workgroups of the job's running stage finished and nothing says where (aggregated hooks): the prediction is all
+    // there is, so they are released where they were predicted, lowest compute unit first.
+    void release_predicted(job::Job* job, unsigned num);
 
     double dot(job::Job* job) const { return total_.dot(job); }
     double dot_normalized(job::Job* job) const { return total_.dot_normalized(job); }

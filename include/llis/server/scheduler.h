@@ -42,6 +42,10 @@ struct SchedulerOptions {
     // --noti_batch: workgroups covered by one aggregated notification (a power of two, at most 128).  0 = the
     // library's default of 64; 16 is the reference's constant (reference include/llis/job/finished_block_notifier.h:118).
     unsigned noti_batch = 0;
+    // --placement per_cu (full3): admission asks the per-compute-unit model (GpuResources: does every XCD have room for
+    // its share of the grid) instead of the pooled budget, predicts where the workgroups will land and, for kernels that
+    // report through the un-aggregated hooks, reconciles the prediction with the compute unit each message names.
+    bool per_cu_placement = false;
 };
 
 class Scheduler {
@@ -113,6 +117,9 @@ class StreamPoolScheduler : public Scheduler {
 
     SchedulerOptions options_;
     unsigned num_jobs_ = 0;
+    // Compute-unit id of the message being handled (InstrumentInfo.smid): meaningful inside handle_block_start / _finish for
+    // stages whose kernels use the un-aggregated hooks.
+    unsigned cur_smid_ = 0;
 
   private:
     static void mem_notification_callback(void* job);

@@ -11,13 +11,21 @@
 //    otherwise it may still be issued as an "unfit" kernel while fewer than `extra_kernels` such kernels
 //    are waiting to become fully resident (bounded over-subscription keeps the GPU's own queue short).
 //
+//  * With --placement per_cu the occupancy model is the per-compute-unit one (llis/server/gpu_resources.h): a kernel fits
+//    if every XCD has room for its share of the grid, its workgroups are charged to the compute units the model predicts,
+//    and for kernels that report through the un-aggregated hooks the prediction is reconciled with the compute unit every
+//    start message names (reference src/server/scheduler_full.cpp:98-121 did that for an older scheduler; the reference's
+//    full3 never got it).  Kernels with aggregated hooks are released where they were predicted.
+//
 // Policy and bookkeeping follow reference include/llis/server/scheduler_full3.h:26-269 and
 // src/server/scheduler_full3.cpp:25-478.
 
+#include <llis/server/gpu_resources.h>
 #include <llis/server/scheduler.h>
 #include <llis/server/sm_resources.h>
 
 #include <cstdint>
+#include <memory>
 #include <set>
 #include <vector>
 
@@ -75,6 +83,8 @@ class SchedulerFull3 : public StreamPoolScheduler {
     explicit SchedulerFull3(const SchedulerOptions& options);
     // For tests: an explicit occupancy budget instead of the device's.
     SchedulerFull3(const SchedulerOptions& options, const SmResources& budget);
+    // For tests: per-compute-unit placement (options.per_cu_placement) over an explicit topology instead of the device's.
+    SchedulerFull3(const SchedulerOptions& options, std::unique_ptr<GpuResources> per_cu);
 
     void set_server(Server* server) override;
     void handle_new_job(std::unique_ptr<job::Job> job) override;
@@ -91,6 +101,7 @@ class SchedulerFull3 : public StreamPoolScheduler {
 
     JobQueue job_queue_;
     SmResources gpu_resources_;
+    std::unique_ptr<GpuResources> per_cu_;   // options.per_cu_placement: admission and accounting per compute unit instead
     int num_outstanding_kernels_ = 0;
 };
 

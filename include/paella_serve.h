@@ -40,6 +40,9 @@ typedef struct paella_server_options {
     int print_ipc_latency;     /* 1: --print_ipc_latency: LAUNCH_JOB carries its send time and the server reports the request ring's mean
                                   latency (the reference's PRINT_LAUNCH_JOB_IPC_LATENCY build, reference src/server/server.cpp:121-141).  The
                                   switch is process-wide: clients of this process send the time from then on; 0 leaves it as it is */
+    int placement;             /* --placement: 0 = pooled occupancy budget (the reference's full3), 1 = per_cu: admission against the
+                                  per-compute-unit model (include/llis/server/gpu_resources.h; the reference sketches it in
+                                  include/llis/server/gpu_resources.h:10-58 and builds it into no scheduler it ships); full3 only */
 } paella_server_options;
 
 int paella_server_start(const paella_server_options* options, paella_server** out);

@@ -18,6 +18,9 @@ a job without stages is released without touching the id pool.
 Log grammar (one event per line), inputs J/B/M/L and decisions D/S/E:
   J id type unique first_is_mem | B id is_start num | M id | L id stage hexfloat
   D id stage stream notifier is_mem unfit | S id | E id
+With per-compute-unit placement (Full3(per_cu=...), this build's own: the reference's full3 has only the pooled budget; the
+reconciliation restates reference src/server/scheduler_full.cpp:98-121) a B line of a raw-hook stage carries a fourth
+value, the compute unit, and the decisions gain  R id mispredicted_workgroups compute_units.
 Pinning: hand-derived logs and closed forms in tests/test_sched_oracle.py; the JobQueue is written as a
 brute-force search over plain lists, so it doubles as the naive model for the product's tree-based queue.
 """
@@ -33,6 +36,7 @@ class Stage:
     smem: int = 0
     regs: int = 0
     pre_notify: bool = False
+    raw: bool = False   # kernel with un-aggregated hooks: one message per workgroup, naming its compute unit
 
 
 def dummy_stages(n):
@@ -46,7 +50,11 @@ FAKE_TYPES = {
     "fake_mem3": [Stage(True), Stage(False, 40, 128, 1024, 64), Stage(False, 200, 64, 0, 32), Stage(False, 17, 256, 8192, 128),
                   Stage(True, pre_notify=True)],
     "fake_big": [Stage(False, 3000, 256, 0, 64, i == 2) for i in range(3)],
+    "fake_raw": [Stage(False, 40, 256, 0, 32, raw=True), Stage(False, 300, 64, 2048, 64, raw=True), Stage(False, 17, 256, 8192, 128),
+                 Stage(False, 500, 256, 0, 32, True, raw=True)],
 }
+# dummy_raw of the real device (csrc/jobs/dummy_raw.hip)
+DUMMY_RAW = [Stage(False, 64, 256, 0, 32, raw=True), Stage(False, 300, 256, 0, 32, raw=True), Stage(False, 24, 256, 0, 32, True, raw=True)]
 
 
 @dataclass
@@ -68,6 +76,7 @@ class Job:
     stream: int = -1
     notifier: int = -1
     cur: Optional[Stage] = None
+    predicted: dict = field(default_factory=dict)   # per-compute-unit placement: {cu: workgroups predicted there}
 
     @property
     def next(self):
@@ -318,11 +327,12 @@ class Base:
 
 
 class Full3(Base):
-    def __init__(self, types, num_streams, extra_kernels=2, unfair=1e6, budget=FAKE_BUDGET):
+    def __init__(self, types, num_streams, extra_kernels=2, unfair=1e6, budget=FAKE_BUDGET, per_cu=None):
         super().__init__(types, num_streams)
         self._ever = []
         self.queue = JobQueue(unfair)
         self.res = SmResources(*budget)
+        self.per_cu = GpuResources(*per_cu) if per_cu else None   # (cus, xcds, regs, smem, threads, blocks per compute unit)
         self.extra = extra_kernels
         self.outstanding = 0
 
@@ -344,10 +354,23 @@ class Full3(Base):
         self.queue.push(job)
         self.schedule()
 
-    def block(self, job_id, is_start, num, length=None):
+    def _release_predicted(self, job, num):
+        for cu in sorted(job.predicted):
+            n = min(job.predicted[cu], num)
+            if n:
+                self.per_cu.cus[cu].release(job.cur, n)
+                job.predicted[cu] -= n
+                num -= n
+
+    def block(self, job_id, is_start, num, length=None, cu=None):
         job = self._ever[job_id]
+        names_cu = self.per_cu is not None and job.cur.raw
         if is_start:
+            if names_cu:
+                self.per_cu.observe_start(job.cur, job.predicted, cu)
             job.pending_blocks -= num
+            if job.pending_blocks == 0 and names_cu:
+                self.emit("R", job.id, *self.per_cu.reconcile(job.cur, job.predicted))
             if job.pending_blocks == 0 and job.unfit:
                 job.unfit = False
                 self.outstanding -= 1
@@ -363,7 +386,12 @@ class Full3(Base):
                 self.outstanding -= 1
             self.streams.append(job.stream)
             self.notifiers.append(job.notifier)
-        self.res.release(job.cur, num)
+        if self.per_cu is None:
+            self.res.release(job.cur, num)
+        elif names_cu:
+            self.per_cu.cus[cu].release(job.cur, 1)
+        else:
+            self._release_predicted(job, num)
         if over and not job.has_next():
             self.free_ids.append(job.id)
         self.schedule()
@@ -392,7 +420,7 @@ class Full3(Base):
             job = self.queue.top()
             st = job.next
             unfit = False
-            if not st.is_mem and not self.res.fits(st):
+            if not st.is_mem and not (self.per_cu.fits(st) if self.per_cu else self.res.fits(st)):
                 if self.outstanding >= self.extra:
                     break
                 self.outstanding += 1
@@ -404,7 +432,10 @@ class Full3(Base):
             notifier = -1
             if not st.is_mem:
                 notifier = job.notifier = self.notifiers.pop()
-                self.res.acquire(job.cur, job.cur.blocks)
+                if self.per_cu:
+                    job.predicted = self.per_cu.choose(job.cur)
+                else:
+                    self.res.acquire(job.cur, job.cur.blocks)
             self.emit("D", job.id, job.cur_stage, job.stream, notifier, int(st.is_mem), int(unfit))
             if st.pre_notify:
                 self.emit("S", job.id)
@@ -525,7 +556,7 @@ def parse_log(text):
     events = []
     for line in text.splitlines():
         f = line.split()
-        if not f or f[0] not in "JBMLDSE":
+        if not f or f[0] not in "JBMLDSER":
             continue
         if f[0] == "L":
             events.append(("L", int(f[1]), int(f[2]), float.fromhex(f[3])))
@@ -559,12 +590,15 @@ def replay(policy, types, num_streams, events, **kw):
             sched.new_job(ev[2])
         elif ev[0] == "B":
             job = sched.jobs_ever[ev[1]]
-            sched.block(ev[1], ev[2] == 1, ev[3], lambda: next_length(ev[1], job.cur_stage))
+            if len(ev) > 4:
+                sched.block(ev[1], ev[2] == 1, ev[3], lambda: next_length(ev[1], job.cur_stage), cu=ev[4])
+            else:
+                sched.block(ev[1], ev[2] == 1, ev[3], lambda: next_length(ev[1], job.cur_stage))
         elif ev[0] == "M":
             job = sched.jobs_ever[ev[1]]
             if policy == "full3":
                 sched.mem(ev[1], lambda: next_length(ev[1], job.cur_stage))
             else:
                 sched.mem(ev[1])
-    actual = [e for e in events if e[0] in "JDSE"]
+    actual = [e for e in events if e[0] in "JDSER"]
     return sched.out, actual

@@ -51,6 +51,8 @@ int paella_server_start(const paella_server_options* o, paella_server** out) {
         so.mem_marker = o->mem_marker != 0;
         so.measure_block_time = o->measure_block_time != 0;
         so.noti_batch = o->noti_batch;
+        so.per_cu_placement = o->placement == 1;
+        if (so.per_cu_placement && std::string(o->sched) != "full3") return -1;
         if (o->print_ipc_latency) llis::ipc::set_launch_timestamps(true);
         auto s = std::make_unique<paella_server>();
         s->scheduler = llis::server::SchedulerFactory::create(o->sched, so);

@@ -10,7 +10,11 @@ std::string EventLog::to_text() const {
         int n = 0;
         switch (ev.kind) {
             case 'J': n = std::snprintf(line, sizeof(line), "J %lld %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c, (long long)ev.d); break;
-            case 'B': n = std::snprintf(line, sizeof(line), "B %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c); break;
+            case 'B':
+                if (ev.d >= 0) n = std::snprintf(line, sizeof(line), "B %lld %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c, (long long)ev.d);
+                else n = std::snprintf(line, sizeof(line), "B %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c);
+                break;
+            case 'R': n = std::snprintf(line, sizeof(line), "R %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c); break;
             case 'L': n = std::snprintf(line, sizeof(line), "L %lld %lld %a\n", (long long)ev.a, (long long)ev.b, ev.x); break;
             case 'D': n = std::snprintf(line, sizeof(line), "D %lld %lld %lld %lld %lld %lld\n", (long long)ev.a, (long long)ev.b, (long long)ev.c, (long long)ev.d, (long long)ev.e, (long long)ev.x); break;
             default:  n = std::snprintf(line, sizeof(line), "%c %lld\n", ev.kind, (long long)ev.a); break;

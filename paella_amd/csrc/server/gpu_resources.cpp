@@ -82,8 +82,20 @@ void GpuResources::choose_cus(job::Job* job) {
 }
 
 void GpuResources::observe_block_start(job::Job* job, unsigned cu) {
+    if (cu >= cus_.size()) return;
     if (job->has_predicted_smid(cu)) job->dec_predicted_smid(cu);
     else acquire(cu, job, 1);
+}
+
+void GpuResources::release_predicted(job::Job* job, unsigned num) {
+    const unsigned* predicted = job->get_predicted_smid_nums();
+    for (unsigned c = 0; c < cus_.size() && num > 0; ++c) {
+        const unsigned n = predicted[c] < num ? predicted[c] : num;
+        if (n == 0) continue;
+        release(c, job, (int)n);
+        for (unsigned i = 0; i < n; ++i) job->dec_predicted_smid(c);
+        num -= n;
+    }
 }
 
 unsigned GpuResources::reconcile(job::Job* job, unsigned* wrong_cus) {

@@ -67,11 +67,14 @@ void StreamPoolScheduler::try_handle_block_start_finish() {
         LLIS_PHASE(kRing);
         const job::InstrumentInfo info = gpu2sched_channel_.read<job::InstrumentInfo>();
         job::Job* job = job_of(info.job_id);
+        cur_smid_ = info.smid;
+        // the compute unit goes into the log only where the scheduler reads it
+        const int64_t logged_cu = options_.per_cu_placement && job->reports_cu() ? (int64_t)info.smid : -1;
         if (info.is_start == 1) {
-            log_->add('B', info.job_id, 1, info.num);
+            log_->add('B', info.job_id, 1, info.num, logged_cu);
             handle_block_start(job, info.num);
         } else if (info.is_start == 0) {
-            log_->add('B', info.job_id, 0, info.num);
+            log_->add('B', info.job_id, 0, info.num, logged_cu);
             handle_block_finish(job, info.num);
         } else {
             log_->add('M', info.job_id);

@@ -71,6 +71,13 @@ job::Job* JobQueue::pop() {
 
 SchedulerFull3::SchedulerFull3(const SchedulerOptions& options) : StreamPoolScheduler(options, 409600), job_queue_(options.unfair) {
     job::Context::set_stage_by_stage(true);
+    if (options.per_cu_placement) per_cu_ = std::make_unique<GpuResources>();
+}
+
+SchedulerFull3::SchedulerFull3(const SchedulerOptions& options, std::unique_ptr<GpuResources> per_cu)
+    : StreamPoolScheduler(options, 409600), job_queue_(options.unfair), per_cu_(std::move(per_cu)) {
+    job::Context::set_stage_by_stage(true);
+    options_.per_cu_placement = true;
 }
 
 SchedulerFull3::SchedulerFull3(const SchedulerOptions& options, const SmResources& budget)
@@ -81,6 +88,7 @@ SchedulerFull3::SchedulerFull3(const SchedulerOptions& options, const SmResource
 void SchedulerFull3::set_server(Server* server) {
     Scheduler::set_server(server);
     gpu_resources_.set_profiler(profiler_);
+    if (per_cu_) per_cu_->set_profiler(profiler_);
 }
 
 double SchedulerFull3::take_priority(job::Job* job) const {
@@ -111,7 +119,15 @@ void SchedulerFull3::handle_new_job(std::unique_ptr<job::Job> owned) {
 }
 
 void SchedulerFull3::handle_block_start(job::Job* job, unsigned num) {
+    const bool names_cu = per_cu_ && job->reports_cu();
+    if (names_cu) per_cu_->observe_block_start(job, cur_smid_);
     if (job->mark_block_start(num)) return;  // some workgroups still waiting for a CU
+    if (names_cu) {
+        // every workgroup has said where it runs: predictions that did not come true are given back
+        unsigned wrong_cus = 0;
+        const unsigned wrong = per_cu_->reconcile(job, &wrong_cus);
+        log_->add('R', job->get_id(), wrong, wrong_cus);
+    }
     if (job->is_unfit()) {
         // The over-subscribed kernel is now fully resident: its credit returns and the queue may move.
         job->unset_unfit();
@@ -156,7 +172,9 @@ void SchedulerFull3::handle_block_finish(job::Job* job, unsigned num) {
         give_stream(job);
         give_notifier(job);
     }
-    gpu_resources_.release(job, (int)num);
+    if (!per_cu_) gpu_resources_.release(job, (int)num);
+    else if (job->reports_cu()) per_cu_->observe_block_finish(job, cur_smid_);
+    else per_cu_->release_predicted(job, num);
     if (stage_over && !job->has_next()) retire(job);
     schedule_job();
 }
@@ -178,7 +196,7 @@ void SchedulerFull3::schedule_job() {
         const bool is_mem = job->is_mem();
         const bool posts_itself = is_mem && job->completes_itself();  // read before run_next declares the stage after
         bool unfit = false;
-        if (!is_mem && !gpu_resources_.job_fits(job)) {
+        if (!is_mem && !(per_cu_ ? per_cu_->job_fits(job) : gpu_resources_.job_fits(job))) {
             if (num_outstanding_kernels_ >= (int)options_.extra_kernels) {
                 profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SCHED_ABORT);
                 break;  // head-of-queue blocking is intended: nothing overtakes the best job
@@ -196,7 +214,8 @@ void SchedulerFull3::schedule_job() {
         if (!is_mem) {
             notifier = take_notifier();
             job->set_finished_block_notifier(notifier_ptr((unsigned)notifier));
-            gpu_resources_.acquire(job, (int)job->get_cur_num_blocks());
+            if (per_cu_) per_cu_->choose_cus(job);
+            else gpu_resources_.acquire(job, (int)job->get_cur_num_blocks());
         }
         log_->add('D', job->get_id(), job->get_cur_stage(), stream, notifier, is_mem, unfit);
         if (job->is_pre_notify()) {
@@ -216,6 +235,8 @@ void SchedulerFull3::schedule_job() {
                 job->run_next();
             }
             if (is_mem && !posts_itself) post_mem_completion(job);
+            // a kernel stage that did not ask for its notifier reports through the un-aggregated hooks
+            if (per_cu_) job->set_reports_cu(!is_mem && !job->used_finished_block_notifier());
         }
         profiler_->record_job_event(job->get_id(), Profiler::JobEvent::KERNEL_SUBMIT_END);
     }

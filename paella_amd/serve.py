@@ -11,7 +11,8 @@ c_int, c_uint, c_float, c_double, c_char_p, c_void_p, c_size_t = (ctypes.c_int, 
 
 class ServerOptions(ctypes.Structure):
     _fields_ = [("name", c_char_p), ("sched", c_char_p), ("num_streams", c_uint), ("extra_kernels", c_uint), ("unfair", c_float),
-                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int), ("noti_batch", c_uint), ("print_ipc_latency", c_int)]
+                ("sched_sleep", c_uint), ("mem_marker", c_int), ("event_log", c_int), ("cpu", c_int), ("measure_block_time", c_int), ("noti_batch", c_uint), ("print_ipc_latency", c_int),
+                ("placement", c_int)]
 
 
 class LoadOptions(ctypes.Structure):
@@ -81,9 +82,10 @@ class Server:
     """`with Server('name', 'full3', num_streams=64) as s: ...`; s.event_log() after the block."""
 
     def __init__(self, name, sched, num_streams=500, extra_kernels=2, unfair=1e6, sched_sleep=0, mem_marker=True, event_log=False,
-                 cpu=-1, measure_block_time=False, noti_batch=0, print_ipc_latency=False):
+                 cpu=-1, measure_block_time=False, noti_batch=0, print_ipc_latency=False, placement="pooled"):
         self.opts = ServerOptions(name.encode(), sched.encode(), num_streams, extra_kernels, unfair, sched_sleep, int(mem_marker),
-                                  int(event_log), cpu, int(measure_block_time), noti_batch, int(print_ipc_latency))
+                                  int(event_log), cpu, int(measure_block_time), noti_batch, int(print_ipc_latency),
+                                  {"pooled": 0, "per_cu": 1}[placement])
         self.name = name
         self.handle = c_void_p()
 

@@ -6,7 +6,8 @@
 // callback, copy).  An operation executes when the test says so (fake_hip_step*) or, with
 // FAKE_HIP_AUTORUN=1, on a background thread that always runs the oldest issued operation that is at the
 // head of its stream.  Executing a kernel means posting exactly the messages the aggregated workgroup hooks
-// post: ceil(n/B) start messages then ceil(n/B) end messages (full batches of B = noti_batch_size first, remainder last).
+// post: ceil(n/B) start messages then ceil(n/B) end messages (full batches of B = noti_batch_size first, remainder last);
+// a raw-hook kernel (fake_hip_raw_kernel_launch) posts one start and one end message per workgroup with a compute-unit id.
 
 #include "paella_hip.h"
 
@@ -34,6 +35,8 @@ struct Op {
     uint64_t seq;
     uint32_t job_id = 0;
     unsigned nblocks = 0;
+    bool raw = false;       // kernel with un-aggregated hooks: one message per workgroup, naming a compute unit
+    unsigned first_xcd = 0; // raw kernels: XCD of workgroup 0
     int phase = 0;  // kernels: 0 = not started, 1 = start messages posted
     uint64_t message = 0;
     uint64_t* slots = nullptr;
@@ -64,10 +67,36 @@ void post(uint8_t is_start, unsigned num, uint32_t job_id) {
 
 unsigned g_batch = llis::job::FinishedBlockNotifier::noti_batch_size;
 
+// Where the scripted device runs workgroup i of a raw-hook kernel: XCDs take turns from where the last raw kernel stopped
+// (as on the real part); inside the XCD a fixed scatter that knows nothing of what is resident -- so an occupancy model's
+// predictions hold for the XCD and often miss the compute unit.
+unsigned g_raw_next_xcd = 0;
+
+unsigned raw_cu(const struct Op& op, unsigned i);
+
+void post_raw(uint8_t is_start, const struct Op& op);
+
 void post_batches(uint8_t is_start, unsigned n, uint32_t job_id) {
     const unsigned B = g_batch;
     for (unsigned i = 0; i < n / B; ++i) post(is_start, B, job_id);
     if (n % B) post(is_start, n % B, job_id);
+}
+
+unsigned raw_cu(const Op& op, unsigned i) {
+    const unsigned xcd = (op.first_xcd + i) % 8;
+    const unsigned in_xcd = (i / 8 * 5 + (unsigned)(op.seq % 7) * 3) % 32;
+    return xcd * 32 + in_xcd;
+}
+
+void post_raw(uint8_t is_start, const Op& op) {
+    for (unsigned i = 0; i < op.nblocks; ++i) {
+        llis::job::InstrumentInfo info;
+        info.is_start = is_start;
+        info.smid = (uint8_t)raw_cu(op, i);
+        info.num = 1;
+        info.job_id = op.job_id;
+        llis::job::Context::get_gpu2sched_channel()->write(info);
+    }
 }
 
 // Advances the head operation of `s` by one phase (full = run it to completion).  Caller holds g_mtx,
@@ -78,11 +107,18 @@ bool advance(Stream* s, bool full, std::unique_lock<std::mutex>& lk) {
     switch (op.kind) {
         case OP_KERNEL:
             if (op.phase == 0) {
-                post_batches(1, op.nblocks, op.job_id);
+                if (op.raw) {
+                    op.first_xcd = g_raw_next_xcd;
+                    g_raw_next_xcd = (g_raw_next_xcd + op.nblocks) % 8;
+                    post_raw(1, op);
+                } else {
+                    post_batches(1, op.nblocks, op.job_id);
+                }
                 op.phase = 1;
                 if (!full) return true;
             }
-            post_batches(0, op.nblocks, op.job_id);
+            if (op.raw) post_raw(0, op);
+            else post_batches(0, op.nblocks, op.job_id);
             break;
         case OP_MARKER: {
             unsigned old = __atomic_load_n(op.cursor, __ATOMIC_RELAXED);
@@ -152,6 +188,16 @@ int fake_hip_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks) {
     Op op{OP_KERNEL, 0};
     op.job_id = job_id;
     op.nblocks = nblocks;
+    enqueue(stream, op);
+    return 0;
+}
+
+// A kernel whose workgroups report one by one through the un-aggregated hooks.
+int fake_hip_raw_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks) {
+    Op op{OP_KERNEL, 0};
+    op.job_id = job_id;
+    op.nblocks = nblocks;
+    op.raw = true;
     enqueue(stream, op);
     return 0;
 }

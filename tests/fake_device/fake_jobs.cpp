@@ -7,6 +7,8 @@
 //   FAKE_VARIANT 4  fake_self  : a copy stage that reports its own completion (from a thread of its own after 300 us when
 //                                FAKE_SELF_THREAD=1, else before it returns), copy, kernel of 40, copy(pre-notify); output = input + 1
 //   FAKE_VARIANT 5  fake_flaky : fake_mem3 whose every FAKE_FLAKY_EVERY-th run (counted over the process) answers with one wrong byte
+//   FAKE_VARIANT 6  fake_raw   : kernels of 40 and 300 workgroups with un-aggregated hooks, one of 17 with aggregated hooks, one of 500
+//                                with un-aggregated hooks (pre-notify)
 
 #include <llis/job/context.h>
 #include <llis/job/coroutine_job.h>
@@ -20,6 +22,7 @@
 #include <unistd.h>
 
 extern "C" int fake_hip_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks);
+extern "C" int fake_hip_raw_kernel_launch(void* stream, uint32_t job_id, unsigned nblocks);
 
 #ifndef FAKE_VARIANT
 #error "define FAKE_VARIANT"
@@ -43,7 +46,19 @@ class FakeJob : public llis::job::CoroutineJob {
         set_num_registers_per_thread(regs);
         if (pre_notify) set_pre_notify();
         yield();
+        (void)get_finished_block_notifier();  // a real kernel with aggregated hooks takes it as an argument
         fake_hip_kernel_launch(reinterpret_cast<void*>(get_cuda_stream()), get_id(), blocks);
+    }
+
+    void raw_kernel(unsigned blocks, unsigned threads, unsigned smem, unsigned regs, bool pre_notify) {
+        unset_is_mem();
+        set_num_blocks(blocks);
+        set_num_threads_per_block(threads);
+        set_smem_size_per_block(smem);
+        set_num_registers_per_thread(regs);
+        if (pre_notify) set_pre_notify();
+        yield();
+        fake_hip_raw_kernel_launch(reinterpret_cast<void*>(get_cuda_stream()), get_id(), blocks);
     }
 
     void body(void* io_ptr) override {
@@ -98,6 +113,11 @@ class FakeJob : public llis::job::CoroutineJob {
         set_pre_notify();
         yield();
         llis_hip_memcpy_async(reinterpret_cast<char*>(io_ptr) + 100, buf_, 100, LLIS_HIP_D2H, reinterpret_cast<void*>(get_cuda_stream()));
+#elif FAKE_VARIANT == 6
+        raw_kernel(40, 256, 0, 32, false);
+        raw_kernel(300, 64, 2048, 64, false);
+        kernel(17, 256, 8192, 128, false);
+        raw_kernel(500, 256, 0, 32, true);
 #else
         for (int i = 0; i < 3; ++i) kernel(3000, 256, 0, 64, i == 2);
 #endif

@@ -3,6 +3,7 @@
 // stdin, prints replies and finally the scheduler's event log on stdout.
 //
 //   sched NAME streams N [extra K] [unfair X] [mem marker|hostfunc] [budget REGS SMEM THREADS BLOCKS] [batch B]
+//         [percu CUS XCDS REGS SMEM THREADS BLOCKS]   full3 with per-compute-unit placement over that topology
 //   client                      register a client                      -> "client ID"
 //   job PATH                    register a job type, grow its pool     -> "job TYPE"
 //   launch TYPE [SLOT]          LAUNCH_JOB for slot SLOT of the pool
@@ -133,8 +134,8 @@ int main() {
             in >> name;
             server::SchedulerOptions opt;
             opt.ring_slots = 4096;
-            bool have_budget = false;
-            long long b[4] = {0, 0, 0, 0};
+            bool have_budget = false, have_percu = false;
+            long long b[4] = {0, 0, 0, 0}, pc[6] = {0, 0, 0, 0, 0, 0};
             while (in >> key) {
                 if (key == "streams") in >> opt.num_streams;
                 else if (key == "extra") in >> opt.extra_kernels;
@@ -142,8 +143,12 @@ int main() {
                 else if (key == "mem") { std::string m; in >> m; opt.mem_marker = (m == "marker"); }
                 else if (key == "batch") { in >> opt.noti_batch; fake_hip_set_batch(opt.noti_batch); }
                 else if (key == "budget") { in >> b[0] >> b[1] >> b[2] >> b[3]; have_budget = true; }
+                else if (key == "percu") { in >> pc[0] >> pc[1] >> pc[2] >> pc[3] >> pc[4] >> pc[5]; have_percu = true; }
             }
-            if (have_budget && name == "full3") h.scheduler = std::make_unique<server::SchedulerFull3>(opt, server::SmResources(b[0], b[1], b[2], b[3]));
+            if (have_percu && name == "full3")
+                h.scheduler = std::make_unique<server::SchedulerFull3>(
+                    opt, std::make_unique<server::GpuResources>((unsigned)pc[0], (unsigned)pc[1], pc[2], pc[3], pc[4], pc[5]));
+            else if (have_budget && name == "full3") h.scheduler = std::make_unique<server::SchedulerFull3>(opt, server::SmResources(b[0], b[1], b[2], b[3]));
             else h.scheduler = server::SchedulerFactory::create(name, opt);
             h.server = std::make_unique<server::Server>(h.server_name, h.scheduler.get());
             h.server->get_event_log()->enable(true);

@@ -125,3 +125,43 @@ def test_reference_notification_batch_reaches_the_scheduler_in_sixteens():
         per_stage = [16] * 187 + [8]
         assert len(nums) % 188 == 0 and nums == per_stage * (len(nums) // 188)
     assert [r for r in replies if r.startswith("done")] == ["done 4000"]
+
+
+# ---- per-compute-unit placement (--placement per_cu)
+
+PER_CU = (256, 8, 131072, 163840, 2048, 32)   # the scripted device's topology: compute units, XCDs, and per compute unit registers, LDS, threads, workgroups
+RAW_TYPES = ["fake_mem3", "fake_raw", "fake_big"]
+RAW_MIX = "launch 1 0\nlaunch 0 0\nstep 3\nlaunch 1 1\nlaunch 2 0\nstep 4\nlaunch 0 1\nlaunch 1 2\ndrain\n"
+
+
+@pytest.mark.parametrize("streams", [2, 8])
+def test_per_cu_placement_matches_oracle_and_reports_mispredictions(streams):
+    """full3 admitting against the per-compute-unit model: jobs with aggregated hooks are charged and released where the
+    model predicted them, jobs with un-aggregated hooks (fake_raw: every message names a compute unit, and the scripted
+    device scatters workgroups inside an XCD in its own way) are reconciled -- one R record per raw-hook kernel with the
+    number of workgroups predicted elsewhere.  Every decision, every R record and the compute units in the log replay
+    through the oracle's GpuResources."""
+    replies, events = check("full3", streams, RAW_MIX, extra="extra 2 percu %d %d %d %d %d %d" % PER_CU, types=RAW_TYPES, per_cu=PER_CU, extra_kernels=2)
+    assert len([r for r in replies if r.startswith("done")]) == 6
+    recon = [e for e in events if e[0] == "R"]
+    assert len(recon) == 3 * 3                                # three raw-hook kernels in each of three fake_raw requests
+    assert any(e[2] > 0 for e in recon) and all(e[2] <= 500 and e[3] <= 256 for e in recon)
+    raw_msgs = [e for e in events if e[0] == "B" and len(e) > 4]
+    assert len(raw_msgs) == 3 * 2 * (40 + 300 + 500)          # a start and an end message per workgroup, each with its compute unit
+    assert any(e[0] == "D" and e[6] == 1 for e in events)     # fake_big (3000 workgroups of 4 waves) never fits: credit path taken
+
+
+def test_per_cu_model_admits_by_the_share_of_each_xcd():
+    """One workgroup per compute unit: an XCD of 32 compute units takes 32.  fake_raw's 40 workgroups (5 per XCD) fit, its
+    300 (38 per XCD) do not and go out on credit; with two per compute unit (64 per XCD) they fit, and so do the 500 (63)."""
+    tight = (256, 8, 1 << 30, 1 << 30, 1 << 30, 1)
+    _, events = check("full3", 4, "launch 1 0\ndrain\n", extra="extra 1 percu %d %d %d %d %d %d" % tight, types=RAW_TYPES, per_cu=tight, extra_kernels=1)
+    assert [e[6] for e in events if e[0] == "D"] == [0, 1, 0, 1]
+    roomy = (256, 8, 1 << 30, 1 << 30, 1 << 30, 2)
+    _, events = check("full3", 4, "launch 1 0\ndrain\n", extra="extra 1 percu %d %d %d %d %d %d" % roomy, types=RAW_TYPES, per_cu=roomy, extra_kernels=1)
+    assert [e[6] for e in events if e[0] == "D"] == [0, 0, 0, 0]
+
+
+def test_raw_hook_jobs_under_the_pooled_budget_log_no_compute_units():
+    _, events = check("full3", 4, "launch 1 0\nlaunch 0 0\ndrain\n", types=RAW_TYPES)
+    assert all(len(e) == 4 for e in events if e[0] == "B") and not any(e[0] == "R" for e in events)

@@ -214,3 +214,33 @@ def test_occupancy_closed_form_in_gfx950_units():
     assert sched.wg_charge(sched.Stage(False, 3, 10, 100, 20)) == (64 * 24, 1280, 64)
     r = sched.SmResources(64 * 24 * 3, 1280 * 3, 64 * 3, 3)
     assert r.fits(sched.Stage(False, 3, 10, 100, 20)) and not r.fits(sched.Stage(False, 3, 10, 100, 25))
+
+
+def test_per_cu_placement_hand_derived_reconciliation():
+    """Two XCDs of two compute units, one workgroup of 64 threads each.  A raw-hook kernel of 4 workgroups: the model sends
+    workgroup 0 to XCD 0 (compute unit 0: ties go to the search pointer), 1 to XCD 1 (unit 2), 2 to XCD 0 (unit 1, the pointer
+    has moved on), 3 to XCD 1 (unit 3).  The device reports 0, 2, 0, 3: the second report of unit 0 was not predicted, the
+    prediction for unit 1 never came true -> one mispredicted workgroup on one compute unit; unit 0 then holds two, unit 1
+    none.  A second kernel of 3 workgroups starts on XCD 0 again (4 mod 2) and no longer fits: XCD 0 has one free slot for
+    a share of two."""
+    topo = (4, 2, 1 << 20, 1 << 20, 64, 4)
+    st4 = sched.Stage(False, 4, 64, 0, 16, raw=True)
+    g = sched.GpuResources(*topo)
+    assert g.fits(st4)
+    pred = g.choose(st4)
+    assert pred == {0: 1, 2: 1, 1: 1, 3: 1}
+    for cu in (0, 2, 0, 3):
+        g.observe_start(st4, pred, cu)
+    assert g.reconcile(st4, pred) == (1, 1)
+    assert [r.free[2] for r in g.cus] == [64 - 128, 64, 0, 0]
+    st3 = sched.Stage(False, 3, 64, 0, 16, raw=True)
+    assert g.next_xcd == 0 and not g.fits(st3)
+    # the whole path through the policy: the same kernel as a one-stage job, messages as above
+    f = sched.Full3([[sched.Stage(False, 4, 64, 0, 16, True, raw=True)]], 2, per_cu=topo)
+    f.new_job(0)
+    for cu in (0, 2, 0, 3):
+        f.block(0, True, 1, cu=cu)
+    for i, cu in enumerate((0, 2, 0, 3)):
+        f.block(0, False, 1, length=lambda: 5.0, cu=cu)
+    assert f.out == [("J", 0, 0, 0, 0), ("D", 0, 0, 1, 1, 0, 0), ("S", 0), ("R", 0, 1, 1), ("E", 0)]
+    assert all(r.free == [1 << 20, 1 << 20, 64, 4] for r in f.per_cu.cus)   # everything given back

@@ -353,3 +353,54 @@ def test_stream_order_independence_of_results(cuda):
             hip.llis_hip_stream_destroy(s)
         lib.paella_ring_destroy(ring)
         ex.close()
+
+
+def device_topology():
+    from paella_amd import _abi
+    caps = _abi.DeviceCaps()
+    _abi.check(_abi.hip().llis_hip_get_device_caps(ctypes.byref(caps)))
+    return (caps.num_cus, 8 if caps.num_cus % 8 == 0 else 1, caps.vgprs_per_cu, caps.lds_bytes_per_cu, caps.max_threads_per_cu, caps.max_blocks_per_cu)
+
+
+def test_per_cu_placement_on_the_device_replays_and_fills_the_mis_alloc_record(cuda, tmp_path):
+    """--placement per_cu under full3 with a raw-hook job (dummy_raw: kernels of 64, 300 and 24 workgroups whose every
+    message names the compute unit it ran on) next to an aggregated-hook job (dummy_10): the event log -- with the compute
+    units the hardware reported -- replays through the oracle's per-compute-unit model decision for decision, one R record
+    per raw-hook kernel, and the profiler's kernel_block_mis_alloc file holds the same figures for the measured phase."""
+    from paella_amd import serve
+    streams, n = 8, 12
+    prof = str(tmp_path / "pc")
+    with serve.Server(server_name("percu"), "full3", num_streams=streams, event_log=True, placement="per_cu") as srv:
+        r = serve.client_run(srv.name, [(serve.job_path("dummy_raw"), 0.6, 3), (serve.job_path("dummy_10"), 0.4, 2)], 2000.0, 4, n, seed=5,
+                             profile_prefix=prof)
+    assert r["all"]["count"] == n
+    events = sched.parse_log(srv.event_log())
+    topo = device_topology()
+    expected, actual = sched.replay("full3", [sched.DUMMY_RAW, sched.dummy_stages(10)], streams, events, per_cu=topo)
+    assert expected == actual, next((i, a, b) for i, (a, b) in enumerate(zip(expected + [None], actual + [None])) if a != b)
+    recon = [e for e in events if e[0] == "R"]
+    raw_jobs = sum(1 for e in events if e[0] == "J" and e[2] == 0)
+    assert len(recon) == 3 * raw_jobs and raw_jobs >= 3 + 2            # warm-up runs of the three pooled instances and some of the n
+    cus = [e[4] for e in events if e[0] == "B" and len(e) > 4]
+    assert len(cus) == 2 * (64 + 300 + 24) * raw_jobs and max(cus) < topo[0]
+    rows = [tuple(int(v) for v in l.split()) for l in open(prof + "_kernel_block_mis_alloc.txt")]
+    assert rows, "kernel_block_mis_alloc must not be empty under per_cu placement with a raw-hook job"
+    assert all(total in (64, 300, 24) and wrong <= total and wrong_cus <= min(wrong, topo[0]) for total, wrong, wrong_cus in rows)
+    # the file covers the measured phase: its rows are the tail of the log's R records
+    assert [(w, c) for _, w, c in rows] == [(e[2], e[3]) for e in recon][-len(rows):]
+    # how good the prediction is on this part: the XCD is right by construction, the compute unit inside it often is not
+    by_grid = {}
+    for total, wrong, _ in rows:
+        by_grid.setdefault(total, []).append(wrong / total)
+    print("mispredicted share of workgroups by grid size:", {k: round(sum(v) / len(v), 3) for k, v in sorted(by_grid.items())})
+
+
+def test_per_cu_placement_serves_models_with_correct_outputs(cuda):
+    """The aggregated-hook path under per_cu placement (charged and released where predicted): ResNet-18 and the small CNN
+    under load with every output checked."""
+    from paella_amd import serve
+    os.environ["LLIS_MODEL_SEED"] = "1"
+    with serve.Server(server_name("percu_models"), "full3", num_streams=32, extra_kernels=8, placement="per_cu") as srv:
+        r = serve.client_run(srv.name, [(serve.job_path("tvm_mnist"), 0.8, 16), (serve.job_path("tvm_resnet18"), 0.2, 8)], 0.0, 24, 1500,
+                             warmup_jobs=100, seed=1, verify=2)
+    assert r["all"]["count"] == 1500 and r["mismatches"] == 0 and r["verified_requests"] >= 1500
