@@ -528,7 +528,7 @@ def main():
         print(json.dumps({"zoo_ops": table}), flush=True)
         return
     if args.overlap_probe:
-        lib = _abi.ops()
+        lib = _abi.probes()
         out = {}
         log("[bench] four matrix instructions + N multiply-adds per iteration, eight waves per SIMD, register-resident (paella_mfma_valu_overlap_probe)")
         log("[bench] %4s %12s %14s %10s" % ("N", "both, us", "vector alone", "TFLOP/s"))
@@ -555,7 +555,7 @@ def main():
             row = []
             for label, per, nq, ordered in cases:
                 us = ctypes.c_double()
-                _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 16, per, nq, ordered, 200, ctypes.byref(us)), "paella_queue_concurrency_probe")
+                _abi.check(_abi.probes().paella_queue_concurrency_probe(ctypes.byref(d), 16, per, nq, ordered, 200, ctypes.byref(us)), "paella_queue_concurrency_probe")
                 row.append(us.value)
             out[name] = dict(zip([c[0] for c in cases], row))
             log("[bench] %-34s " % name + " ".join("%24.2f" % v for v in row))
@@ -796,10 +796,10 @@ def main():
         except RuntimeError as ex:
             log("[bench]   direct-dispatch queues unavailable: %s" % ex)
     peak = ctypes.c_double()
-    if lib.paella_mfma_peak_probe(ctypes.byref(peak)) == 0:
+    if _abi.probes().paella_mfma_peak_probe(ctypes.byref(peak)) == 0:
         roofline["peak_measured"] = peak.value  # register-resident fp32 MFMA loop on this box; `peak` stays the published figure
     floor = ctypes.c_double()
-    if lib.paella_empty_kernel_probe(200, ctypes.byref(floor)) == 0 and floor.value > 0:
+    if _abi.probes().paella_empty_kernel_probe(200, ctypes.byref(floor)) == 0 and floor.value > 0:
         # what the same time stamps report for a kernel that does nothing: every per-launch figure taken this way contains it
         roofline["empty_kernel_us"] = floor.value
     notify = {}

@@ -211,6 +211,13 @@ class ShmChannelWriter : public ShmChannelBase<for_gpu> {
         write(&value, sizeof(T));
     }
 
+    // True if write() of `size` bytes would return without waiting for the reader.
+    bool has_room(size_t size) {
+        this->my_read_ = this->load_pos(this->read_pos_);
+        const size_t used = this->my_write_ >= this->my_read_ ? this->my_write_ - this->my_read_ : this->size_ - this->my_read_ + this->my_write_;
+        return this->size_ - 1 - used >= size;
+    }
+
     void write(const std::string& str) {
         write(str.size());
         write(str.data(), str.size());

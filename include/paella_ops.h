@@ -109,9 +109,15 @@ int paella_conv2d_launch(const paella_conv_plan* plan, const float* x, const voi
  * stream, not a direct-dispatch queue (PAELLA_ENOSUP); all calls on one GPU share the one array, so two calls that may
  * overlap in time on that GPU (different streams, no dependency between them) race -- serialise them.  Every call
  * first zeroes the counters it will use with a small fill kernel on `stream` (the array keeps whatever the last
- * call, or an interrupted one, left behind). */
+ * call, or an interrupted one, left behind); arguments are checked before that kernel goes out, so a refused call launches
+ * nothing.  The first use on a GPU looks up that GPU's copy of the array (a runtime call that may load the code object: not
+ * for a stream under capture): call paella_conv2d_static_init() once per GPU, with that GPU current, before capturing, or
+ * make the first paella_conv2d_launch_static call there outside capture.  paella_conv2d_static_workspace() hands out the
+ * array's device address on the current GPU (diagnostics and tests: what is in it between calls is the library's). */
 #define PAELLA_CONV_STATIC_WORKSPACE_BYTES (4u << 20)
 #define PAELLA_ETOOBIG (-4)  /* the request exceeds a fixed capacity of the library */
+int paella_conv2d_static_init(void);
+int paella_conv2d_static_workspace(void** ptr);
 int paella_conv2d_launch_static(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
                                 const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
                                 void* notifier);

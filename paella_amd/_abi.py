@@ -111,6 +111,8 @@ OPS_SYMBOLS = {
     "paella_kernel_vgprs": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
     "paella_conv_kernel_vgprs": (c_int, [c_int] * 4 + [ctypes.POINTER(c_uint)]),
     "paella_conv2d_launch_static": (c_int, [ctypes.POINTER(ConvPlan)] + [c_void_p] * 6 + _TAIL),
+    "paella_conv2d_static_init": (c_int, []),
+    "paella_conv2d_static_workspace": (c_int, [ctypes.POINTER(c_void_p)]),
     "paella_kernel_occupancy": (c_int, [c_char_p, c_uint, c_uint, ctypes.POINTER(c_int)]),
     "paella_conv_kernel_occupancy": (c_int, [c_int] * 6 + [c_uint, ctypes.POINTER(c_int), ctypes.POINTER(c_uint), ctypes.POINTER(c_uint)]),
     "paella_kernel_static_lds": (c_int, [c_char_p, ctypes.POINTER(c_uint)]),
@@ -136,8 +138,12 @@ RING_SYMBOLS = {
     "paella_ring_drain": (c_size_t, [c_void_p, c_void_p, c_size_t, c_double]),
     "paella_ring_bench_drain": (c_int, [c_void_p, c_uint, c_uint, c_int, c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_pingpong": (c_int, [c_int, c_int, ctypes.POINTER(c_double), ctypes.POINTER(c_double), c_void_p]),
-    "paella_empty_kernel_probe": (c_int, [c_int, ctypes.POINTER(c_double)]),
     "paella_ring_bench_echo": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
+}
+
+# libpaella_probes.so (include/paella_probes.h): measurement only, loaded by the bench and the tests
+PROBE_SYMBOLS = {
+    "paella_empty_kernel_probe": (c_int, [c_int, ctypes.POINTER(c_double)]),
     "paella_mfma_peak_probe": (c_int, [ctypes.POINTER(c_double)]),
     "paella_mfma_valu_overlap_probe": (c_int, [c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "paella_queue_concurrency_probe": (c_int, [ctypes.POINTER(ConvDesc), c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_double)]),
@@ -170,6 +176,8 @@ def load(name):
         _bind(lib, RING_SYMBOLS)
         from . import _abi_models
         _abi_models.bind(lib)
+    elif name == "paella_probes":
+        _bind(lib, PROBE_SYMBOLS)
     _cache[name] = lib
     return lib
 
@@ -181,6 +189,11 @@ def hip():
 def ops():
     hip()
     return load("paella_ops")
+
+
+def probes():
+    ops()
+    return load("paella_probes")
 
 
 def check(rc, what=""):

@@ -1264,6 +1264,7 @@ bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n
 int pack_send(PackList& list, int kw, int k_order, bool only_full) {
     int launches = 0;
     size_t done = 0;
+    bool failed = false;
     while (done < list.items.size()) {
         if (only_full && list.members < kPackMax) break;
         ConvGroupArgs g;
@@ -1294,8 +1295,11 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
             ++n;
         }
         void* target = nullptr;
-        if (paella_direct_queue_shared(&target) != 0) return -1;
-        int rc;
+        int rc = paella_direct_queue_shared(&target) != 0 ? -1 : 0;
+        if (rc != 0) {
+            failed = true;
+            break;
+        }
         if (n == 1) {  // nothing to share the launch with: the plain kernel, whose argument block is a quarter of the group's
             ConvKernel kern = pick_kernel(1, 1, kw, k_order);
             g.m[0].conv.hook_blocks = 0;
@@ -1307,7 +1311,10 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         } else {
             rc = launch_group_args(g, n, kw, k_order, grid, dyn_lds, target);
         }
-        if (rc != 0) return -1;
+        if (rc != 0) {
+            failed = true;
+            break;
+        }
         ++launches;
         g_pack_launches.fetch_add(1, std::memory_order_relaxed);
         g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
@@ -1315,8 +1322,9 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         g_pack.held -= (int)(i - done);
         done = i;
     }
+    // what went out leaves the list on every path: a failed launch must not send its predecessors again on the next turn
     list.items.erase(list.items.begin(), list.items.begin() + (long)done);
-    return launches;
+    return failed ? -1 : launches;
 }
 
 unsigned units_to_grid(const SeqRecord& r) {
@@ -1365,29 +1373,35 @@ int seq_send_batch(const std::vector<Sequence>& seqs, size_t first, int n, void*
     const bool was_ordered = paella::direct_queue_ordered(q);
     paella_direct_queue_set_ordered(target, 1);
     int launches = 0;
-    for (size_t k = 0; k < seqs[first].recs.size(); ++k) {
-        if (seq_launch_position(seqs, first, n, k, target) != 0) return -1;
-        ++launches;
+    bool failed = false;
+    for (size_t k = 0; k < seqs[first].recs.size() && !failed; ++k) {
+        if (seq_launch_position(seqs, first, n, k, target) != 0) failed = true;
+        else ++launches;
     }
-    if (!was_ordered) paella_direct_queue_set_ordered(target, 0);
-    return launches;
+    if (!was_ordered) paella_direct_queue_set_ordered(target, 0);   // on every path: the queue is shared
+    return failed ? -1 : launches;
 }
 
 int seq_send(SeqList& list, bool only_full) {
     int launches = 0;
     size_t done = 0;
+    bool failed = false;
     while (done < list.seqs.size()) {
         const size_t left = list.seqs.size() - done;
         if (only_full && left < (size_t)kPackMax) break;
         const int n = (int)std::min<size_t>(left, (size_t)kPackMax);
         const int r = seq_send_batch(list.seqs, done, n, nullptr);
-        if (r < 0) return -1;
-        launches += r;
+        // a batch that failed part of the way is gone too: its first launches are on the queue and cannot be sent again
         done += (size_t)n;
         g_pack.held -= n;
+        if (r < 0) {
+            failed = true;
+            break;
+        }
+        launches += r;
     }
     list.seqs.erase(list.seqs.begin(), list.seqs.begin() + (long)done);
-    return launches;
+    return failed ? -1 : launches;
 }
 
 bool same_signature(const Sequence& a, const Sequence& b) {
@@ -1512,7 +1526,14 @@ extern "C" int paella_pack_poll(void) {
     return pack_send_all(true);
 }
 
-extern "C" void paella_pack_poll_hook(void) { (void)paella_pack_poll(); }
+extern "C" void paella_pack_poll_hook(void) {
+    // Held launches that cannot be sent leave their requests without completion messages for good: nothing the serving loop
+    // could do about it but stop, loudly.
+    if (paella_pack_poll() < 0) {
+        std::fprintf(stderr, "[paella] launch packing: held launches could not be sent\n");
+        std::abort();
+    }
+}
 
 extern "C" int paella_pack_stats(uint64_t* launches, uint64_t* members) {
     if (launches) *launches = g_pack_launches.load(std::memory_order_relaxed);
@@ -1693,15 +1714,32 @@ int static_workspace(void** out) {
 
 }  // namespace
 
+extern "C" int paella_conv2d_static_init(void) {
+    void* ws = nullptr;
+    return static_workspace(&ws);
+}
+
+extern "C" int paella_conv2d_static_workspace(void** ptr) {
+    if (!ptr) return PAELLA_EINVAL;
+    return static_workspace(ptr);
+}
+
 extern "C" int paella_conv2d_launch_static(const paella_conv_plan* plan, const float* x, const void* blob_dev, const float* bias,
                                            const float* residual, const float* slope, float* y, void* stream, uint32_t job_id,
                                            void* notifier) {
-    if (!plan) return PAELLA_EINVAL;
+    if (!plan || !x || !blob_dev || !y) return PAELLA_EINVAL;
+    if (plan->d.act == PAELLA_ACT_PRELU && !slope) return PAELLA_EINVAL;
     if (plan->workspace_bytes > PAELLA_CONV_STATIC_WORKSPACE_BYTES) return PAELLA_ETOOBIG;
     if (paella::direct_queue_lookup(stream)) return PAELLA_ENOSUP;  // the counter fill below needs stream order
     void* ws = nullptr;
     if (plan->workspace_bytes) {
         if (int rc = static_workspace(&ws)) return rc;
+        // Everything the launch itself would refuse is refused here, before the fill kernel goes out.
+        if (plan->kind != 0 || plan->splits < 1 || !pick_kernel(plan->mi, plan->ni, plan->kw, plan->k_order, plan->depth)) return PAELLA_EINVAL;
+        ConvArgs probe;
+        if (int rc = fill_args(plan, x, blob_dev, bias, residual, slope, y, ws, job_id,
+                               reinterpret_cast<llis::job::FinishedBlockNotifier*>(notifier), probe))
+            return rc;
         // One arrival counter per output tile, at the head of the workspace.
         const unsigned tiles = plan->dims.grid / (unsigned)plan->splits;
         hipLaunchKernelGGL(zero_words_kernel, dim3((tiles + 255u) / 256u), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
@@ -1764,10 +1802,10 @@ int pre_send_all(bool only_full) {
             if (only_full && left < (size_t)kPackMax) break;
             const int n = (int)std::min<size_t>(left, (size_t)kPackMax);
             void* target = nullptr;
-            if (paella_direct_queue_shared(&target) != 0) return -1;
             unsigned grid = 0, dyn_lds = 0;
-            int rc = 0;
-            if (n == 1) {
+            int rc = paella_direct_queue_shared(&target) != 0 ? -1 : 0;
+            if (rc != 0) {
+            } else if (n == 1) {
                 ConvPreKernel kern = pick_pre_kernel(kw);
                 ConvPreArgs a = list[done].a;
                 a.conv.hook_blocks = 0;
@@ -1794,7 +1832,10 @@ int pre_send_all(bool only_full) {
                     rc = (int)hipGetLastError();
                 }
             }
-            if (rc != 0) return -1;
+            if (rc != 0) {  // what went out before leaves the list all the same
+                list.erase(list.begin(), list.begin() + (long)done);
+                return -1;
+            }
             ++launches;
             g_pack_launches.fetch_add(1, std::memory_order_relaxed);
             g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);

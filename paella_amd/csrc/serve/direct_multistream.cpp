@@ -102,10 +102,14 @@ class DirectRunner {
 
     // The whole request on one stream; the caller holds mtx_ (or runs alone).
     void issue(Module* m, void* stream) {
-        m->stream = stream;
         check(llis_hip_memcpy_async(paella_exec_input(m->exec), m->host_in, m->in_bytes, LLIS_HIP_H2D, stream), "input copy");
         check(paella_exec_forward(m->exec, stream), "paella_exec_forward");
         check(llis_hip_memcpy_async(m->host_out, paella_exec_output(m->exec), m->out_bytes, LLIS_HIP_D2H, stream), "output copy");
+        // Published last: the monitor scans without the lock and takes "stream set and idle" for "request done".  Set before the
+        // work is on the stream (where the reference sets it, reference tests/simple/tvm_direct_multistream.cpp:143-156) an idle
+        // stream would pass for a finished request of no latency, and the instance would be handed out again while this thread
+        // still issues onto it.
+        __atomic_store_n(&m->stream, stream, __ATOMIC_RELEASE);
     }
 
     void launch(unsigned type, double scheduled_arrival_us) {

@@ -159,9 +159,7 @@ void Server::notify_job_starts(job::Job* job) {
 
 void Server::notify_job_ends(job::Job* job) {
     job->on_complete();
-    ClientConnection* conn = client_connections_[job->get_client_id()].get();
-    if (conn->is_dead()) return;  // nobody reads that ring any more; writing to it would block once it is full
-    conn->get_s2c_channel()->write(job->get_remote_ptr());
+    total_owed_wakeups_ -= client_connections_[job->get_client_id()]->post_completion(job->get_remote_ptr());
 }
 
 void Server::release_job_instance(std::unique_ptr<job::Job> job) {

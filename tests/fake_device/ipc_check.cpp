@@ -16,6 +16,7 @@
 #include <llis/ipc/shm_channel.h>
 #include <llis/ipc/shm_primitive_channel.h>
 #include <llis/ipc/unix_datagram_socket.h>
+#include <llis/server/client_connection.h>
 #include <llis/job/instrument_info.h>
 
 #include <unistd.h>
@@ -208,6 +209,43 @@ int main(int argc, char** argv) {
         const bool ok = got == 42 && sent >= 1 && refused >= 1 && drained == sent && peer.try_write(&b, 1);
         std::printf(ok ? "OK socket sent=%d refused=%d\n" : "ERROR socket sent=%d refused=%d\n", sent, refused);
         return !ok;
+    }
+    if (cmd == "deadclient") {
+        // A peer that refuses every wake-up is taken for dead after two seconds, gets completions only while its ring has
+        // room (the serving thread never waits for it), and comes back when a wake-up gets through again.
+        const std::string tag = "dead" + std::to_string(getpid());
+        const std::string sock_name = s2c_socket_name(tag, 3);
+        UnixDatagramSocket sender;
+        llis::server::ClientConnection conn(3);
+        ShmChannelCpuReader ring(s2c_channel_name(tag, 3), 64);   // the client's end; 63 usable bytes = 7 completions
+        conn.use_s2c_channel(ShmChannelCpuWriter(s2c_channel_name(tag, 3)));
+        conn.use_s2c_socket(sender.connect(sock_name));           // nobody is bound there yet
+        int bad = 0;
+        for (int i = 0; i < 5; ++i) bad += !conn.wake();          // all owed
+        const auto t0 = std::chrono::steady_clock::now();
+        while (!conn.is_dead() && std::chrono::steady_clock::now() - t0 < std::chrono::seconds(4)) {
+            bad += conn.retry_wakeups() != 0;
+            usleep(1000);
+        }
+        bad += !conn.is_dead();
+        unsigned gave_back = 0;
+        for (uintptr_t i = 1; i <= 10; ++i) gave_back += conn.post_completion(reinterpret_cast<void*>(i));   // returns at once, every time
+        bad += conn.dropped_completions() != 3 || gave_back != 3;  // 7 fit; each dropped one takes an owed wake-up with it
+        UnixDatagramSocket receiver(sock_name);                    // the "client" shows up after all
+        usleep(250000);
+        const unsigned settled = conn.retry_wakeups();
+        bad += conn.is_dead() || settled != 2;
+        char b;
+        for (unsigned i = 0; i < settled; ++i) receiver.read(&b, 1);
+        for (uintptr_t i = 1; i <= 7; ++i) {
+            void* p = nullptr;
+            ring.read(&p);
+            bad += p != reinterpret_cast<void*>(i);
+        }
+        bad += ring.can_read();
+        bad += conn.wake();   // goes straight out again
+        std::printf(bad ? "ERROR deadclient %d\n" : "OK deadclient\n", bad);
+        return bad != 0;
     }
     std::fprintf(stderr, "unknown check\n");
     return 2;

@@ -10,7 +10,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 HEADERS = {"paella_hip.h": "llis_hip", "paella_ops.h": "paella_ops", "paella_ring.h": "paella_ops", "paella_models.h": "paella_ops",
-           "paella_serve.h": "paella_serve"}
+           "paella_serve.h": "paella_serve", "paella_probes.h": "paella_probes"}
 
 
 def declared(header):
@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported(header):
     _abi.hip()
     lib = ctypes.CDLL(os.path.join(_abi.LIB_DIR, "lib%s.so" % HEADERS[header]), mode=ctypes.RTLD_GLOBAL)
     names = declared(header)
-    assert len(names) >= 5
+    assert len(names) >= 4
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
 
@@ -33,7 +33,8 @@ def test_every_declared_symbol_is_exported(header):
 def test_python_tables_cover_the_headers():
     from paella_amd import _abi, _abi_models, serve
     tables = {"paella_hip.h": _abi.HIP_SYMBOLS, "paella_ops.h": _abi.OPS_SYMBOLS, "paella_ring.h": _abi.RING_SYMBOLS,
-              "paella_models.h": _abi_models.MODEL_SYMBOLS, "paella_serve.h": serve.SERVE_SYMBOLS}
+              "paella_models.h": _abi_models.MODEL_SYMBOLS, "paella_serve.h": serve.SERVE_SYMBOLS,
+              "paella_probes.h": _abi.PROBE_SYMBOLS}
     for header, table in tables.items():
         assert sorted(table) == declared(header), header
 

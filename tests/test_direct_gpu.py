@@ -117,12 +117,12 @@ def test_queue_concurrency_probe_runs_and_reports_a_time(cuda):
     lib = _abi.ops()
     d = ConvDesc(64, 14, 14, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 0.0)
     us = ctypes.c_double()
-    assert lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 3, 2, 1, 5, ctypes.byref(us)) == -1  # 8 instances, 3 per launch
-    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 1, 1, 20, ctypes.byref(us)), "probe, one queue")
+    assert _abi.probes().paella_queue_concurrency_probe(ctypes.byref(d), 8, 3, 2, 1, 5, ctypes.byref(us)) == -1  # 8 instances, 3 per launch
+    _abi.check(_abi.probes().paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 1, 1, 20, ctypes.byref(us)), "probe, one queue")
     one = us.value
-    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 4, 1, 20, ctypes.byref(us)), "probe, four queues")
+    _abi.check(_abi.probes().paella_queue_concurrency_probe(ctypes.byref(d), 8, 1, 4, 1, 20, ctypes.byref(us)), "probe, four queues")
     four = us.value
-    _abi.check(lib.paella_queue_concurrency_probe(ctypes.byref(d), 8, 4, 4, 1, 20, ctypes.byref(us)), "probe, four per launch")
+    _abi.check(_abi.probes().paella_queue_concurrency_probe(ctypes.byref(d), 8, 4, 4, 1, 20, ctypes.byref(us)), "probe, four per launch")
     assert 0.1 < four <= one * 1.1 and 0.05 < us.value < one * 1.1, (one, four, us.value)
 
 
@@ -135,7 +135,7 @@ def test_vector_alu_work_adds_to_matrix_instruction_time(cuda):
 
     def probe(n):
         both, alone, tf = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
-        _abi.check(lib.paella_mfma_valu_overlap_probe(n, ctypes.byref(both), ctypes.byref(alone), ctypes.byref(tf)), "paella_mfma_valu_overlap_probe")
+        _abi.check(_abi.probes().paella_mfma_valu_overlap_probe(n, ctypes.byref(both), ctypes.byref(alone), ctypes.byref(tf)), "paella_mfma_valu_overlap_probe")
         return both.value, alone.value, tf.value
 
     base, _, peak = probe(0)
@@ -144,4 +144,4 @@ def test_vector_alu_work_adds_to_matrix_instruction_time(cuda):
         both, alone, tf = probe(n)
         assert alone > 0 and 0.9 * (base + alone) < both < 1.1 * (base + alone), (n, base, alone, both)
         assert tf < peak
-    assert lib.paella_mfma_valu_overlap_probe(7, None, None, None) == -1
+    assert _abi.probes().paella_mfma_valu_overlap_probe(7, None, None, None) == -1

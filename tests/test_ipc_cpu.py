@@ -20,7 +20,7 @@ def built():
     ensure_built()
 
 
-@pytest.mark.parametrize("check", ["threads", "messages", "multiwriter", "pring", "socket", "pollhooks"])
+@pytest.mark.parametrize("check", ["threads", "messages", "multiwriter", "pring", "socket", "pollhooks", "deadclient"])
 def test_ipc_self_checks(check):
     out = subprocess.run([CHECK, check], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout + out.stderr

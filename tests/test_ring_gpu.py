@@ -179,7 +179,7 @@ def test_notify_latency_probes_report_sane_numbers(ring):
     _abi.check(lib.paella_ring_bench_pingpong(50, 500, ctypes.byref(flag), ctypes.byref(sync), None))
     assert 0.5 < flag.value < 2000.0 and 0.5 < sync.value < 5000.0
     floor = ctypes.c_double()
-    _abi.check(lib.paella_empty_kernel_probe(50, ctypes.byref(floor)))
+    _abi.check(_abi.probes().paella_empty_kernel_probe(50, ctypes.byref(floor)))
     assert 0.2 < floor.value < 200.0
     print("ring drain 64 blocks: %.2f us/iter; flag ping-pong %.2f us; stream sync %.2f us; empty kernel %.2f us" %
           (us.value, flag.value, sync.value, floor.value))

@@ -65,3 +65,46 @@ def test_static_workspace_rejects_what_does_not_fit_and_unsplit_plans_need_none(
     assert rc == PAELLA_ETOOBIG
     torch.cuda.synchronize()
     assert bool(torch.isnan(got).all())           # nothing was launched
+
+
+def test_static_workspace_survives_counters_left_dirty(cuda):
+    """An interrupted call may leave arrival counters at any value: the array is dirtied through its device address (every
+    word a call could use as a counter or a partial sum set to a pattern) and the next call still gives the same bits."""
+    from paella_amd import _abi
+    conv, x = make(512, 7, 128, 3, seed=15)
+    assert conv.plan.splits > 1
+    want = conv(x)
+    torch.cuda.synchronize()
+    assert conv.lib.paella_conv2d_static_init() == 0
+    ws = ctypes.c_void_p()
+    assert conv.lib.paella_conv2d_static_workspace(ctypes.byref(ws)) == 0 and ws.value
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for pattern in (0xFFFFFFFF, 0x00000001, 0x7FC00000):
+        _abi.check(_abi.hip().llis_hip_fill_u32_async(ws, pattern, STATIC_BYTES // 4, stream))
+        rc, got = launch_static(conv, x)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), hex(pattern)
+
+
+def test_static_entry_point_checks_its_arguments_before_it_launches_anything(cuda):
+    """A refused call must not have sent the counter fill either: the array keeps the pattern written before the call."""
+    from paella_amd import _abi
+    conv, x = make(512, 7, 128, 3, seed=16)
+    ws = ctypes.c_void_p()
+    assert conv.lib.paella_conv2d_static_workspace(ctypes.byref(ws)) == 0
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _abi.check(_abi.hip().llis_hip_fill_u32_async(ws, 0xA5A5A5A5, 1024, stream))
+    p = conv.plan
+    y = torch.zeros((1, p.d.K, p.P, p.Q), device="cuda:0")
+    rc = conv.lib.paella_conv2d_launch_static(ctypes.byref(p), None, ctypes.c_void_p(conv.blob.data_ptr()), ctypes.c_void_p(conv.bias.data_ptr()),
+                                              None, None, ctypes.c_void_p(y.data_ptr()), stream, 0, None)
+    assert rc == -1  # PAELLA_EINVAL: no input
+    head = torch.empty(1024, dtype=torch.int32, device="cuda:0")
+    _abi.check(_abi.hip().llis_hip_memcpy_async(ctypes.c_void_p(head.data_ptr()), ws, 4096, 3, stream))  # device to device
+    torch.cuda.synchronize()
+    assert bool((head == torch.tensor(0xA5A5A5A5 - (1 << 32), dtype=torch.int32, device="cuda:0")).all())
+    rc, got = launch_static(conv, x)   # and the entry point still works afterwards
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, conv(x))
