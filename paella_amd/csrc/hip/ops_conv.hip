@@ -144,6 +144,18 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     unsigned long long tl[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #endif
     TL_STAMP(0);
+#ifndef PAELLA_CONV_LAZY_ARGS
+    // The fields the prologue uses, requested together and waited for once.  Read where they are used, each costs a trip to
+    // the scalar cache of its own, one after the other -- some twenty of them before a wave's first operand load -- and with
+    // every wave of a launch in its prologue at the same time those trips are what the launch waits for.
+    {
+        const unsigned long long a0 = (unsigned long long)p.x, a1 = (unsigned long long)p.wpk, a2 = (unsigned long long)p.notifier;
+        asm volatile("" ::"s"(a0), "s"(a1), "s"(a2), "s"(p.H), "s"(p.W), "s"(p.Q), "s"(p.PQ), "s"(p.sh), "s"(p.sw), "s"(p.ph), "s"(p.pw), "s"(p.m_pad),
+                     "s"(p.nchunks), "s"(p.CB), "s"(p.w_bytes), "s"(p.splits), "s"(p.chunks_per_split), "s"(p.n_tiles_n), "s"(p.n_tiles_m),
+                     "s"(p.slab_major), "s"(p.x_bytes), "s"(p.job_id), "s"(p.hook_blocks), "s"(p.fast_div));
+        asm volatile("" ::"s"(p.div_w.mul), "s"(p.div_w.one), "s"(p.div_tm.mul), "s"(p.div_tm.one), "s"(p.div_q.mul), "s"(p.div_q.one));
+    }
+#endif
     if (bid >= (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
@@ -236,7 +248,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // a lane's part of an offset sits in a register that changes only when the filter tap does, the chunk's part rides in the
     // load's scalar offset (not range-checked: an out-of-range lane offset stays out of range, a valid one stays valid), and a
     // chunk outside the wave's range reads through a descriptor of zero length instead of an offset made invalid per lane.
-    const __amdgpu_buffer_rsrc_t nores = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, 0, 0x00027000);
+    // (the same descriptor with length zero: choosing between the two is then one scalar select, on the length word)
+    const char* const x_base = reinterpret_cast<const char*>(p.x) - pad_off;
+    const unsigned x_len = p.x_bytes + pad_off, w_len = p.w_bytes;
     const int wlane = (int)(((unsigned)kk * (unsigned)p.m_pad + (unsigned)(m0 + j)) * 16u);
     const int wstep = p.m_pad * 32;  // bytes of weights per chunk and row block: two reduction steps of m_pad rows of 16 bytes
     int tap_voff[NI];
@@ -245,7 +259,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     int tap_off = 0;  // byte offset of the current filter tap, wave-uniform
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
         if (TAP_MAJOR) {
-            const __amdgpu_buffer_rsrc_t wr = valid ? wres : nores;
+            const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, valid ? w_len : 0u, 0x00027000);
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi) {
                 const auto v = __builtin_amdgcn_raw_buffer_load_b128(wr, wlane, c * wstep + mi * 32 * 16, 0);
@@ -270,7 +284,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 }
                 tap_soff = tap_off;
             }
-            const __amdgpu_buffer_rsrc_t xr = valid ? xres : nores;
+            const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void*)x_base, 0, valid ? x_len : 0u, 0x00027000);
             const int chunk_off = cb * 8 * HW4 + tap_soff;
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
