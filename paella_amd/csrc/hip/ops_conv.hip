@@ -144,18 +144,16 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     unsigned long long tl[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #endif
     TL_STAMP(0);
-#ifndef PAELLA_CONV_LAZY_ARGS
     // The fields the prologue uses, requested together and waited for once.  Read where they are used, each costs a trip to
-    // the scalar cache of its own, one after the other -- some twenty of them before a wave's first operand load -- and with
-    // every wave of a launch in its prologue at the same time those trips are what the launch waits for.
-    {
+    // the scalar cache of its own, one after the other -- some twenty of them before a wave's first operand load.  (Only where
+    // the scalar registers are there for it: the eight-wave small tile, which is what nearly every launch runs.)
+    if (KW == 8 && MI * NI == 1 && DEPTH == 0) {
         const unsigned long long a0 = (unsigned long long)p.x, a1 = (unsigned long long)p.wpk, a2 = (unsigned long long)p.notifier;
         asm volatile("" ::"s"(a0), "s"(a1), "s"(a2), "s"(p.H), "s"(p.W), "s"(p.Q), "s"(p.PQ), "s"(p.sh), "s"(p.sw), "s"(p.ph), "s"(p.pw), "s"(p.m_pad),
                      "s"(p.nchunks), "s"(p.CB), "s"(p.w_bytes), "s"(p.splits), "s"(p.chunks_per_split), "s"(p.n_tiles_n), "s"(p.n_tiles_m),
                      "s"(p.slab_major), "s"(p.x_bytes), "s"(p.job_id), "s"(p.hook_blocks), "s"(p.fast_div));
         asm volatile("" ::"s"(p.div_w.mul), "s"(p.div_w.one), "s"(p.div_tm.mul), "s"(p.div_tm.one), "s"(p.div_q.mul), "s"(p.div_q.one));
     }
-#endif
     if (bid >= (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
@@ -371,17 +369,24 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const int rows_tile = max(p.K - m0, 0);  // channels from this tile's first one to the last that exists (may exceed the tile)
     const float* const res_tile = p.residual ? p.residual + (size_t)m0 * p.PQ : nullptr;
     float* const y_tile = p.y + (size_t)m0 * p.PQ;
-    // The hardware holds lane offset + scalar offset against the length, so the length is that of all the tile's channels; a
-    // row that does not exist gets length zero and scalar offset zero (no sum that could pass a wrapped comparison).
-    auto row_exists = [&](int rr) { return row_of(rr) < rows_tile; };
-    auto plane_rsrc = [&](const float* tile_base, int rr) {
-        return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, row_exists(rr) ? (unsigned)rows_tile * plane : 0u, 0x00027000);
+    // The hardware tests lane offset >= length - scalar offset (unsigned), so the length is that of all the tile's channels and
+    // a row's scalar offset is held at that length: the difference is then zero for a row that does not exist and every lane of
+    // the access is out of range (an offset past the length would wrap the difference and pass the test).  One descriptor per
+    // tensor; what changes with the register is a scalar offset of two instructions.
+    const unsigned tile_len = (unsigned)rows_tile * plane;
+    const unsigned chan_len = (unsigned)rows_tile * 4u;
+    auto plane_rsrc = [&](const float* tile_base, int) { return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, tile_len, 0x00027000); };
+    auto chan_rsrc = [&](const float* per_channel, int) {  // bias, slope: one float per channel
+        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, chan_len, 0x00027000);
     };
-    auto chan_rsrc = [&](const float* per_channel, int rr) {  // bias, slope: one float per channel
-        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, row_exists(rr) ? (unsigned)rows_tile * 4u : 0u, 0x00027000);
-    };
-    auto plane_soff = [&](int rr) { return row_exists(rr) ? (int)((unsigned)row_of(rr) * plane) : 0; };
-    auto chan_soff = [&](int rr) { return row_exists(rr) ? row_of(rr) * 4 : 0; };
+    int plane_soffs[RPW], chan_soffs[RPW];
+#pragma unroll
+    for (int rr = 0; rr < RPW; ++rr) {
+        plane_soffs[rr] = (int)min((unsigned)row_of(rr) * plane, tile_len);
+        chan_soffs[rr] = (int)min((unsigned)row_of(rr) * 4u, chan_len);
+    }
+    auto plane_soff = [&](int rr) { return plane_soffs[rr]; };
+    auto chan_soff = [&](int rr) { return chan_soffs[rr]; };
     const int chan_voff = kk * 16;
     // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
     // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
