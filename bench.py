@@ -780,14 +780,28 @@ def main():
             roofline["under_load"] = {"forward_passes_per_s": mq, "conv_tflops": mq * rl["conv_flops"] / 1e12,
                                       "frac": mq * rl["conv_flops"] / 1e12 / FP32_MFMA_PEAK_TFLOPS,
                                       "how": "4 Inception-v3 forward passes in flight on 4 ordered direct-dispatch queues, no hooks, no scheduler"}
-            with serve.Server("bench_inc_%d" % os.getpid(), "full3", num_streams=streams, cpu=4, extra_kernels=ek) as srv:
-                r = serve.client_run(srv.name, [(serve.job_path("tvm_inception_v3"), 1.0, 16)], 0.0, 16, 3000, warmup_jobs=300, pin_threads=True)
-            served = r["throughput_rps"]
+            # closed loop at two depths: 16 requests in flight is what the headline mix keeps (more of the large model in flight costs
+            # the small one its p99), 32 is where the rate of the model alone stops growing (24: +6 %, 32: +8 %, 48: +7 % over 16)
+            by_depth = {}
+            for depth in (16, 32):
+                with serve.Server("bench_inc%d_%d" % (depth, os.getpid()), "full3", num_streams=streams, cpu=4, extra_kernels=ek) as srv:
+                    r = serve.client_run(srv.name, [(serve.job_path("tvm_inception_v3"), 1.0, depth)], 0.0, depth, 4000, warmup_jobs=400, pin_threads=True,
+                                         verify=Arm.verify)
+                if Arm.verify:
+                    Arm.verified += r["verified_requests"]
+                    Arm.mismatches += r["mismatches"]
+                by_depth[depth] = r["throughput_rps"]
+            best = max(by_depth, key=by_depth.get)
+            served = by_depth[best]
             roofline["served"] = {"forward_passes_per_s": served, "conv_tflops": served * rl["conv_flops"] / 1e12,
                                   "frac": served * rl["conv_flops"] / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-                                  "how": "Inception-v3 alone through full3 at saturation (16 requests outstanding, input copy per request): conv launches of "
-                                         "different requests packed into shared launches"}
-            log("[bench] Inception-v3 alone through full3 at saturation: %.0f requests/s = %.1f%% of peak over the conv work" % (served, 100 * roofline["served"]["frac"]))
+                                  "requests_outstanding": best,
+                                  "requests_per_s_by_requests_outstanding": {str(k): v for k, v in by_depth.items()},
+                                  "frac_at_16_outstanding": by_depth[16] * rl["conv_flops"] / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                                  "how": "Inception-v3 alone through full3 at saturation (closed loop with 16 and with 32 requests outstanding, the higher "
+                                         "rate; input copy per request): conv launches of different requests packed into shared launches"}
+            log("[bench] Inception-v3 alone through full3 at saturation: %.0f requests/s with 16 outstanding, %.0f with 32 = %.1f%% of peak over the conv work" %
+                (by_depth[16], by_depth[32], 100 * roofline["served"]["frac"]))
             mq18 = multi_queue_rate(models, "resnet18")
             side["resnet18_four_passes_in_flight"] = {"forward_passes_per_s": mq18, "conv_tflops": mq18 * rl18["conv_flops"] / 1e12,
                                                       "frac_of_fp32_mfma_peak": mq18 * rl18["conv_flops"] / 1e12 / FP32_MFMA_PEAK_TFLOPS}
@@ -930,6 +944,9 @@ def headline(out):
     for k in ("served", "under_load", "full_device"):
         if isinstance(rf.get(k), dict):
             r[k] = {"frac": rf[k].get("frac"), "tflops": rf[k].get("conv_tflops", rf[k].get("achieved"))}
+            if "requests_outstanding" in rf[k]:
+                r[k]["requests_outstanding"] = rf[k]["requests_outstanding"]
+                r[k]["frac_at_16_outstanding"] = rf[k].get("frac_at_16_outstanding")
     line["roofline"] = r
     for key in ("cpu_baseline", "cpu_baseline_torch"):
         c = out.get(key)

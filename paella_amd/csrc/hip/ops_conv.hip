@@ -346,7 +346,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     constexpr int NACC = MI * NI * 16;
     constexpr int RPW = NACC / KW;
     // (a variant with a deeper operand pipeline keeps its registers for the chunks in flight)
-    constexpr bool kPrefetchEpilogue = DEPTH ? RPW <= 4 : RPW <= 16;
+    // (nor does the variant with an input transform: its scale and shift operands take the registers, and with the epilogue's
+    // operands requested after the loop it fits the 64 registers of eight waves per SIMD)
+    constexpr bool kPrefetchEpilogue = !PRE && (DEPTH ? RPW <= 4 : RPW <= 16);
     // Output addressing.  Register r of the tile (r = wave * RPW + rr for this wave) holds, in lane (j, kk), output channel
     // m0 + row(r) + 4 * kk at pixel n0 + 32 * ni(r) + j.  Everything that depends on the tile, the wave or r is wave-uniform and
     // goes into buffer descriptors and scalar offsets built on the scalar unit: per tensor a descriptor at the tile's first
@@ -650,7 +652,7 @@ struct ConvPreArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW) void conv_mfma_pre_kernel(ConvPreArgs args) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_pre_kernel(ConvPreArgs args) {
     int idx = 0;  // see conv_mfma_kernel
     asm volatile("" : "+s"(idx));
     const ConvPreArgs& a = (&args)[idx];
@@ -665,7 +667,7 @@ struct ConvPreGroupArgs {
 };
 
 template <int KW>
-__global__ __launch_bounds__(64 * KW) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
+__global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
     int idx = 0;
 #pragma unroll
     for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
