@@ -147,14 +147,23 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // The fields the prologue uses, requested together and waited for once.  Read where they are used, each costs a trip to
     // the scalar cache of its own, one after the other -- some twenty of them before a wave's first operand load.  (Only where
     // the scalar registers are there for it: the eight-wave small tile, which is what nearly every launch runs.)
+    // ... and held in scalar registers until the prologue is through with them: as results of an (empty) asm statement the
+    // compiler cannot fetch them again where they are used, which it otherwise does, one trip each.
+    struct Held {
+        int n_tiles_n, n_tiles_m, splits, slab_major, fast_div;
+        FastDiv div_w, div_tm;
+    } a;
+    a.n_tiles_n = p.n_tiles_n; a.n_tiles_m = p.n_tiles_m; a.splits = p.splits; a.slab_major = p.slab_major; a.fast_div = p.fast_div;
+    a.div_w = p.div_w; a.div_tm = p.div_tm;
     if (KW == 8 && MI * NI == 1 && DEPTH == 0) {
         const unsigned long long a0 = (unsigned long long)p.x, a1 = (unsigned long long)p.wpk, a2 = (unsigned long long)p.notifier;
         asm volatile("" ::"s"(a0), "s"(a1), "s"(a2), "s"(p.H), "s"(p.W), "s"(p.Q), "s"(p.PQ), "s"(p.sh), "s"(p.sw), "s"(p.ph), "s"(p.pw), "s"(p.m_pad),
-                     "s"(p.nchunks), "s"(p.CB), "s"(p.w_bytes), "s"(p.splits), "s"(p.chunks_per_split), "s"(p.n_tiles_n), "s"(p.n_tiles_m),
-                     "s"(p.slab_major), "s"(p.x_bytes), "s"(p.job_id), "s"(p.hook_blocks), "s"(p.fast_div));
-        asm volatile("" ::"s"(p.div_w.mul), "s"(p.div_w.one), "s"(p.div_tm.mul), "s"(p.div_tm.one), "s"(p.div_q.mul), "s"(p.div_q.one));
+                     "s"(p.nchunks), "s"(p.CB), "s"(p.w_bytes), "s"(p.chunks_per_split), "s"(p.x_bytes), "s"(p.job_id), "s"(p.hook_blocks),
+                     "s"(p.div_q.mul), "s"(p.div_q.one));
+        asm volatile("" : "+s"(a.n_tiles_n), "+s"(a.n_tiles_m), "+s"(a.splits), "+s"(a.slab_major), "+s"(a.fast_div), "+s"(a.div_w.mul), "+s"(a.div_w.one),
+                     "+s"(a.div_tm.mul), "+s"(a.div_tm.one));
     }
-    if (bid >= (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits)) return;
+    if (bid >= (unsigned)(a.n_tiles_n * a.n_tiles_m * a.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
     // Waves of this workgroup whose result stores have been acknowledged (see the end of this function); cleared here, and
@@ -177,21 +186,21 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // with small feature maps) or neighbouring pixel tiles, whose 3x3 halos overlap (layers with large ones).
     int tile_n, tile_m, split;
     {
-        const unsigned total = (unsigned)(p.n_tiles_n * p.n_tiles_m * p.splits);
+        const unsigned total = (unsigned)(a.n_tiles_n * a.n_tiles_m * a.splits);
         const unsigned xcd = bid & 7u, j = bid >> 3;
         const unsigned q = total >> 3, r = total & 7u;
-        const unsigned w = p.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
-        if (p.slab_major) {
-            const unsigned slab = quot(w, (unsigned)p.n_tiles_n, p.div_w, p.fast_div);
-            tile_n = (int)(w - slab * (unsigned)p.n_tiles_n);
-            split = (int)quot(slab, (unsigned)p.n_tiles_m, p.div_tm, p.fast_div);
-            tile_m = (int)(slab - (unsigned)split * (unsigned)p.n_tiles_m);
+        const unsigned w = a.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
+        if (a.slab_major) {
+            const unsigned slab = quot(w, (unsigned)a.n_tiles_n, a.div_w, a.fast_div);
+            tile_n = (int)(w - slab * (unsigned)a.n_tiles_n);
+            split = (int)quot(slab, (unsigned)a.n_tiles_m, a.div_tm, a.fast_div);
+            tile_m = (int)(slab - (unsigned)split * (unsigned)a.n_tiles_m);
         } else {
-            const unsigned per_n = (unsigned)(p.n_tiles_m * p.splits);
-            tile_n = (int)quot(w, per_n, p.div_w, p.fast_div);
+            const unsigned per_n = (unsigned)(a.n_tiles_m * a.splits);
+            tile_n = (int)quot(w, per_n, a.div_w, a.fast_div);
             const unsigned rest = w - (unsigned)tile_n * per_n;
-            split = (int)quot(rest, (unsigned)p.n_tiles_m, p.div_tm, p.fast_div);
-            tile_m = (int)(rest - (unsigned)split * (unsigned)p.n_tiles_m);
+            split = (int)quot(rest, (unsigned)a.n_tiles_m, a.div_tm, a.fast_div);
+            tile_m = (int)(rest - (unsigned)split * (unsigned)a.n_tiles_m);
         }
     }
     const int m0 = tile_m * (32 * MI);
@@ -214,7 +223,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             base[ni] = pix < p.PQ ? pix * 4 + kk4hw : -1;
             continue;
         }
-        const int ho = (int)quot((unsigned)pix, (unsigned)p.Q, p.div_q, p.fast_div);
+        const int ho = (int)quot((unsigned)pix, (unsigned)p.Q, p.div_q, a.fast_div);
         const int wo = pix - __mul24(ho, p.Q);  // every factor here is a pixel coordinate or an extent: far below 2^23
         hb[ni] = (pix < p.PQ) ? __mul24(ho, p.sh) - p.ph : -0x100000;
         wb[ni] = __mul24(wo, p.sw) - p.pw;
