@@ -834,6 +834,38 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
     paella::hook_exit(p.notifier, p.job_id);
 }
 
+// The same for up to PAELLA_CONV_PACK_MAX depthwise convs of different requests in one launch (launch packing): a model of
+// many short kernels is bound by how many launches the four queues start per second, and its depthwise layers are a third
+// of them.  A member's workgroups behave exactly as in a launch of their own (same elements per thread, same messages).
+struct DwGroupArgs {
+    unsigned start[PAELLA_CONV_PACK_MAX];  // first workgroup id of each member; 0xFFFFFFFF for unused entries
+    unsigned grids[PAELLA_CONV_PACK_MAX];  // workgroups of each member
+    DwArgs m[PAELLA_CONV_PACK_MAX];        // only the used entries are written to the argument ring
+};
+
+__global__ __launch_bounds__(256) void dwconv_group_kernel(DwGroupArgs g) {
+    int member = 0;
+#pragma unroll
+    for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
+        if (blockIdx.x >= g.start[i]) member = i;
+    const DwArgs& p = g.m[member];
+    const unsigned grid = g.grids[member];
+    const unsigned bid = blockIdx.x - g.start[member];
+    paella::hook_entry(p.notifier, p.job_id, grid);
+    const int PQ = p.P * p.Q;
+    const int total = p.C * PQ;
+    const int stride = (int)grid * 256;
+    int idx = (int)bid * 256 + threadIdx.x;
+    if (stride >= total) {
+        if (idx < total) dw_element(p, idx, PQ);
+    } else {
+#pragma unroll
+        for (int k = 0; k < kDwPerThread; ++k, idx += stride)
+            if (idx < total) dw_element(p, idx, PQ);
+    }
+    paella::hook_exit(p.notifier, p.job_id, grid);
+}
+
 typedef void (*ConvKernel)(ConvArgs);
 
 template <int MI, int NI, bool TM>
@@ -1226,6 +1258,11 @@ struct PackState {
     int held = 0;                 // items and sequences over all lists
     uint64_t first_held_ns = 0;
     PackList lists[4][2];         // by log2(waves per workgroup) and reduction order
+    struct DwItem {
+        DwArgs a;
+        unsigned grid;
+    };
+    std::vector<DwItem> dw_list;   // depthwise convs, packed among themselves
     std::vector<SeqList> seq_lists;
     struct PreItem {
         ConvPreArgs a;
@@ -1251,6 +1288,62 @@ uint64_t now_ns() {
 int kw_index(int kw) { return kw == 1 ? 0 : kw == 2 ? 1 : kw == 4 ? 2 : 3; }
 
 // Holds the call back if packing applies to it.  Returns false when the caller must launch it itself.
+// A depthwise conv bound for an unordered direct queue is held like a small-tile conv and packed with other requests' depthwise convs.
+bool pack_hold_dw(const DwArgs& a, unsigned grid, void* stream) {
+    if (paella::g_pack_recording || !g_pack.enabled || paella::timing_events().start != nullptr) return false;
+    paella::DirectQueue* q = paella::direct_queue_lookup(stream);
+    if (!q || paella::direct_queue_ordered(q)) return false;
+    g_pack.dw_list.push_back(PackState::DwItem{a, grid});
+    if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
+    return true;
+}
+
+int dw_send_all(bool only_full) {
+    std::vector<PackState::DwItem>& list = g_pack.dw_list;
+    int launches = 0;
+    size_t done = 0;
+    bool failed = false;
+    while (done < list.size()) {
+        const size_t left = list.size() - done;
+        if (only_full && left < (size_t)kPackMax) break;
+        const int n = (int)std::min<size_t>(left, (size_t)kPackMax);
+        void* target = nullptr;
+        int rc = paella_direct_queue_shared(&target) != 0 ? -1 : 0;
+        if (rc != 0) {
+        } else if (n == 1) {
+            paella::launch(dwconv_kernel, dim3(list[done].grid), dim3(256), 0, reinterpret_cast<hipStream_t>(target), list[done].a);
+            rc = (int)hipGetLastError();
+        } else {
+            DwGroupArgs g;
+            unsigned grid = 0;
+            for (int i = 0; i < n; ++i) {
+                g.m[i] = list[done + (size_t)i].a;
+                g.start[i] = grid;
+                g.grids[i] = list[done + (size_t)i].grid;
+                grid += g.grids[i];
+            }
+            for (int i = n; i < kPackMax; ++i) {
+                g.start[i] = 0xFFFFFFFFu;
+                g.grids[i] = 0;
+            }
+            paella::launch_used(dwconv_group_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(target),
+                                offsetof(DwGroupArgs, m) + (size_t)n * sizeof(DwArgs), g);
+            rc = (int)hipGetLastError();
+        }
+        if (rc != 0) {
+            failed = true;
+            break;
+        }
+        ++launches;
+        g_pack_launches.fetch_add(1, std::memory_order_relaxed);
+        g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
+        g_pack.held -= n;
+        done += (size_t)n;
+    }
+    list.erase(list.begin(), list.begin() + (long)done);   // what went out leaves the list on every path
+    return failed ? -1 : launches;
+}
+
 bool pack_hold(const paella_conv_plan* const* plans, const ConvArgs* args, int n, void* stream, const paella::PoolArgs* pool = nullptr,
                unsigned pool_grid = 0) {
     if (paella::g_pack_recording) {
@@ -1444,11 +1537,17 @@ bool same_signature(const Sequence& a, const Sequence& b) {
 }
 
 int pre_send_all(bool only_full);  // below, with the kernels it launches
+int dw_send_all(bool only_full);
 
 int pack_send_all(bool only_full) {
     int launches = 0;
     {
         const int r = pre_send_all(only_full);
+        if (r < 0) return PAELLA_ENOSUP;
+        launches += r;
+    }
+    {
+        const int r = dw_send_all(only_full);
         if (r < 0) return PAELLA_ENOSUP;
         launches += r;
     }
@@ -1704,6 +1803,7 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
     a.job_id = job_id;
     a.notifier = nf;
+    if (pack_hold_dw(a, plan->dims.grid, stream)) return 0;
     paella::launch(dwconv_kernel, dim3(plan->dims.grid), dim3(256), 0, st, a);
     return (int)hipGetLastError();
 }

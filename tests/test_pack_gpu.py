@@ -255,6 +255,61 @@ def test_convs_with_a_fused_input_transform_are_packed_among_themselves(ring, cu
         assert torch.equal(a, b)
 
 
+def test_depthwise_convs_are_packed_among_themselves(ring, cuda):
+    """Depthwise convs of several jobs in one launch (dwconv_group_kernel): bit-identical to launches of their own -- the small
+    layers with one output per thread and the large ones with four -- and every notifier counts its own workgroups; a depthwise
+    conv alone in the list goes out through the plain kernel."""
+    lib, h = ring
+    from paella_amd import ops
+    rng = np.random.default_rng(17)
+    cases = []
+    for c, hw, stride, act in [(32, 112, 1, ops.ACT_RELU6), (96, 112, 2, ops.ACT_RELU6), (144, 56, 1, ops.ACT_RELU6), (192, 28, 2, ops.ACT_NONE),
+                               (384, 14, 1, ops.ACT_RELU6), (960, 7, 1, ops.ACT_RELU), (24, 19, 1, ops.ACT_RELU)]:
+        w = rng.standard_normal((c, 1, 3, 3)).astype(np.float32) / 3.0
+        b = rng.standard_normal(c).astype(np.float32)
+        conv = ops.Conv2d(w, b, stride=stride, pad=1, groups=c, act=act, in_hw=(hw, hw))
+        assert conv.plan.kind == 1
+        x = torch.tensor(rng.standard_normal((1, c, hw, hw)).astype(np.float32), device=cuda)
+        cases.append((conv, x))
+    assert any(c.plan.dims.grid * 256 < c.plan.d.K * c.plan.P * c.plan.Q for c, _ in cases)      # four outputs per thread
+    assert any(c.plan.dims.grid * 256 >= c.plan.d.K * c.plan.P * c.plan.Q for c, _ in cases)     # one output per thread
+    alone = [conv(x) for conv, x in cases]
+    torch.cuda.synchronize()
+    batch = lib.paella_ring_batch_size()
+    with ops.DirectQueue() as q:
+        assert lib.paella_pack_enable(1) == 0
+        try:
+            before = stats(lib)
+            outs = []
+            for j, (conv, x) in enumerate(cases):
+                y = torch.zeros_like(alone[j])
+                conv(x, out=y, stream=q.handle, job_id=(j + 1) | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, j)))
+                outs.append(y)
+            assert held(lib) == len(cases)
+            assert lib.paella_pack_flush() == 1 and held(lib) == 0
+            after = stats(lib)
+            assert (after[0] - before[0], after[1] - before[1]) == (1, len(cases))
+            want = sum((c[0].plan.dims.grid + batch - 1) // batch for c in cases)
+            buf = np.zeros(want, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want, 20.0) == want
+            m = decode(buf)
+            for j, c in enumerate(cases):
+                assert m["num"][m["job_id"] == j + 1].sum() == c[0].plan.dims.grid
+            # one alone: the plain kernel, same bits
+            y = torch.zeros_like(alone[0])
+            cases[0][0](cases[0][1], out=y, stream=q.handle, job_id=9 | NO_START, notifier=ctypes.c_void_p(lib.paella_ring_notifier(h, 9)))
+            assert held(lib) == 1 and lib.paella_pack_flush() == 1
+            want = (cases[0][0].plan.dims.grid + batch - 1) // batch
+            buf = np.zeros(want, np.uint64)
+            assert lib.paella_ring_drain(h, buf.ctypes.data, want, 20.0) == want
+            assert torch.equal(y, alone[0])
+        finally:
+            lib.paella_pack_enable(0)
+    torch.cuda.synchronize()
+    for a, b in zip(alone, outs):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("seed", [21, 22, 23])
 def test_random_mixes_of_calls_pack_to_the_bits_of_separate_launches(ring, cuda, seed):
     """Seeded mixes of single convs (both reduction orders, 2 to 8 waves), pairs and conv + pool calls, each under its own job id:
