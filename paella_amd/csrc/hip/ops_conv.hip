@@ -43,10 +43,15 @@
 #include "pack.h"
 
 #ifdef PAELLA_CONV_TIMELINE
-// Measurement build only: every wave of a conv leaves eight realtime-counter samples (100 MHz) in this buffer.
+// Measurement build only: every wave of a conv leaves sixteen realtime-counter samples (100 MHz) in this buffer.
 __device__ unsigned long long* g_tl_buf = nullptr;
 __device__ unsigned g_tl_cap = 0;
-#define TL_STAMP(i) tl[i] = wall_clock64()
+#define TL_STAMP(i)                           \
+    do {                                      \
+        __builtin_amdgcn_sched_barrier(0);    \
+        tl[i] = (unsigned)wall_clock64();     \
+        __builtin_amdgcn_sched_barrier(0);    \
+    } while (0)
 extern "C" int paella_conv_timeline_set(void* buf, unsigned waves) {
     if (hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_tl_buf), &buf, sizeof(buf))) return (int)e;
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_tl_cap), &waves, sizeof(waves));
@@ -97,12 +102,7 @@ struct ConvArgs {
     int pointwise;                  // tap-major only: 1x1 filter, stride 1, no padding
 };
 
-__device__ __forceinline__ unsigned quot(unsigned a, unsigned d, const FastDiv& f, int fast) {
-    return fast ? __umulhi(a, f.mul) + (a & f.one) : a / d;
-}
-
-// The same without the fallback, for dividends and divisors the host has checked (chunk numbers by chunks per tap, taps by
-// filter width).
+// The quotient for dividends and divisors the host has checked; where it could not, the kernel divides (ConvArgs::fast_div).
 __device__ __forceinline__ unsigned quot_fast(unsigned a, const FastDiv& f) { return __umulhi(a, f.mul) + (a & f.one); }
 
 __device__ __forceinline__ float apply_act(float v, int act, float slope, float lo, float hi) {
@@ -141,7 +141,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // A grouped launch starts every conv at a multiple of eight workgroups (see align_start): the ids between the end of one
     // problem and the start of the next belong to no tile and report to nobody.
 #ifdef PAELLA_CONV_TIMELINE
-    unsigned long long tl[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned tl[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};  // low words: a launch is over long before they wrap (43 s)
 #endif
     TL_STAMP(0);
     // The fields the prologue uses, requested together and waited for once.  Read where they are used, each costs a trip to
@@ -163,13 +163,13 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         asm volatile("" : "+s"(a.n_tiles_n), "+s"(a.n_tiles_m), "+s"(a.splits), "+s"(a.slab_major), "+s"(a.fast_div), "+s"(a.div_w.mul), "+s"(a.div_w.one),
                      "+s"(a.div_tm.mul), "+s"(a.div_tm.one));
     }
+    TL_STAMP(8);
     if (bid >= (unsigned)(a.n_tiles_n * a.n_tiles_m * a.splits)) return;
     const unsigned hook_blocks = p.hook_blocks ? p.hook_blocks : gridDim.x;
     paella::hook_entry(p.notifier, p.job_id, hook_blocks);
     // Waves of this workgroup whose result stores have been acknowledged (see the end of this function); cleared here, and
     // the barrier of the cross-wave sum lies between this store and the first increment.
     __shared__ unsigned waves_done;
-    if (KW > 1 && threadIdx.x == 0) waves_done = 0;
 
     // One LDS region, used first for the k -> offset table and, after the reduction loop, for the partial tiles.
     extern __shared__ __align__(16) char smem[];
@@ -178,8 +178,18 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and the compiler may know it
+    if (KW > 1 && wave == 0) waves_done = 0;  // every lane of the first wave stores the same zero: no compare on the vector unit
+    // One lane of the workgroup, tested afresh at each use: held from the first use to the last, the lane mask costs two scalar
+    // registers that the loop has no room for (they went to a vector register's lanes and back, a vector instruction each way).
+    auto first_thread = [&]() {
+        int l = lane, w = wave;
+        asm volatile("" : "+v"(l), "+s"(w));
+        return w == 0 && l == 0;
+    };
     const int j = lane & 31;
     const int kk = lane >> 5;
+    // 0 or -1: a product of kk and a wave-uniform value is then one `and` (a 32-bit vector multiply takes four passes)
+    const int negkk = -kk;
     // Workgroup -> (pixel tile, channel tile, reduction split).  Workgroup ids go round-robin over the eight
     // XCDs, each with its own L2; the ids that land on one XCD are given a contiguous run of the work list, and
     // the list is ordered so that a run shares what the layer reads most of: the same slab of weights (layers
@@ -190,21 +200,28 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         const unsigned xcd = bid & 7u, j = bid >> 3;
         const unsigned q = total >> 3, r = total & 7u;
         const unsigned w = a.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
-        if (a.slab_major) {
-            const unsigned slab = quot(w, (unsigned)a.n_tiles_n, a.div_w, a.fast_div);
-            tile_n = (int)(w - slab * (unsigned)a.n_tiles_n);
-            split = (int)quot(slab, (unsigned)a.n_tiles_m, a.div_tm, a.fast_div);
-            tile_m = (int)(slab - (unsigned)split * (unsigned)a.n_tiles_m);
-        } else {
-            const unsigned per_n = (unsigned)(a.n_tiles_m * a.splits);
-            tile_n = (int)quot(w, per_n, a.div_w, a.fast_div);
-            const unsigned rest = w - (unsigned)tile_n * per_n;
-            split = (int)quot(rest, (unsigned)a.n_tiles_m, a.div_tm, a.fast_div);
-            tile_m = (int)(rest - (unsigned)split * (unsigned)a.n_tiles_m);
-        }
+        // (one scalar branch on fast_div around the whole decode: tested inside each quotient it ends up as a per-lane select)
+        auto decode = [&](auto div) {
+            if (a.slab_major) {
+                const unsigned slab = div(w, (unsigned)a.n_tiles_n, a.div_w);
+                tile_n = (int)(w - slab * (unsigned)a.n_tiles_n);
+                split = (int)div(slab, (unsigned)a.n_tiles_m, a.div_tm);
+                tile_m = (int)(slab - (unsigned)split * (unsigned)a.n_tiles_m);
+            } else {
+                const unsigned per_n = (unsigned)(a.n_tiles_m * a.splits);
+                tile_n = (int)div(w, per_n, a.div_w);
+                const unsigned rest = w - (unsigned)tile_n * per_n;
+                split = (int)div(rest, (unsigned)a.n_tiles_m, a.div_tm);
+                tile_m = (int)(rest - (unsigned)split * (unsigned)a.n_tiles_m);
+            }
+        };
+        // (readfirstlane: the compiler takes the result of an asm statement for a per-lane value and would test it on the vector unit)
+        if (__builtin_amdgcn_readfirstlane(a.fast_div)) decode([](unsigned x, unsigned, const FastDiv& f) { return quot_fast(x, f); });
+        else decode([](unsigned x, unsigned d, const FastDiv&) { return x / d; });
     }
     const int m0 = tile_m * (32 * MI);
     const int n0 = tile_n * (32 * NI);
+    TL_STAMP(9);
 
     // The input through a descriptor that starts pad_off bytes in front of the tensor, pad_off = (pad_h * W + pad_w) * 4: a lane's
     // offset is then that of input element (ho * stride_h, wo * stride_w) -- never negative, so a filter tap's offset
@@ -212,23 +229,34 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const unsigned pad_off = TAP_MAJOR ? (unsigned)(p.ph * p.W + p.pw) * 4u : 0u;
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(p.x) - pad_off), 0, p.x_bytes + pad_off, 0x00027000);
 
+    const unsigned plane = (unsigned)p.PQ * 4u;  // bytes of one output channel
+    // A lane's offset within its tile's output channels (see the output addressing below), one per pixel tile, computed once and held (as the result of an empty asm
+    // statement: the compiler otherwise works it out again at each of its four uses, four vector instructions a time).
+    int lane_offs[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int pix = n0 + ni * 32 + j;
+        lane_offs[ni] = pix < p.PQ ? (int)((unsigned)(negkk & (int)(4u * plane)) + (unsigned)pix * 4u) : (int)0x80000000u;
+        asm volatile("" : "+v"(lane_offs[ni]));
+    }
     const int HW4 = p.H * p.W * 4;
-    const int kk4hw = kk * 4 * HW4;
+    const int kk4hw = negkk & (4 * HW4);
     int hb[NI], wb[NI], base[NI];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int pix = n0 + ni * 32 + j;
         if (PW) {  // input pixel = output pixel
             hb[ni] = wb[ni] = 0;
-            base[ni] = pix < p.PQ ? pix * 4 + kk4hw : -1;
+            base[ni] = lane_offs[ni];  // H * W = P * Q here: the same offset, out of range (negative) past the last pixel
             continue;
         }
-        const int ho = (int)quot((unsigned)pix, (unsigned)p.Q, p.div_q, a.fast_div);
+        const int ho = __builtin_amdgcn_readfirstlane(a.fast_div) ? (int)quot_fast((unsigned)pix, p.div_q) : (int)((unsigned)pix / (unsigned)p.Q);
         const int wo = pix - __mul24(ho, p.Q);  // every factor here is a pixel coordinate or an extent: far below 2^23
         hb[ni] = (pix < p.PQ) ? __mul24(ho, p.sh) - p.ph : -0x100000;
         wb[ni] = __mul24(wo, p.sw) - p.pw;
         base[ni] = (__mul24(hb[ni], p.W) + wb[ni]) * 4 + (TAP_MAJOR ? (int)pad_off + kk4hw : 0);
     }
+    TL_STAMP(10);
 
     // Reduction range of this workgroup (grid-level split), then of this wave inside it.
     const int g_begin = split * p.chunks_per_split;
@@ -258,7 +286,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // (the same descriptor with length zero: choosing between the two is then one scalar select, on the length word)
     const char* const x_base = reinterpret_cast<const char*>(p.x) - pad_off;
     const unsigned x_len = p.x_bytes + pad_off, w_len = p.w_bytes;
-    const int wlane = (int)(((unsigned)kk * (unsigned)p.m_pad + (unsigned)(m0 + j)) * 16u);
+    const int wlane = (int)(((unsigned)(negkk & p.m_pad) + (unsigned)(m0 + j)) * 16u);
     const int wstep = p.m_pad * 32;  // bytes of weights per chunk and row block: two reduction steps of m_pad rows of 16 bytes
     int tap_voff[NI];
     bool tap_ok[NI];
@@ -299,7 +327,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
 #pragma unroll
                 for (int t = 0; t < 4; ++t) f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, voff, chunk_off + t * HW4, 0));
                 if (PRE) {  // a tap outside the image gets scale = shift = 0, so it stays the zero the padding asks for
-                    const bool inside = PW ? base[ni] != -1 : tap_ok[ni];
+                    const bool inside = PW ? base[ni] >= 0 : tap_ok[ni];
                     const int soff = (valid & inside) ? (cb * 8 + kk * 4) * 4 : -1;
                     f.sc = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(sres, soff, 0, 0));
                     f.sh = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(hres, soff, 0, 0));
@@ -366,17 +394,12 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // any length for a pixel past P*Q -- and the hardware holds the sum against the descriptor's length: rows at or past K and
     // pixels past P*Q read as zero and their stores are dropped, without a compare on the vector unit.
     // (K * P * Q * 4 < 2^31 is a condition of the plan.)
-    const unsigned plane = (unsigned)p.PQ * 4u;
-    auto row_of = [&](int rr) {
-        const int r = wave * RPW + rr;
+    auto row_of = [&](int w, int rr) {
+        const int r = w * RPW + rr;
         const int e = r & 15;
         return ((r >> 4) / NI) * 32 + (e >> 2) * 8 + (e & 3);
     };
-    auto lane_off = [&](int rr) {  // the same registers for every rr of one pixel tile (one tile unless the wave owns several)
-        const int ni = ((wave * RPW + rr) >> 4) % NI;
-        const int pix = n0 + ni * 32 + j;
-        return pix < p.PQ ? (int)((unsigned)kk * 4u * plane + (unsigned)pix * 4u) : (int)0x80000000u;
-    };
+    auto lane_off = [&](int rr) { return lane_offs[((wave * RPW + rr) >> 4) % NI]; };
     const int rows_tile = max(p.K - m0, 0);  // channels from this tile's first one to the last that exists (may exceed the tile)
     const float* const res_tile = p.residual ? p.residual + (size_t)m0 * p.PQ : nullptr;
     float* const y_tile = p.y + (size_t)m0 * p.PQ;
@@ -390,14 +413,21 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     auto chan_rsrc = [&](const float* per_channel, int) {  // bias, slope: one float per channel
         return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, chan_len, 0x00027000);
     };
-    int plane_soffs[RPW], chan_soffs[RPW];
+    // Worked out twice, before the loop for the operands requested there and again after it (from a wave number the compiler
+    // cannot tell is the same): held across the loop, these scalars had no register left and went to a vector register's lanes
+    // and back -- a vector instruction and a wait each way, where a dozen scalar instructions do.
+    struct RowOffsets {
+        int plane[RPW], chan[RPW];
+    };
+    auto row_offsets = [&](int w) {
+        RowOffsets o;
 #pragma unroll
-    for (int rr = 0; rr < RPW; ++rr) {
-        plane_soffs[rr] = (int)min((unsigned)row_of(rr) * plane, tile_len);
-        chan_soffs[rr] = (int)min((unsigned)row_of(rr) * 4u, chan_len);
-    }
-    auto plane_soff = [&](int rr) { return plane_soffs[rr]; };
-    auto chan_soff = [&](int rr) { return chan_soffs[rr]; };
+        for (int rr = 0; rr < RPW; ++rr) {
+            o.plane[rr] = (int)min((unsigned)row_of(w, rr) * plane, tile_len);
+            o.chan[rr] = (int)min((unsigned)row_of(w, rr) * 4u, chan_len);
+        }
+        return o;
+    };
     const int chan_voff = kk * 16;
     // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
     // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
@@ -405,10 +435,11 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     float bias_v[RPW], res_v[RPW];
     auto prefetch_epilogue = [&]() {
         if (!kPrefetchEpilogue) return;
+        const RowOffsets o = row_offsets(wave);
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
-            res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), plane_soff(rr), 0)) : 0.f;
+            bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0)) : 0.f;
+            res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0)) : 0.f;
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -450,7 +481,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // nothing alone and nothing or -10 % with four passes in flight: 15.8 / 14.2 / 15.8 thousand ResNet-18 passes per second.
     // The opposite, priority 3 outside the loop so that prologues and epilogues get their few vector instructions in between
     // other waves' matrix instructions: +2 % with the device full while a wave still executed some 130 vector instructions
-    // around its loop, -1 % everywhere once those were down to about 70.)
+    // around its loop, -1 % everywhere once those were down to about 70; at 56: priority 2 from entry to the first operand
+    // requests -4 % with the device full and -2 % served, priority for the loop, for the epilogue or for both within +-0.5 %.)
     TL_STAMP(1);
     if (c_begin < c_end) {
         Frag<MI, NI> frag[D];
@@ -458,6 +490,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         for (int d = 0; d < D; ++d) {
             load_frag(c_begin + d, c_begin + d < c_end, frag[d]);
             __builtin_amdgcn_sched_barrier(0);  // same issue order as in the steady state
+#ifdef PAELLA_CONV_TIMELINE
+            if (d < 2) TL_STAMP(11 + d);
+#endif
         }
         prefetch_epilogue();
         TL_STAMP(2);
@@ -512,13 +547,21 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // to back: a load between two stores would make the compiler wait for the earlier store as well (one counter
     // covers both), and a write-through store takes about 0.3 us to be acknowledged.
     auto epilogue_all = [&](float (&v)[RPW]) {
+        int wave_again = wave;
+        asm volatile("" : "+s"(wave_again));
+        const RowOffsets o = row_offsets(wave_again);
+        const int act = p.act;  // wave-uniform: one scalar branch per kind of activation around straight-line code for all registers
         float sl[RPW];
+        if (act == PAELLA_ACT_PRELU) {
 #pragma unroll
-        for (int rr = 0; rr < RPW; ++rr) {
-            sl[rr] = p.act == PAELLA_ACT_PRELU ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.slope, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
-            if (!kPrefetchEpilogue) {
-                bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, chan_soff(rr), 0)) : 0.f;
-                res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), plane_soff(rr), 0)) : 0.f;
+            for (int rr = 0; rr < RPW; ++rr)
+                sl[rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.slope, rr), chan_voff, o.chan[rr], 0));
+        }
+        if (!kPrefetchEpilogue) {
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) {
+                bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0)) : 0.f;
+                res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0)) : 0.f;
             }
         }
 #pragma unroll
@@ -526,11 +569,23 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             v[rr] += bias_v[rr];
             v[rr] += res_v[rr];
         }
+        if (act == PAELLA_ACT_RELU) {
 #pragma unroll
-        for (int rr = 0; rr < RPW; ++rr) v[rr] = apply_act(v[rr], p.act, sl[rr], p.lo, p.hi);
+            for (int rr = 0; rr < RPW; ++rr) v[rr] = fmaxf(v[rr], 0.f);
+        } else if (act == PAELLA_ACT_RELU6) {
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) v[rr] = fminf(fmaxf(v[rr], 0.f), 6.f);
+        } else if (act == PAELLA_ACT_PRELU) {
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) v[rr] = v[rr] > 0.f ? v[rr] : v[rr] * sl[rr];
+        } else if (act == PAELLA_ACT_CLIP) {
+            const float lo = p.lo, hi = p.hi;
+#pragma unroll
+            for (int rr = 0; rr < RPW; ++rr) v[rr] = fminf(fmaxf(v[rr], lo), hi);
+        }
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr)  // write-through (sc1), like store_out
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[rr]), plane_rsrc(y_tile, rr), lane_off(rr), plane_soff(rr), 16);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[rr]), plane_rsrc(y_tile, rr), lane_off(rr), o.plane[rr], 16);
     };
 
     TL_STAMP(4);
@@ -552,12 +607,14 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     red[((wave * NACC) + (mi * NI + ni) * 16 + e) * 64 + lane] = acc[mi][ni][e];
+        TL_STAMP(13);
         __syncthreads();
+        TL_STAMP(14);
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            float v = 0.f;
+            float v = red[(wave * RPW + rr) * 64 + lane];  // wave order: the sum does not depend on which wave finished first
 #pragma unroll
-            for (int w = 0; w < KW; ++w) v += red[((w * NACC) + wave * RPW + rr) * 64 + lane];
+            for (int w = 1; w < KW; ++w) v += red[((w * NACC) + wave * RPW + rr) * 64 + lane];
             mine[rr] = v;
         }
     }
@@ -573,10 +630,16 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         // the partial tile is in memory, ahead of the counter bump that follows the barrier; the last arriver reads the
         // partials with device-scope atomic loads, which do not hit in its own caches.  A release on the bump and an acquire
         // after it would add a cache write-back and an invalidate per workgroup for data that never sat in a cache.
+        // Everything the last arriver needs is read here, ahead of the counter bump, and the arrival number is made wave-uniform
+        // for the compiler: fetched again after an atomic inside a one-lane branch, the split count and the pointers counted as
+        // per-lane values, and every load through a descriptor built from them was wrapped in a loop over the lanes' values.
+        const int nsplits = __builtin_amdgcn_readfirstlane(p.splits);
         const int tile = tile_m * p.n_tiles_n + tile_n;
+        unsigned* const counter = p.ws_counters + tile;
         // the tile's partial tiles, [split][NACC][64 lanes]: one descriptor, a lane's offset is its lane number
-        const __amdgpu_buffer_rsrc_t pres = __builtin_amdgcn_make_buffer_rsrc((void*)(p.ws_partials + (size_t)tile * p.splits * (NACC * 64)), 0,
-                                                                               (unsigned)p.splits * (NACC * 256u), 0x00027000);
+        float* const partials = p.ws_partials + (size_t)tile * nsplits * (NACC * 64);
+        const unsigned partials_len = (unsigned)nsplits * (NACC * 256u);
+        const __amdgpu_buffer_rsrc_t pres = __builtin_amdgcn_make_buffer_rsrc((void*)partials, 0, partials_len, 0x00027000);
         const int lane4 = lane * 4;
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr)
@@ -584,31 +647,42 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         __shared__ unsigned arrived;
-        if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(p.ws_counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (first_thread()) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (arrived == (unsigned)p.splits - 1) {
+        if (__builtin_amdgcn_readfirstlane(arrived) == (unsigned)nsplits - 1) {
             float v[RPW];
 #pragma unroll
             for (int rr = 0; rr < RPW; ++rr) v[rr] = 0.f;
-            constexpr int ZB = RPW <= 4 ? 8 : (RPW <= 16 ? 4 : 1);  // partial tiles requested together
-            for (int z0 = 0; z0 < p.splits; z0 += ZB) {
-                float t[ZB][RPW];
+            // Partial tiles are requested in batches (eight, then four, two, one: as many as are left, all in flight together) and
+            // added in split order: the sum does not depend on which workgroup came last.  Device scope (sc1): they were written
+            // by other workgroups and must not come from this one's caches.
+            auto add_batch = [&](int z0, auto batch) {
+                constexpr int Z = decltype(batch)::value;
+                float t[Z][RPW];
 #pragma unroll
-                for (int u = 0; u < ZB; ++u) {
-                    // a split past the last one reads through a descriptor of zero length (zeros, no memory touched); device
-                    // scope (sc1): the partial tiles were written by other workgroups and must not come from this one's caches
-                    const __amdgpu_buffer_rsrc_t zr = z0 + u < p.splits ? pres : __builtin_amdgcn_make_buffer_rsrc((void*)p.ws_partials, 0, 0, 0x00027000);
+                for (int u = 0; u < Z; ++u)
 #pragma unroll
                     for (int rr = 0; rr < RPW; ++rr)
-                        t[u][rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(zr, lane4, ((z0 + u) * NACC + wave * RPW + rr) * 256, 16));
-                }
+                        t[u][rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pres, lane4, ((z0 + u) * NACC + wave * RPW + rr) * 256, 16));
 #pragma unroll
-                for (int u = 0; u < ZB; ++u)  // split order: the sum does not depend on which workgroup came last
+                for (int u = 0; u < Z; ++u)
 #pragma unroll
                     for (int rr = 0; rr < RPW; ++rr) v[rr] += t[u][rr];
+            };
+            constexpr int ZB = RPW <= 4 ? 8 : (RPW <= 16 ? 4 : 1);  // the largest batch the registers have room for
+            int z0 = 0;
+            for (; z0 + ZB <= nsplits; z0 += ZB) add_batch(z0, std::integral_constant<int, ZB>{});
+            if (ZB > 4 && nsplits - z0 >= 4) {
+                add_batch(z0, std::integral_constant<int, 4>{});
+                z0 += 4;
             }
+            if (ZB > 2 && nsplits - z0 >= 2) {
+                add_batch(z0, std::integral_constant<int, 2>{});
+                z0 += 2;
+            }
+            if (ZB > 1 && nsplits - z0 >= 1) add_batch(z0, std::integral_constant<int, 1>{});
             epilogue_all(v);
-            if (threadIdx.x == 0) __hip_atomic_store(p.ws_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (first_thread()) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 
@@ -620,7 +694,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         const unsigned widx = bid * KW + (unsigned)wave;
         if (lane == 0 && g_tl_buf && widx < g_tl_cap) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) g_tl_buf[(size_t)widx * 8 + i] = tl[i];
+            for (int i = 0; i < 16; ++i) g_tl_buf[(size_t)widx * 16 + i] = tl[i];
         }
     }
 #endif
