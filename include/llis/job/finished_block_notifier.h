@@ -106,7 +106,7 @@ class FinishedBlockNotifier {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if ((threadIdx.x | threadIdx.y | threadIdx.z) == 0) {
-            if (timed && measure_block_time_) send_block_time_first();  // the member is looked at only when timing was asked for
+            if (timed && timing_is_on()) send_block_time_first();  // the member is looked at only when timing was asked for
             announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
         }
     }
@@ -118,7 +118,7 @@ class FinishedBlockNotifier {
         end_from_one_lane(job_id, timed, gridDim.x * gridDim.y * gridDim.z);
     }
     __device__ __forceinline__ void end_from_one_lane(JobId job_id, bool timed, unsigned num_blocks) {
-        if (timed && measure_block_time_) send_block_time_first();
+        if (timed && timing_is_on()) send_block_time_first();
         announce<false>(&agg_counter_end_, 0, job_id, num_blocks);
     }
 #endif
@@ -138,6 +138,10 @@ class FinishedBlockNotifier {
         __shared__ unsigned entry_clock;
         return &entry_clock;
     }
+
+    // The flag through a volatile access: an ordinary load is hoisted above the test of `timed`, and a workgroup that was not
+    // asked for timing then waits for a trip to memory of its own before it may count itself in.
+    __device__ __forceinline__ bool timing_is_on() const { return *const_cast<const volatile unsigned*>(&measure_block_time_) != 0; }
 
     __device__ __forceinline__ void send_block_time() {
         const unsigned s = *entry_clock_slot();

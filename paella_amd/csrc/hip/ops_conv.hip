@@ -200,20 +200,17 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         const unsigned xcd = bid & 7u, j = bid >> 3;
         const unsigned q = total >> 3, r = total & 7u;
         const unsigned w = a.slab_major == 2 ? bid : xcd * q + (xcd < r ? xcd : r) + j;  // 2: plain order (experiments)
-        // (one scalar branch on fast_div around the whole decode: tested inside each quotient it ends up as a per-lane select)
+        // Both orders are one division of the work-list position and one of its quotient or remainder, so the order only selects
+        // (scalar selects, no branch; branches here came out as a flag in a vector register tested on the vector unit).
         auto decode = [&](auto div) {
-            if (a.slab_major) {
-                const unsigned slab = div(w, (unsigned)a.n_tiles_n, a.div_w);
-                tile_n = (int)(w - slab * (unsigned)a.n_tiles_n);
-                split = (int)div(slab, (unsigned)a.n_tiles_m, a.div_tm);
-                tile_m = (int)(slab - (unsigned)split * (unsigned)a.n_tiles_m);
-            } else {
-                const unsigned per_n = (unsigned)(a.n_tiles_m * a.splits);
-                tile_n = (int)div(w, per_n, a.div_w);
-                const unsigned rest = w - (unsigned)tile_n * per_n;
-                split = (int)div(rest, (unsigned)a.n_tiles_m, a.div_tm);
-                tile_m = (int)(rest - (unsigned)split * (unsigned)a.n_tiles_m);
-            }
+            const bool slabs = a.slab_major != 0;
+            const unsigned d_w = slabs ? (unsigned)a.n_tiles_n : (unsigned)(a.n_tiles_m * a.splits);
+            const unsigned q = div(w, d_w, a.div_w);
+            const unsigned r = w - q * d_w;
+            const unsigned rest = slabs ? q : r;  // slab number (channel tile and split), or position within the pixel tile's share
+            tile_n = (int)(slabs ? r : q);
+            split = (int)div(rest, (unsigned)a.n_tiles_m, a.div_tm);
+            tile_m = (int)(rest - (unsigned)split * (unsigned)a.n_tiles_m);
         };
         // (readfirstlane: the compiler takes the result of an asm statement for a per-lane value and would test it on the vector unit)
         if (__builtin_amdgcn_readfirstlane(a.fast_div)) decode([](unsigned x, unsigned, const FastDiv& f) { return quot_fast(x, f); });
