@@ -748,12 +748,18 @@ struct ConvPreGroupArgs {
 
 template <int KW>
 __global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_pre_group_kernel(ConvPreGroupArgs g) {
+    // The member's first workgroup id is carried along with its number: looked up afterwards, it is one more trip to the argument
+    // block before the member's own arguments can be requested.
     int idx = 0;
+    unsigned first = g.start[0];
 #pragma unroll
     for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
-        if (blockIdx.x >= g.start[i]) idx = i;
-    if (g.m[idx].conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
-    else conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - g.start[idx], g.m[idx].pre);
+        if (blockIdx.x >= g.start[i]) {
+            idx = i;
+            first = g.start[i];
+        }
+    if (g.m[idx].conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(g.m[idx].conv, blockIdx.x - first, g.m[idx].pre);
+    else conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - first, g.m[idx].pre);
 }
 
 // Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
@@ -787,10 +793,14 @@ struct ConvGroupArgs {
 template <int KW, bool TAP_MAJOR>
 __global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_group_kernel(ConvGroupArgs g) {
     int idx = 0;
+    unsigned first = g.start[0];  // carried along: see conv_mfma_pre_group_kernel
 #pragma unroll
     for (int i = 1; i < kPackMax; ++i)
-        if (blockIdx.x >= g.start[i]) idx = i;
-    const unsigned bid = blockIdx.x - g.start[idx];
+        if (blockIdx.x >= g.start[i]) {
+            idx = i;
+            first = g.start[i];
+        }
+    const unsigned bid = blockIdx.x - first;
     const unsigned kind = (g.kinds >> (2 * idx)) & 3u;
     if (kind == kMemberPool) {
         const paella::PoolArgs& p = g.m[idx].pool;
@@ -916,12 +926,16 @@ struct DwGroupArgs {
 
 __global__ __launch_bounds__(256) void dwconv_group_kernel(DwGroupArgs g) {
     int member = 0;
+    unsigned first = g.start[0], grid = g.grids[0];  // carried along: see conv_mfma_pre_group_kernel
 #pragma unroll
     for (int i = 1; i < PAELLA_CONV_PACK_MAX; ++i)
-        if (blockIdx.x >= g.start[i]) member = i;
+        if (blockIdx.x >= g.start[i]) {
+            member = i;
+            first = g.start[i];
+            grid = g.grids[i];
+        }
     const DwArgs& p = g.m[member];
-    const unsigned grid = g.grids[member];
-    const unsigned bid = blockIdx.x - g.start[member];
+    const unsigned bid = blockIdx.x - first;
     paella::hook_entry(p.notifier, p.job_id, grid);
     const int PQ = p.P * p.Q;
     const int total = p.C * PQ;
@@ -1184,7 +1198,7 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     a.x_bytes = (unsigned)((size_t)d.C * d.H * d.W * 4);
     a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
     a.job_id = job_id;
-    a.hook_blocks = 0;
+    a.hook_blocks = plan->dims.grid;  // a launch of its own: all of its workgroups (0 would make the kernel fetch the grid size itself)
     a.notifier = nf;
     a.n_tiles_n = (PQ + 32 * plan->ni - 1) / (32 * plan->ni);
     a.n_tiles_m = plan->m_pad / (32 * plan->mi);
@@ -1498,7 +1512,7 @@ int pack_send(PackList& list, int kw, int k_order, bool only_full) {
         }
         if (n == 1) {  // nothing to share the launch with: the plain kernel, whose argument block is a quarter of the group's
             ConvKernel kern = pick_kernel(1, 1, kw, k_order);
-            g.m[0].conv.hook_blocks = 0;
+            g.m[0].conv.hook_blocks = grid;
             rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds);
             if (rc == 0) {
                 paella::launch(kern, dim3(grid), dim3(64u * (unsigned)kw), dyn_lds, reinterpret_cast<hipStream_t>(target), g.m[0].conv);
@@ -1552,7 +1566,7 @@ int seq_launch_position(const std::vector<Sequence>& seqs, size_t first, int n, 
     g_pack_members.fetch_add((uint64_t)n, std::memory_order_relaxed);
     if (n == 1 && head.kind == kMemberConv) {
         ConvKernel kern = pick_kernel(1, 1, head.kw, head.k_order);
-        g.m[0].conv.hook_blocks = 0;
+        g.m[0].conv.hook_blocks = grid;
         if (int rc = allow_lds(reinterpret_cast<const void*>(kern), dyn_lds)) return rc;
         paella::launch(kern, dim3(grid), dim3(64u * (unsigned)head.kw), dyn_lds, reinterpret_cast<hipStream_t>(queue), g.m[0].conv);
         return (int)hipGetLastError();
@@ -2011,7 +2025,7 @@ int pre_send_all(bool only_full) {
             } else if (n == 1) {
                 ConvPreKernel kern = pick_pre_kernel(kw);
                 ConvPreArgs a = list[done].a;
-                a.conv.hook_blocks = 0;
+                a.conv.hook_blocks = list[done].grid;
                 rc = allow_lds(reinterpret_cast<const void*>(kern), list[done].dyn_lds);
                 if (rc == 0) {
                     paella::launch(kern, dim3(list[done].grid), dim3(64u * (unsigned)kw), list[done].dyn_lds, reinterpret_cast<hipStream_t>(target), a);
