@@ -448,7 +448,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // waves hide the latency that a deeper pipeline would.  Three slots with the refill issued ahead of the current
     // chunk's matrix instructions were no better either (23.8 against 24.9 TFLOP/s over a ResNet-18 pass): the loop is
     // bound by what the compute unit's vector cache can take in -- each wave fetches its own 32 x 8 operand
-    // fragments, 147 KB per workgroup for a 64-channel 3x3 layer -- not by exposed latency.
+    // fragments, 147 KB per workgroup for a 64-channel 3x3 layer -- not by exposed latency.  (Again once the kernel had shrunk to
+    // 44 registers, so that depth 3 and 4 fit eight waves per SIMD at 52 and 60: 76.8 and 76.4 against 78.1 TFLOP/s with the
+    // device full.  Requesting one input dword per chunk instead of four -- wrong results, timing only -- gives 84 against 77:
+    // the load path is worth at most 9 % here, and half again on the stride-2 layers, whose lanes use every other pixel of a line.)
     constexpr int D = DEPTH ? DEPTH : (MI * NI == 1) ? 2 : 4;
     // first: the accumulators hold nothing yet, the first matrix instruction into each takes zero as its addend
     auto compute = [&](const Frag<MI, NI>& f, auto first) {
