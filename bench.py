@@ -59,7 +59,7 @@ def log(*a):
 # HBM-side bytes per conv launch (mean over the conv launches of one forward pass), from FETCH_SIZE / WRITE_SIZE
 # counter passes of `bench.py --counter-pass MODEL` scaled by the copy-kernel calibration (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); counters cannot be collected from inside this process, so the figures are carried here.
-CONV_TRAFFIC_BYTES_PER_LAUNCH = {"inception_v3": 8.64e6, "resnet18": 6.99e6, "resnet50": 7.11e6, "mobilenetv2": 1.88e6}
+CONV_TRAFFIC_BYTES_PER_LAUNCH = {"inception_v3": 8.63e6, "resnet18": 6.97e6, "resnet50": 7.06e6, "mobilenetv2": 1.84e6}
 
 
 def under_counter_collection():
