@@ -188,8 +188,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     };
     const int j = lane & 31;
     const int kk = lane >> 5;
-    // 0 or -1: a product of kk and a wave-uniform value is then one `and` (a 32-bit vector multiply takes four passes)
-    const int negkk = -kk;
+    // 0 or -1 (one signed bit-field extract): a product of kk and a wave-uniform value is then one `and` (a 32-bit vector
+    // multiply takes four passes)
+    const int negkk = (int)((unsigned)lane << 26) >> 31;
     // Workgroup -> (pixel tile, channel tile, reduction split).  Workgroup ids go round-robin over the eight
     // XCDs, each with its own L2; the ids that land on one XCD are given a contiguous run of the work list, and
     // the list is ordered so that a run shares what the layer reads most of: the same slab of weights (layers
@@ -406,9 +407,11 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // tensor; what changes with the register is a scalar offset of two instructions.
     const unsigned tile_len = (unsigned)rows_tile * plane;
     const unsigned chan_len = (unsigned)rows_tile * 4u;
-    auto plane_rsrc = [&](const float* tile_base, int) { return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, tile_len, 0x00027000); };
+    // An operand that is not there (no bias, no residual) is read through a descriptor of length zero: zeros without a branch, a
+    // register move and a memory access.
+    auto plane_rsrc = [&](const float* tile_base, int) { return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, tile_base ? tile_len : 0u, 0x00027000); };
     auto chan_rsrc = [&](const float* per_channel, int) {  // bias, slope: one float per channel
-        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, chan_len, 0x00027000);
+        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, per_channel ? chan_len : 0u, 0x00027000);
     };
     // Worked out twice, before the loop for the operands requested there and again after it (from a wave number the compiler
     // cannot tell is the same): held across the loop, these scalars had no register left and went to a vector register's lanes
@@ -425,7 +428,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         }
         return o;
     };
-    const int chan_voff = kk * 16;
+    const int chan_voff = negkk & 16;
     // The wave finally owns RPW of the tile's NACC accumulator registers (summed over the KW waves).  Request
     // the epilogue's operands for them now, so that their latency hides behind the reduction loop.
     // (requested once the first chunks' operand loads are out: the loop cannot start before those arrive)
@@ -435,8 +438,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         const RowOffsets o = row_offsets(wave);
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0)) : 0.f;
-            res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0)) : 0.f;
+            bias_v[rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0));
+            res_v[rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0));
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -560,8 +563,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         if (!kPrefetchEpilogue) {
 #pragma unroll
             for (int rr = 0; rr < RPW; ++rr) {
-                bias_v[rr] = p.bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0)) : 0.f;
-                res_v[rr] = res_tile ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0)) : 0.f;
+                bias_v[rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(chan_rsrc(p.bias, rr), chan_voff, o.chan[rr], 0));
+                res_v[rr] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane_rsrc(res_tile, rr), lane_off(rr), o.plane[rr], 0));
             }
         }
 #pragma unroll
@@ -612,7 +615,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         TL_STAMP(14);
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            float v = red[(wave * RPW + rr) * 64 + lane];  // wave order: the sum does not depend on which wave finished first
+            float v = red[((0 * NACC) + wave * RPW + rr) * 64 + lane];  // wave order: the sum does not depend on which wave finished first
 #pragma unroll
             for (int w = 1; w < KW; ++w) v += red[((w * NACC) + wave * RPW + rr) * 64 + lane];
             mine[rr] = v;
