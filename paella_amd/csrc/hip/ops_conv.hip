@@ -259,7 +259,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // Reduction range of this workgroup (grid-level split), then of this wave inside it.
     const int g_begin = split * p.chunks_per_split;
     const int g_end = min(p.nchunks, g_begin + p.chunks_per_split);
-    const int cpw = (g_end - g_begin + KW - 1) / KW;
+    const int cpw = (int)((unsigned)(g_end - g_begin + KW - 1) / (unsigned)KW);  // the plan leaves no split empty: never negative
     const int c_begin = g_begin + wave * cpw;
     const int c_end = min(g_end, c_begin + cpw);
 
@@ -411,7 +411,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // register move and a memory access.
     auto plane_rsrc = [&](const float* tile_base, int) { return __builtin_amdgcn_make_buffer_rsrc((void*)tile_base, 0, tile_base ? tile_len : 0u, 0x00027000); };
     auto chan_rsrc = [&](const float* per_channel, int) {  // bias, slope: one float per channel
-        return __builtin_amdgcn_make_buffer_rsrc((void*)(per_channel + m0), 0, per_channel ? chan_len : 0u, 0x00027000);
+        // (the base as an integer sum: arithmetic on a null pointer would let the compiler conclude that it is not null)
+        return __builtin_amdgcn_make_buffer_rsrc((void*)((uintptr_t)per_channel + (uintptr_t)m0 * 4u), 0, per_channel ? chan_len : 0u, 0x00027000);
     };
     // Worked out twice, before the loop for the operands requested there and again after it (from a wave number the compiler
     // cannot tell is the same): held across the loop, these scalars had no register left and went to a vector register's lanes
