@@ -847,6 +847,11 @@ struct DwArgs {
     float lo, hi;
     uint32_t job_id;
     llis::job::FinishedBlockNotifier* notifier;
+    // 3 x 3 filters whose sizes the host has checked (fast = 1): output column and row by multiply-high, operands through buffer
+    // descriptors with 32-bit offsets
+    FastDiv div_q, div_p;
+    int fast;
+    unsigned x_bytes, out_bytes;
 };
 
 // All taps of one output element.  With the filter size known the loads of a window leave back to back (a tap outside the
@@ -906,12 +911,102 @@ __device__ __forceinline__ void dw_element(const DwArgs& p, int idx, int PQ) {
 constexpr int kDwPerThread = 4;
 constexpr int kDwWideFrom = 65536;  // elements from which a thread takes several
 
-__global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
-    paella::hook_entry(p.notifier, p.job_id);
+// K output elements of a 3 x 3 depthwise conv, a grid stride apart, with every operand of all K requested before the first
+// multiply.  Addresses are 32-bit offsets into buffer descriptors: a tap outside the image gets an offset out of range and
+// reads as zero, a thread past the last element computes the last one again and has its store dropped -- no branch and no
+// 64-bit address per load (the plain form above spends some 190 vector instructions per element, most of them on addresses,
+// and waits for memory once per element).  Same taps in the same order: the same bits as dw_element.
+template <int K>
+__device__ __forceinline__ void dw_batch3x3(const DwArgs& p, const int idx, const int stride, const int total) {
+    // the input through a descriptor that starts (pad_h * W + pad_w) elements in front of it, so that a lane's offset -- that of
+    // input element (ho * stride_h, wo * stride_w) of its channel -- is never negative; a tap's share is wave-uniform
+    const unsigned pad_off = (unsigned)(p.ph * p.W + p.pw) * 4u;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(p.x) - pad_off), 0, p.x_bytes + pad_off, 0x00027000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, (unsigned)p.C * 36u, 0x00027000);
+    const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc((void*)p.bias, 0, p.bias ? (unsigned)p.C * 4u : 0u, 0x00027000);
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc((void*)p.residual, 0, p.residual ? p.out_bytes : 0u, 0x00027000);
+    const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc((void*)p.slope, 0, p.act == PAELLA_ACT_PRELU ? (unsigned)p.C * 4u : 0u, 0x00027000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void*)p.y, 0, p.out_bytes, 0x00027000);
+    int tap_soff[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int t = 0; t < 3; ++t) tap_soff[r * 3 + t] = (r * p.dh * p.W + t * p.dw) * 4;
+    float v[K][9], wt[K][9], acc[K], res[K], sl[K];
+    int out_off[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = idx + k * stride;
+        const bool live = i < total;
+        const int e = live ? i : total - 1;
+        const int row = (int)quot_fast((unsigned)e, p.div_q);  // over (channel, output row)
+        // every factor below is under 2^23 (checked by the host): 24-bit multiplies, a quarter of the passes of a 32-bit one
+        const int wo = e - __mul24(row, p.Q);
+        const int c = (int)quot_fast((unsigned)row, p.div_p);
+        const int ho = row - __mul24(c, p.P);
+        const int hs = __mul24(ho, p.sh), ws = __mul24(wo, p.sw);
+        const int h0 = hs - p.ph, w0 = ws - p.pw;
+        const int base = (__mul24(__mul24(c, p.H) + hs, p.W) + ws) * 4;
+        // a row or a column outside the image sets the offset's top bit: beyond any length, the tap reads as zero (three-operand
+        // `or` per tap; flags combined as booleans cost five vector instructions per tap)
+        int row_bad[3], col_bad[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            row_bad[r] = (unsigned)(h0 + r * p.dh) < (unsigned)p.H ? 0 : (int)0x80000000u;
+            col_bad[r] = (unsigned)(w0 + r * p.dw) < (unsigned)p.W ? 0 : (int)0x80000000u;
+        }
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+                v[k][r * 3 + t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, base | row_bad[r] | col_bad[t], tap_soff[r * 3 + t], 0));
+        const int woff = __mul24(c, 36);
+#pragma unroll
+        for (int t = 0; t < 9; ++t) wt[k][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(wr, woff, t * 4, 0));
+        acc[k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, c * 4, 0, 0));
+        out_off[k] = live ? e * 4 : -1;
+        res[k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, out_off[k], 0, 0));
+        sl[k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sr, c * 4, 0, 0));  // length zero unless PReLU
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int t = 0; t < 9; ++t) acc[k] = fmaf(v[k][t], wt[k][t], acc[k]);
+    if (p.residual) {  // (not added as a zero: -0 + 0 is +0)
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] += res[k];
+    }
+    const int act = p.act;  // one scalar branch per kind of activation around all K elements
+    if (act == PAELLA_ACT_RELU) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = fmaxf(acc[k], 0.f);
+    } else if (act == PAELLA_ACT_RELU6) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = fminf(fmaxf(acc[k], 0.f), 6.f);
+    } else if (act == PAELLA_ACT_PRELU) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = acc[k] > 0.f ? acc[k] : acc[k] * sl[k];
+    } else if (act == PAELLA_ACT_CLIP) {
+        const float lo = p.lo, hi = p.hi;
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = fminf(fmaxf(acc[k], lo), hi);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k)  // write-through (sc1), like store_out
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc[k]), yr, out_off[k], 0, 16);
+}
+
+// One workgroup's share of a depthwise conv of `grid` workgroups.
+__device__ __forceinline__ void dw_block(const DwArgs& p, const unsigned bid, const unsigned grid) {
     const int PQ = p.P * p.Q;
     const int total = p.C * PQ;
-    const int stride = (int)gridDim.x * 256;
-    int idx = blockIdx.x * 256 + threadIdx.x;  // over (channel, pixel): small feature maps still fill their workgroups
+    const int stride = (int)grid * 256;
+    int idx = (int)bid * 256 + threadIdx.x;  // over (channel, pixel): small feature maps still fill their workgroups
+    if (p.fast) {
+        if (stride >= total) dw_batch3x3<1>(p, idx, stride, total);
+        else dw_batch3x3<kDwPerThread>(p, idx, stride, total);
+        return;
+    }
     if (stride >= total) {
         if (idx < total) dw_element(p, idx, PQ);
     } else {
@@ -919,6 +1014,11 @@ __global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
         for (int k = 0; k < kDwPerThread; ++k, idx += stride)
             if (idx < total) dw_element(p, idx, PQ);
     }
+}
+
+__global__ __launch_bounds__(256) void dwconv_kernel(DwArgs p) {
+    paella::hook_entry(p.notifier, p.job_id);
+    dw_block(p, blockIdx.x, gridDim.x);
     paella::hook_exit(p.notifier, p.job_id);
 }
 
@@ -944,17 +1044,7 @@ __global__ __launch_bounds__(256) void dwconv_group_kernel(DwGroupArgs g) {
     const DwArgs& p = g.m[member];
     const unsigned bid = blockIdx.x - first;
     paella::hook_entry(p.notifier, p.job_id, grid);
-    const int PQ = p.P * p.Q;
-    const int total = p.C * PQ;
-    const int stride = (int)grid * 256;
-    int idx = (int)bid * 256 + threadIdx.x;
-    if (stride >= total) {
-        if (idx < total) dw_element(p, idx, PQ);
-    } else {
-#pragma unroll
-        for (int k = 0; k < kDwPerThread; ++k, idx += stride)
-            if (idx < total) dw_element(p, idx, PQ);
-    }
+    dw_block(p, bid, grid);
     paella::hook_exit(p.notifier, p.job_id, grid);
 }
 
@@ -1897,6 +1987,19 @@ extern "C" int paella_conv2d_launch(const paella_conv_plan* plan, const float* x
     a.act = d.act; a.lo = d.act_lo; a.hi = d.act_hi;
     a.job_id = job_id;
     a.notifier = nf;
+    {
+        // The batched 3 x 3 form: divisions by multiply-high are exact while dividend x divisor < 2^32 (elements by Q, rows by P),
+        // offsets are 32-bit byte offsets, coordinates go through 24-bit multiplies.
+        const uint64_t elements = (uint64_t)d.C * plan->P * plan->Q, rows = (uint64_t)d.C * plan->P;
+        const uint64_t x_bytes = (uint64_t)d.C * d.H * d.W * 4, pad = ((uint64_t)d.pad_h * d.W + d.pad_w) * 4;
+        a.fast = d.R == 3 && d.S == 3 && elements * (uint64_t)plan->Q < ((uint64_t)1 << 32) && rows * (uint64_t)plan->P < ((uint64_t)1 << 32) &&
+                 x_bytes + pad + (uint64_t)(2 * d.dil_h * d.W + 2 * d.dil_w) * 4 < ((uint64_t)1 << 31) && elements * 4 < ((uint64_t)1 << 31) &&
+                 elements < (1u << 23) && (uint64_t)d.C * d.H < (1u << 23) && d.W < (1 << 23) && plan->Q < (1 << 23) ? 1 : 0;
+        a.div_q = fast_div((unsigned)plan->Q);
+        a.div_p = fast_div((unsigned)plan->P);
+        a.x_bytes = (unsigned)std::min<uint64_t>(x_bytes, 0xFFFFFFFFu);
+        a.out_bytes = (unsigned)std::min<uint64_t>(elements * 4, 0xFFFFFFFFu);
+    }
     if (pack_hold_dw(a, plan->dims.grid, stream)) return 0;
     paella::launch(dwconv_kernel, dim3(plan->dims.grid), dim3(256), 0, st, a);
     return (int)hipGetLastError();
