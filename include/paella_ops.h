@@ -79,7 +79,8 @@ typedef struct paella_conv_plan {
     double flops;                /* algorithmic: 2*K*(C/g)*R*S*P*Q */
     double bytes;                /* algorithmic: 4*(C*H*W + K*(C/g)*R*S + K + K*P*Q [+K*P*Q residual]) */
     int depth;                   /* chunks of operands a wave keeps in flight; 0 = the tile's default */
-    int reserved;
+    int pair_taps;               /* 0, or 1 + the first of two filter columns whose chunks are interleaved in the blob: a stride-2
+                                    3-wide filter reads them as neighbouring input pixels (see the kernel's operand fetch) */
 } paella_conv_plan;
 
 /* Pure host arithmetic: picks the kernel variant and launch shape.  tile_hint = 0 lets the library

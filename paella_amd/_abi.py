@@ -23,7 +23,7 @@ class ConvDesc(ctypes.Structure):
 class ConvPlan(ctypes.Structure):
     _fields_ = [("d", ConvDesc), ("P", c_int), ("Q", c_int), ("kind", c_int), ("mi", c_int), ("ni", c_int),
                 ("kw", c_int), ("splits", c_int), ("m_pad", c_int), ("k_pad", c_int), ("k_order", c_int), ("wg_order", c_int), ("fast_div", c_int), ("blob_bytes", c_size_t), ("workspace_bytes", c_size_t), ("dims", LaunchDims),
-                ("flops", c_double), ("bytes", c_double), ("depth", c_int), ("reserved", c_int)]
+                ("flops", c_double), ("bytes", c_double), ("depth", c_int), ("pair_taps", c_int)]
 
 
 class ConvOperands(ctypes.Structure):

@@ -100,6 +100,7 @@ struct ConvArgs {
     FastDiv div_w, div_tm, div_q, div_cb, div_s;
     int fast_div;
     int pointwise;                  // tap-major only: 1x1 filter, stride 1, no padding
+    int pair_s0;                    // tap-major, 3-wide stride-2 filters: first of the two paired filter columns, or -1 (see load_frag)
 };
 
 // The quotient for dividends and divisors the host has checked; where it could not, the kernel divides (ConvArgs::fast_div).
@@ -290,6 +291,17 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     bool tap_ok[NI];
     bool tap_stale = true;
     int tap_off = 0;  // byte offset of the current filter tap, wave-uniform
+    // Paired filter columns (stride 2 across a 3-wide filter, pair_s0 >= 0).  With stride 2 a lane's pixels are every other
+    // element of a line, so each line fetched delivers half as many operands.  Two neighbouring filter columns read
+    // neighbouring input pixels: for their chunks the half wave selects the COLUMN instead of four more channels -- lane (j, kk)
+    // reads pixel 2 q_j + kk, the 64 lanes of a load cover 64 consecutive elements -- and a chunk holds four channels of both
+    // columns.  The host packs the weights to match: per filter row, CB chunks of the unpaired column (eight channels each), then
+    // 2 CB chunks of the pair (four channels of both columns each), so a row is 3 CB chunks either way and chunk c is still
+    // (unit c / CB, block c % CB).  The host has checked that both columns lie inside the image for every output pixel.
+    const int pair_s0 = (TAP_MAJOR && !PW && MI * NI == 1) ? p.pair_s0 : -1;
+    const int pair_delta = (negkk & (p.dw * 4)) - kk4hw;  // from the lane's offset for a plain chunk to that for a paired one
+    int seg_chan0 = 0, seg_chans = 8;  // first channel of the current unit's chunks, channels per chunk; wave-uniform
+    bool seg_pair = false;
     auto load_frag = [&](int c, bool valid, Frag<MI, NI>& f) {
         if (TAP_MAJOR) {
             const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, valid ? w_len : 0u, 0x00027000);
@@ -306,19 +318,34 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 cb = c - tap * p.CB;
                 if (tap_stale | (cb == 0)) {  // wave-uniform: once per filter tap
                     const int r = (int)quot_fast((unsigned)tap, p.div_s);
-                    const int dy = r * p.dh, dx = (tap - r * p.S) * p.dw;
+                    int col = tap - r * p.S;  // the filter column, or with paired columns the unit's place in its row
+                    seg_pair = false;
+                    seg_chan0 = 0;
+                    seg_chans = 8;
+                    if (pair_s0 >= 0) {
+                        seg_pair = col != 0;                     // places 1 and 2: the two halves of the pair's chunks
+                        seg_chan0 = col == 2 ? p.CB * 4 : 0;
+                        seg_chans = seg_pair ? 4 : 8;
+                        col = seg_pair ? pair_s0 : 2 - 2 * pair_s0;  // the pair's first column; the unpaired one is 2 or 0
+                    }
+                    const int dy = r * p.dh, dx = col * p.dw;
                     tap_off = (dy * p.W + dx) * 4;
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         tap_ok[ni] = ((unsigned)(hb[ni] + dy) < (unsigned)p.H) & ((unsigned)(wb[ni] + dx) < (unsigned)p.W);
                         tap_voff[ni] = tap_ok[ni] ? base[ni] : -1;
                     }
+                    if (seg_pair) {
+#pragma unroll
+                        for (int ni = 0; ni < NI; ++ni) tap_voff[ni] = tap_ok[ni] ? base[ni] + pair_delta : -1;
+                    }
                     tap_stale = false;
                 }
                 tap_soff = tap_off;
             }
             const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void*)x_base, 0, valid ? x_len : 0u, 0x00027000);
-            const int chunk_off = cb * 8 * HW4 + tap_soff;
+            const int chan0 = PW ? cb * 8 : seg_chan0 + cb * seg_chans;  // first channel of the chunk
+            const int chunk_off = chan0 * HW4 + tap_soff;
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
                 const int voff = PW ? base[ni] : tap_voff[ni];
@@ -326,7 +353,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 for (int t = 0; t < 4; ++t) f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, voff, chunk_off + t * HW4, 0));
                 if (PRE) {  // a tap outside the image gets scale = shift = 0, so it stays the zero the padding asks for
                     const bool inside = PW ? base[ni] >= 0 : tap_ok[ni];
-                    const int soff = (valid & inside) ? (cb * 8 + kk * 4) * 4 : -1;
+                    const int soff = (valid & inside) ? (chan0 + ((!PW && seg_pair) ? 0 : kk * 4)) * 4 : -1;
                     f.sc = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(sres, soff, 0, 0));
                     f.sh = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(hres, soff, 0, 0));
                 }
@@ -1207,6 +1234,13 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
         plan->k_pad = k_pad;
         // Reduction order: (r, s, c) when whole chunks of 8 share a filter tap, else (c, r, s) with the offset table.
         plan->k_order = d->C % 8 == 0 ? 1 : 0;
+        // Stride 2 across a 3-wide filter: the two columns that read pixels (2 q, 2 q + 1) are paired (see the kernel's operand
+        // fetch) when both lie inside the image for every output column, 2 Q <= W.
+        {
+            static const bool pairing = [] { const char* e = std::getenv("PAELLA_CONV_PAIR_TAPS"); return !e || std::atoi(e) != 0; }();
+            plan->pair_taps = (pairing && plan->k_order && mi == 1 && ni == 1 && d->S == 3 && d->stride_w == 2 && d->dil_w == 1 && d->pad_w <= 1 && 2 * Q <= d->W)
+                                  ? 1 + d->pad_w : 0;
+        }
         // Which workgroups share an XCD.  Weights outweigh the input: those that read one slab of weights; else neighbouring pixels.
         plan->wg_order = (double)d->K * d->C * d->R * d->S > (double)d->C * d->H * d->W ? 1 : 0;
         plan->fast_div = 1;
@@ -1257,7 +1291,14 @@ extern "C" int paella_conv2d_pack(const paella_conv_plan* plan, const float* w, 
     const int RS = d.R * d.S;
     for (int m = 0; m < d.K; ++m)
         for (int k = 0; k < kdim; ++k) {  // k indexes the source in (c, r, s) order
-            const int kp = plan->k_order ? (k % RS) * d.C + k / RS : k;  // position in the kernel's reduction order
+            int kp = plan->k_order ? (k % RS) * d.C + k / RS : k;  // position in the kernel's reduction order
+            if (plan->pair_taps) {
+                // per filter row: the unpaired column's C values, then the pair's 2 C values as chunks of (column 0 | column 1) x
+                // four channels
+                const int c = k / RS, r = (k % RS) / d.S, sx = k % d.S, s0 = plan->pair_taps - 1;
+                if (sx == 2 - 2 * s0) kp = r * 3 * d.C + c;
+                else kp = r * 3 * d.C + d.C + (c / 4) * 8 + (sx - s0) * 4 + (c % 4);
+            }
             wp[((size_t)(kp / 4) * plan->m_pad + m) * 4 + (kp % 4)] = w[(size_t)m * kdim + k];
         }
     return 0;
@@ -1317,6 +1358,7 @@ int fill_args(const paella_conv_plan* plan, const float* x, const void* blob_dev
     // The reduction loop locates its chunks with the multiply-high alone (chunk by chunks per tap, tap by filter width).
     if (((uint64_t)a.nchunks + a.chunks_per_split + 64) * std::max<uint64_t>(d_cb, (uint64_t)d.S) >= ((uint64_t)1 << 32)) return PAELLA_ENOSUP;
     a.pointwise = plan->k_order && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1 && d.pad_h == 0 && d.pad_w == 0 ? 1 : 0;
+    a.pair_s0 = plan->pair_taps - 1;
     return 0;
 }
 

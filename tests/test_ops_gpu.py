@@ -48,7 +48,27 @@ CONV_SHAPES = [
     (5, 9, 11, 7, 3, 3, 1, 1, 1),           # nothing is a multiple of anything
     (16, 12, 12, 40, 3, 3, 1, 2, 2),        # dilation
     (2048, 1, 1, 1000, 1, 1, 1, 0, 1),      # a dense layer expressed as 1x1 conv
+    (288, 35, 35, 384, 3, 3, 2, 0, 1),      # Inception reduction: stride 2 without padding (filter columns 0 and 1 paired)
+    (192, 17, 17, 320, 3, 3, 2, 0, 1),
+    (256, 14, 14, 512, 3, 3, 2, 1, 1),      # residual stage entry: stride 2 with padding (columns 1 and 2 paired)
+    (16, 9, 12, 40, 3, 3, 2, 1, 1),         # even width, ragged everything else
+    (16, 9, 13, 40, 3, 3, 2, 1, 1),         # odd width with padding: the last pair would leave the image, so not paired
+    (24, 11, 10, 33, 1, 3, (1, 2), (0, 1), 1),  # one filter row, stride 2 across only
+    (8, 20, 20, 32, 3, 3, (1, 2), (1, 0), 1),   # stride 2 across, 1 down
 ]
+
+
+def test_paired_filter_columns_are_planned_where_both_columns_stay_inside(cuda):
+    """Stride 2 across a 3-wide filter with C a multiple of 8: paired when 2 Q <= W, first column = the padding."""
+    from paella_amd import ops
+    def planned(c, h, w, k, r, s, stride, pad):
+        return ops.Conv2d(rnd(k, c, r, s), None, stride=stride, pad=pad, in_hw=(h, w)).plan.pair_taps
+    assert planned(288, 35, 35, 384, 3, 3, 2, 0) == 1
+    assert planned(256, 14, 14, 512, 3, 3, 2, 1) == 2
+    assert planned(16, 9, 13, 40, 3, 3, 2, 1) == 0      # Q = 7, W = 13
+    assert planned(16, 9, 12, 40, 3, 3, 1, 1) == 0      # stride 1
+    assert planned(12, 9, 12, 40, 3, 3, 2, 1) == 0      # C no multiple of 8: the other reduction order
+    assert planned(16, 9, 12, 40, 3, 5, 2, (1, 2)) == 0  # 5-wide filter
 
 
 @pytest.mark.parametrize("shape", CONV_SHAPES)
