@@ -103,6 +103,38 @@ def test_weight_packing_layout_tap_major():
                     assert packed[kp // 4, m, kp % 4] == wt[m, cc, rr, ss]
 
 
+@pytest.mark.parametrize("pad_w,first", [(0, 0), (1, 1)])
+def test_weight_packing_layout_with_paired_filter_columns(pad_w, first):
+    """Stride 2 across a 3-wide filter: per filter row the unpaired column's C values (chunks of eight channels), then the pair's 2 C
+    values as chunks of (first column | second column) x four channels; the pair's first column is the padding."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+    c, h, w, k, r, s = 16, 9, 12, 6, 3, 3
+    rc, p = plan((c, h, w, k, r, s, 1, 2, 1, pad_w, 1, 1, 1, 0, 0, 0))
+    assert rc == 0 and p.k_order == 1 and p.pair_taps == 1 + first and p.k_pad == c * r * s
+    wt = np.random.default_rng(2).standard_normal((k, c, r, s)).astype(np.float32)
+    blob = np.zeros(p.blob_bytes, np.uint8)
+    assert lib.paella_conv2d_pack(ctypes.byref(p), wt.ctypes.data, blob.ctypes.data) == 0
+    packed = blob.view(np.float32).reshape(p.k_pad // 4, p.m_pad, 4)
+    unpaired = 2 - 2 * first
+    seen = set()
+    for m in range(k):
+        for cc in range(c):
+            for rr in range(r):
+                for ss in range(s):
+                    if ss == unpaired:
+                        kp = rr * 3 * c + cc
+                    else:
+                        kp = rr * 3 * c + c + (cc // 4) * 8 + (ss - first) * 4 + cc % 4
+                    seen.add(kp)
+                    assert packed[kp // 4, m, kp % 4] == wt[m, cc, rr, ss]
+    assert seen == set(range(c * r * s))   # a permutation of the reduction
+    # not paired: odd width with padding (the last pair would leave the image), stride 1, a 5-wide filter
+    assert plan((c, h, 13, k, r, s, 1, 2, 1, 1, 1, 1, 1, 0, 0, 0))[1].pair_taps == 0
+    assert plan((c, h, w, k, r, s, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0))[1].pair_taps == 0
+    assert plan((c, h, w, k, r, 5, 1, 2, 1, 2, 1, 1, 1, 0, 0, 0))[1].pair_taps == 0
+
+
 def test_pool_out_matches_oracle():
     from oracle import ops as orc
     from paella_amd import _abi
