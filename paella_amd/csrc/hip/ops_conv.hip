@@ -1221,6 +1221,9 @@ extern "C" int paella_conv2d_plan(const paella_conv_desc* d, int has_residual, i
             // the other requests, and the same measurement (one box, packing on) moved the larger layers to 9 chunks per wave:
             // 6 / 8 / 9 / 10 / 12 chunks: Inception-v3 5036 / 5238 / 5286 / 5306 / 5323, ResNet-50 6381 / 6325 / 6438 / 6447 / 6430,
             // DenseNet-121 5173 / 5159 / 5139 / 5043 / 5013 requests/s, the 9 : 1 mix 43.9 / 44.9 / 44.6 / 44.8 / 44.9 thousand.
+            // Once more with the split path cheapened (uniform bookkeeping, exact batches): 4 / 6 / 9 / 12 chunks: Inception-v3 served
+            // with 32 requests outstanding 5.58 / 6.18 / 6.58 / 6.73 thousand, with 16: 5.39 / 5.79 / 6.00 / 6.02, ResNet-50 7.21 / 7.43 /
+            // 7.45 / 7.38, the 9 : 1 mix 49.5 / 51.6 / 53.5 / 53.4 thousand, one launch at a time 7.9 / 7.9 / 7.91 / 8.05 us: 9 stays.
             const int min_chunks = plan->flops < 16e6 ? 2 : 9;
             while (splits < 16 && n_tiles * splits * 2 <= cap && nchunks / (splits * 2 * kw) >= min_chunks) splits *= 2;
         }
