@@ -122,12 +122,14 @@ def conv_roofline(models, hip, model, reps, back_to_back=200):
             "by_op": by_op, "direct_rps": direct_rps, "forward_us": sum(per_stage)}
 
 
-def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None, depth=0, only=None):
+def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None, depth=0, only=None, burst=8):
     """The conv kernel with the device full: every distinct conv layer of the model (groups == 1) over `images` inputs stacked
     along the height, i.e. with `images` times the pixel tiles -- what the compute units see on the serving path, where packed
     launches on four queues keep 16 to 24 problems in flight -- on the 32 x 32 tile with the layer's own waves per workgroup and
     no split of the reduction over workgroups, one launch at a time on a HIP stream.  timed: durations from the kernel's own
-    begin and end stamps; otherwise one launch per layer with a synchronize after each (for counter collection)."""
+    begin and end stamps, of the last of `burst` launches enqueued back to back (stream order: they do not overlap; the ones in
+    front keep the device's clocks from dropping in the idle gap that a synchronize per launch leaves); otherwise one launch per
+    layer with a synchronize after each (for counter collection)."""
     import numpy as np
     import torch
     from paella_amd import ops
@@ -171,7 +173,8 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None
             lib.paella_ops_time_launches(ev[0], ev[1])
             total = 0.0
             for _ in range(reps):
-                conv(xin, out=y, stream=stream.value)
+                for _ in range(max(1, burst)):
+                    conv(xin, out=y, stream=stream.value)
                 hip.llis_hip_stream_synchronize(stream)
                 ms = ctypes.c_float()
                 hip.llis_hip_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms))
@@ -190,8 +193,8 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None
         flops = sum(r["flops"] * r["count"] for r in rows)
         us = sum(r["us"] * r["count"] for r in rows)
         out.update({"achieved": flops / us / 1e6, "frac": flops / us / 1e6 / FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "how": "every conv layer of %s over %d inputs stacked along the height (%d times the pixel tiles), 32 x 32 tile, one launch at a time; "
-                           "layers weighted by their count in a forward pass" % (model, images, images)})
+                    "how": "every conv layer of %s over %d inputs stacked along the height (%d times the pixel tiles), 32 x 32 tile, one launch at a time "
+                           "(the last of %d enqueued back to back); layers weighted by their count in a forward pass" % (model, images, images, max(1, burst))})
     return out
 
 
@@ -458,6 +461,7 @@ def main():
     ap.add_argument("--fd-depth", type=int, default=0, help="with --full-device: chunks of operands in flight per wave (3, 4, 6, 8, 12; default 2)")
     ap.add_argument("--fd-only", default=None, help="with --full-device: comma-separated substrings of the layers to run, e.g. '17x17 768->192'")
     ap.add_argument("--fd-images", type=int, default=16)
+    ap.add_argument("--fd-burst", type=int, default=8, help="with --full-device: launches enqueued back to back per sample; the last one is timed")
     ap.add_argument("--counter-pass", default=None, metavar="MODEL",
                     help="only this: three forward passes of MODEL, one launch at a time with a synchronize after each (the leg to run "
                          "under `rocprofv3 --pmc`: nothing else is in flight and at most one dispatch is ever queued)")
@@ -482,7 +486,7 @@ def main():
         return
     if args.full_device:
         fd = full_device_pass(models, hip, args.full_device, images=args.fd_images, timed=not under_counter_collection(), kw=args.fd_kw, depth=args.fd_depth,
-                              only=args.fd_only.split(",") if args.fd_only else None)
+                              only=args.fd_only.split(",") if args.fd_only else None, burst=args.fd_burst)
         for r in fd["layers"]:
             log("[bench] %-26s x%d  %5d workgroups x %d waves  %8.1f MFLOP  %s" % (r["layer"], r["count"], r["workgroups"], r["waves_per_workgroup"], r["flops"] / 1e6,
                 "%7.2f us  %6.1f TFLOP/s" % (r["us"], r["flops"] / r["us"] / 1e6) if r["us"] else ""))
