@@ -416,3 +416,80 @@ def test_conv_linearity_at_full_size(cuda):
     ya = ops.Conv2d(w1 + w2, None, pad=1, in_hw=(112, 112))(x)
     yb = ops.Conv2d(w1, None, pad=1, in_hw=(112, 112))(x) + ops.Conv2d(w2, None, pad=1, in_hw=(112, 112))(x)
     close(ya, yb.cpu().numpy())
+
+
+def test_random_conv_shapes_match_the_oracle(cuda):
+    """200 seeded shapes over channel counts on both reduction orders, strides, paddings past the filter's reach, dilations,
+    bias / residual / activation present or not: whatever plan they get (split reductions, paired filter columns)."""
+    from paella_amd import ops
+    rng = np.random.default_rng(7)
+    paired = split = done = 0
+    while done < 200:
+        c = int(rng.choice([3, 5, 8, 16, 24, 40, 64, 96, 128, 256]))
+        k = int(rng.integers(1, 130))
+        r, s = int(rng.choice([1, 3, 5])), int(rng.choice([1, 3, 3, 3, 5, 7]))
+        sh, sw = int(rng.choice([1, 2])), int(rng.choice([1, 2, 2]))
+        ph, pw = int(rng.integers(0, r // 2 + 2)), int(rng.integers(0, s // 2 + 2))
+        dh, dw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 1, 2]))
+        h, w = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        if h + 2 * ph - (r - 1) * dh - 1 < 0 or w + 2 * pw - (s - 1) * dw - 1 < 0:
+            continue
+        done += 1
+        act = int(rng.choice([orc.ACT_NONE, orc.ACT_RELU, orc.ACT_RELU6]))
+        x = rng.standard_normal((1, c, h, w)).astype(np.float32)
+        wt = (rng.standard_normal((k, c, r, s)) * (2.0 / (c * r * s)) ** 0.5).astype(np.float32)
+        b = None if rng.random() < 0.3 else (rng.standard_normal(k) * 0.1).astype(np.float32)
+        ref = orc.conv2d(x, wt, b, stride=(sh, sw), pad=(ph, pw), dil=(dh, dw))
+        res = rng.standard_normal(ref.shape).astype(np.float32) if rng.random() < 0.3 else None
+        if res is not None:
+            ref = ref + res
+        ref = np.maximum(ref, 0) if act != orc.ACT_NONE else ref
+        ref = np.minimum(ref, 6) if act == orc.ACT_RELU6 else ref
+        conv = ops.Conv2d(wt, b, stride=(sh, sw), pad=(ph, pw), dil=(dh, dw), act=act, in_hw=(h, w), has_residual=res is not None)
+        paired += conv.plan.pair_taps != 0
+        split += conv.plan.splits > 1
+        got = conv(torch.tensor(x, device=cuda), residual=None if res is None else torch.tensor(res, device=cuda))
+        torch.cuda.synchronize()
+        close(got, ref.astype(np.float32))
+    assert paired >= 10 and split >= 50   # the sweep reaches both
+
+
+def test_random_depthwise_and_pooling_shapes_match_the_oracle(cuda):
+    """150 seeded shapes each; maximum pooling bit for bit."""
+    from paella_amd import ops
+    rng = np.random.default_rng(5)
+    done = 0
+    while done < 150:
+        c, h, w = int(rng.integers(1, 200)), int(rng.integers(3, 60)), int(rng.integers(3, 60))
+        r, st, pad, dil = int(rng.choice([3, 3, 3, 5])), int(rng.choice([1, 2])), int(rng.integers(0, 3)), int(rng.choice([1, 1, 2]))
+        if h + 2 * pad - (r - 1) * dil - 1 < 0 or w + 2 * pad - (r - 1) * dil - 1 < 0:
+            continue
+        done += 1
+        x = rng.standard_normal((1, c, h, w)).astype(np.float32)
+        wt = (rng.standard_normal((c, 1, r, r)) * 0.3).astype(np.float32)
+        b = None if rng.random() < 0.3 else (rng.standard_normal(c) * 0.1).astype(np.float32)
+        act = int(rng.choice([orc.ACT_NONE, orc.ACT_RELU, orc.ACT_RELU6]))
+        ref = orc.conv2d(x, wt, b, stride=st, pad=pad, dil=dil, groups=c, act=act)
+        got = ops.Conv2d(wt, b, stride=st, pad=pad, dil=dil, groups=c, act=act, in_hw=(h, w))(torch.tensor(x, device=cuda))
+        torch.cuda.synchronize()
+        close(got, ref)
+    done = 0
+    while done < 150:
+        c, h, w = int(rng.integers(1, 300)), int(rng.integers(2, 50)), int(rng.integers(2, 50))
+        k, st = int(rng.choice([2, 3, 3])), int(rng.choice([1, 2, 2]))
+        pad, ceil = int(rng.integers(0, k // 2 + 1)), bool(rng.random() < 0.4)
+        is_avg, cip = bool(rng.random() < 0.5), bool(rng.random() < 0.5)
+        if h + 2 * pad < k or w + 2 * pad < k:
+            continue
+        done += 1
+        x = rng.standard_normal((1, c, h, w)).astype(np.float32)
+        ref = orc.avgpool2d(x, k, st, pad=pad, ceil_mode=ceil, count_include_pad=cip) if is_avg else orc.maxpool2d(x, k, st, pad=pad, ceil_mode=ceil)
+        got = ops.pool2d(torch.tensor(x, device=cuda), k, st, pad=pad, ceil_mode=ceil, is_avg=is_avg, count_include_pad=cip)
+        torch.cuda.synchronize()
+        got = got.cpu().numpy()
+        assert got.shape == ref.shape
+        if is_avg:
+            assert np.all(np.abs(got - ref) <= 1e-5 + 1e-5 * np.abs(ref))
+        else:
+            assert np.array_equal(got, ref)
+
