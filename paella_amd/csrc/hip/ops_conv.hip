@@ -135,7 +135,10 @@ struct PreOp {
 // One workgroup's share of a conv: output tile and reduction split number `bid` of the problem `p`.
 // PW ("pointwise"): a 1x1 filter with stride 1 and no padding in tap-major order -- an input pixel is its output pixel, there
 // are no taps to step through and nothing to test per tap.
-template <int MI, int NI, int KW, bool TAP_MAJOR, bool PRE = false, int DEPTH = 0, bool PW = false>
+// PRE: kPreBounded with a lower bound (ReLU), kPreUnbounded without (a batch-norm alone: the four maxima per chunk are not
+// computed at all -- a vector instruction costs a sixteenth of a matrix instruction of pipe time).
+constexpr int kPreNone = 0, kPreBounded = 1, kPreUnbounded = 2;
+template <int MI, int NI, int KW, bool TAP_MAJOR, int PRE = kPreNone, int DEPTH = 0, bool PW = false>
 __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid, const PreOp pre = PreOp{nullptr, nullptr, 0.f}) {
     static_assert(!PRE || (TAP_MAJOR && MI * NI == 1), "the input transform is built for the smallest tile in tap-major order");
     static_assert(!PW || TAP_MAJOR, "the pointwise shortcut belongs to the tap-major order");
@@ -176,6 +179,9 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     extern __shared__ __align__(16) char smem[];
     int2* ltab = reinterpret_cast<int2*>(smem);
     float* red = reinterpret_cast<float*>(smem);
+    // With a fused input transform, behind the partial tiles' region (waves leave the loop at different times): 64 bytes of zeros,
+    // then per four input channels their four scales and their four shifts, 32 bytes.
+    char* const ptab = smem + (KW > 1 ? KW * MI * NI * 16 * 64 * 4 : 0);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and the compiler may know it
@@ -272,11 +278,6 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // Chunks outside [c_begin, c_end) are requested at an out-of-range offset: the loads keep their place in
     // the (static) issue order, return zeros and touch no memory.
     __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.wpk, 0, p.w_bytes, 0x00027000);
-    __amdgpu_buffer_rsrc_t sres, hres;
-    if (PRE) {
-        sres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, (unsigned)(p.CB * 32), 0x00027000);
-        hres = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, (unsigned)(p.CB * 32), 0x00027000);
-    }
     // Vector instructions take their four cycles out of the matrix pipe's time on this part (a matrix instruction and a vector
     // instruction of any wave of the SIMD do not overlap), so the per-chunk address arithmetic is kept on the scalar unit:
     // a lane's part of an offset sits in a register that changes only when the filter tap does, the chunk's part rides in the
@@ -289,6 +290,10 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     const int wstep = p.m_pad * 32;  // bytes of weights per chunk and row block: two reduction steps of m_pad rows of 16 bytes
     int tap_voff[NI];
     bool tap_ok[NI];
+    // With a fused input transform: what a lane keeps of a chunk's table address -- everything in the second half of the wave,
+    // all but the bit that selects the second reduction step's four channels in the first, nothing (the zeros in front of the
+    // table) where the lane's pixel or tap is padding.  It changes only when the tap does.
+    int pre_sel = (PRE && PW) ? (base[0] >= 0 ? (negkk | ~32) : 0) : 0;
     bool tap_stale = true;
     int tap_off = 0;  // byte offset of the current filter tap, wave-uniform
     // Paired filter columns (stride 2 across a 3-wide filter, pair_s0 >= 0).  With stride 2 a lane's pixels are every other
@@ -339,6 +344,7 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
 #pragma unroll
                         for (int ni = 0; ni < NI; ++ni) tap_voff[ni] = tap_ok[ni] ? base[ni] + pair_delta : -1;
                     }
+                    if (PRE) pre_sel = tap_ok[0] ? (seg_pair ? -1 : (negkk | ~32)) : 0;  // a pair's chunk: the same four channels in both halves
                     tap_stale = false;
                 }
                 tap_soff = tap_off;
@@ -351,11 +357,16 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                 const int voff = PW ? base[ni] : tap_voff[ni];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) f.b[ni][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, voff, chunk_off + t * HW4, 0));
-                if (PRE) {  // a tap outside the image gets scale = shift = 0, so it stays the zero the padding asks for
-                    const bool inside = PW ? base[ni] >= 0 : tap_ok[ni];
-                    const int soff = (valid & inside) ? (chan0 + ((!PW && seg_pair) ? 0 : kk * 4)) * 4 : -1;
-                    f.sc = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(sres, soff, 0, 0));
-                    f.sh = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(hres, soff, 0, 0));
+                if (PRE) {
+                    // Scale and shift of the lane's four channels, from the table in LDS: requested through the vector cache like
+                    // the operands, their 2 KB per wave and chunk doubled what the cache has to deliver and cost a fifth of the
+                    // kernel's rate with the device full.  Where the lane's pixel or tap is padding, and for a chunk past the
+                    // wave's range, the address is that of the zeros, and the zero that the operand load returned stays the
+                    // zero the padding asks for.  One vector instruction: the chunk's part of the address is wave-uniform.
+                    const int chunk_addr = valid ? ((64 + chan0 * 8) | ((!PW && seg_pair) ? 0 : 32)) : 0;
+                    const char* const e = ptab + (pre_sel & chunk_addr);
+                    f.sc = *reinterpret_cast<const float4*>(e);
+                    f.sh = *reinterpret_cast<const float4*>(e + 16);
                 }
             }
             return;
@@ -397,6 +408,19 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
             e.y = ((r * p.dh) << 16) | (sx * p.dw);
             if (k >= p.kdim) e = make_int2(0, 0x7FFF0000);  // row far outside the image: the tap reads as zero
             ltab[i] = e;
+        }
+        __syncthreads();
+    }
+    // The table of scales and shifts of a fused input transform: every input channel's, a few entries per thread.
+    if (PRE) {
+        const int n_chan = p.CB * 8;
+        const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, (unsigned)n_chan * 4u, 0x00027000);
+        const __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, (unsigned)n_chan * 4u, 0x00027000);
+        if (threadIdx.x < 16) reinterpret_cast<float*>(ptab)[threadIdx.x] = 0.f;
+        for (int i = threadIdx.x; i < n_chan; i += 64 * KW) {
+            float* const e = reinterpret_cast<float*>(ptab + 64 + (i >> 2) * 32 + (i & 3) * 4);
+            e[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sr, i * 4, 0, 0));
+            e[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(hr, i * 4, 0, 0));
         }
         __syncthreads();
     }
@@ -498,7 +522,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
                     if (PRE) {
                         const float sc = t == 0 ? f.sc.x : t == 1 ? f.sc.y : t == 2 ? f.sc.z : f.sc.w;
                         const float sh = t == 0 ? f.sh.x : t == 1 ? f.sh.y : t == 2 ? f.sh.z : f.sh.w;
-                        bv = fmaxf(bv * sc + sh, pre.lo);  // lo is 0 or -inf: the padding's 0 * 0 + 0 stays 0
+                        bv = bv * sc + sh;  // the padding's 0 * 0 + 0 stays 0, also under a bound of 0
+                        if (PRE == kPreBounded) bv = fmaxf(bv, pre.lo);
                     }
                     if (decltype(first)::value && t == 0) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zero, 0, 0, 0);
                     else acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
@@ -755,8 +780,8 @@ __global__ __launch_bounds__(64 * KW, (MI * NI == 1 && KW == 8 && DEPTH == 0) ? 
     int idx = 0;
     asm volatile("" : "+s"(idx));
     const ConvArgs& p = (&args)[idx];
-    if (TAP_MAJOR && p.pointwise) conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH, TAP_MAJOR>(p, blockIdx.x);
-    else conv_tile<MI, NI, KW, TAP_MAJOR, false, DEPTH>(p, blockIdx.x);
+    if (TAP_MAJOR && p.pointwise) conv_tile<MI, NI, KW, TAP_MAJOR, kPreNone, DEPTH, TAP_MAJOR>(p, blockIdx.x);
+    else conv_tile<MI, NI, KW, TAP_MAJOR, kPreNone, DEPTH>(p, blockIdx.x);
 }
 
 // A conv that applies a per-channel transform to its input on the way (smallest tile, tap-major order).
@@ -766,12 +791,23 @@ struct ConvPreArgs {
 };
 
 template <int KW>
+__device__ __forceinline__ void conv_pre_tile(const ConvPreArgs& a, unsigned bid) {
+    const bool bounded = a.pre.lo > -__builtin_inff();
+    if (a.conv.pointwise) {
+        if (bounded) conv_tile<1, 1, KW, true, kPreBounded, 0, true>(a.conv, bid, a.pre);
+        else conv_tile<1, 1, KW, true, kPreUnbounded, 0, true>(a.conv, bid, a.pre);
+    } else {
+        if (bounded) conv_tile<1, 1, KW, true, kPreBounded>(a.conv, bid, a.pre);
+        else conv_tile<1, 1, KW, true, kPreUnbounded>(a.conv, bid, a.pre);
+    }
+}
+
+template <int KW>
 __global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_pre_kernel(ConvPreArgs args) {
     int idx = 0;  // see conv_mfma_kernel
     asm volatile("" : "+s"(idx));
     const ConvPreArgs& a = (&args)[idx];
-    if (a.conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(a.conv, blockIdx.x, a.pre);
-    else conv_tile<1, 1, KW, true, true>(a.conv, blockIdx.x, a.pre);
+    conv_pre_tile<KW>(a, blockIdx.x);
 }
 
 // The same for up to kPackMax such convs of different requests in one launch (launch packing).
@@ -792,8 +828,7 @@ __global__ __launch_bounds__(64 * KW, KW == 8 ? 8 : 1) void conv_mfma_pre_group_
             idx = i;
             first = g.start[i];
         }
-    if (g.m[idx].conv.pointwise) conv_tile<1, 1, KW, true, true, 0, true>(g.m[idx].conv, blockIdx.x - first, g.m[idx].pre);
-    else conv_tile<1, 1, KW, true, true>(g.m[idx].conv, blockIdx.x - first, g.m[idx].pre);
+    conv_pre_tile<KW>(g.m[idx], blockIdx.x - first);
 }
 
 // Up to four independent convs in one launch: layers whose own grids would leave most of the 256 CUs idle (the 1x1
@@ -2149,6 +2184,10 @@ ConvPreGroupKernel pick_pre_group_kernel(int kw) {
     }
 }
 
+// Dynamic LDS of a launch with a fused input transform: the plan's (the partial tiles of the cross-wave sum) and behind it the
+// table of scales and shifts -- 64 bytes of zeros and 8 bytes per input channel.
+unsigned pre_lds_bytes(const paella_conv_plan* plan) { return plan->dims.lds_bytes + 64u + 8u * (unsigned)((plan->d.C + 7) / 8 * 8); }
+
 // Launch packing of convs with a fused input transform: held like the plain ones (pack_hold), in lists of their own
 // because they run in a kernel of their own.
 bool pack_hold_pre(const paella_conv_plan* plan, const ConvPreArgs& a, void* stream) {
@@ -2158,7 +2197,7 @@ bool pack_hold_pre(const paella_conv_plan* plan, const ConvPreArgs& a, void* str
     PackState::PreItem it;
     it.a = a;
     it.grid = plan->dims.grid;
-    it.dyn_lds = plan->dims.lds_bytes;
+    it.dyn_lds = pre_lds_bytes(plan);
     it.a.conv.hook_blocks = it.grid;
     g_pack.pre_lists[kw_index(plan->kw)].push_back(it);
     if (g_pack.held++ == 0) g_pack.first_held_ns = now_ns();
@@ -2231,6 +2270,7 @@ extern "C" int paella_conv2d_transformed_dims(const paella_conv_plan* plan, pael
     if (!plan || !dims) return PAELLA_EINVAL;
     if (!paella_conv2d_plan_takes_input_transform(plan)) return PAELLA_ENOSUP;
     *dims = plan->dims;
+    dims->lds_bytes = pre_lds_bytes(plan);
     add_kernel_resources(reinterpret_cast<const void*>(pick_pre_kernel(plan->kw)), dims);
     return 0;
 }
@@ -2260,8 +2300,8 @@ extern "C" int paella_conv2d_launch_transformed(const paella_conv_plan* plan, co
     a.pre.shift = in_shift;
     a.pre.lo = in_act == PAELLA_ACT_RELU ? 0.f : -__builtin_inff();
     if (pack_hold_pre(plan, a, stream)) return 0;
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), plan->dims.lds_bytes)) return rc;
-    paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), plan->dims.lds_bytes, reinterpret_cast<hipStream_t>(stream), a);
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), pre_lds_bytes(plan))) return rc;
+    paella::launch(kern, dim3(plan->dims.grid), dim3(plan->dims.block), pre_lds_bytes(plan), reinterpret_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();
 }
 

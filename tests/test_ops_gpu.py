@@ -113,6 +113,10 @@ TRANSFORMED = [
     (40, 19, 23, 72, 3, 3, 1, 2, orc.ACT_RELU, 1, True),
     (40, 19, 23, 72, 3, 3, 1, 2, orc.ACT_NONE, 2, False),
     (40, 19, 23, 72, 5, 3, 2, (2, 1), orc.ACT_RELU, 3, True),
+    (1024, 7, 7, 128, 1, 1, 1, 0, orc.ACT_RELU, -1, False),    # the widest table of scales and shifts in the zoo
+    (8, 9, 11, 40, 3, 3, 1, 1, orc.ACT_NONE, 3, False),        # one chunk per tap: the tap changes with every chunk
+    (64, 16, 16, 96, 3, 3, 2, 1, orc.ACT_RELU, -1, True),      # paired filter columns under the transform, with a bound
+    (24, 12, 20, 48, 3, 3, 2, 0, orc.ACT_NONE, 1, False),      # paired, no padding, two waves
 ]
 
 
