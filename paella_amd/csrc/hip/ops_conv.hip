@@ -182,6 +182,22 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
     // With a fused input transform, behind the partial tiles' region (waves leave the loop at different times): 64 bytes of zeros,
     // then per four input channels their four scales and their four shifts, 32 bytes.
     char* const ptab = smem + (KW > 1 ? KW * MI * NI * 16 * 64 * 4 : 0);
+    // A thread's first two entries of that table are requested here, so that they travel while the tile is decoded (entries
+    // past the last channel read as zero and are not written).
+    constexpr int kPreEarly = 2;
+    float pre_early_s[kPreEarly], pre_early_h[kPreEarly];
+    if (PRE) {
+        const unsigned len = (unsigned)p.CB * 32u;
+        const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, len, 0x00027000);
+        const __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, len, 0x00027000);
+#pragma unroll
+        for (int e = 0; e < kPreEarly; ++e) {
+            const int off = ((int)threadIdx.x + e * 64 * KW) * 4;
+            pre_early_s[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sr, off, 0, 0));
+            pre_early_h[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(hr, off, 0, 0));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and the compiler may know it
@@ -417,10 +433,18 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, const unsigned bid,
         const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.scale, 0, (unsigned)n_chan * 4u, 0x00027000);
         const __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)pre.shift, 0, (unsigned)n_chan * 4u, 0x00027000);
         if (threadIdx.x < 16) reinterpret_cast<float*>(ptab)[threadIdx.x] = 0.f;
-        for (int i = threadIdx.x; i < n_chan; i += 64 * KW) {
-            float* const e = reinterpret_cast<float*>(ptab + 64 + (i >> 2) * 32 + (i & 3) * 4);
-            e[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sr, i * 4, 0, 0));
-            e[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(hr, i * 4, 0, 0));
+        auto entry = [&](int i) { return reinterpret_cast<float*>(ptab + 64 + (i >> 2) * 32 + (i & 3) * 4); };
+#pragma unroll
+        for (int e = 0; e < kPreEarly; ++e) {
+            const int i = (int)threadIdx.x + e * 64 * KW;
+            if (i < n_chan) {
+                entry(i)[0] = pre_early_s[e];
+                entry(i)[4] = pre_early_h[e];
+            }
+        }
+        for (int i = (int)threadIdx.x + kPreEarly * 64 * KW; i < n_chan; i += 64 * KW) {
+            entry(i)[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sr, i * 4, 0, 0));
+            entry(i)[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(hr, i * 4, 0, 0));
         }
         __syncthreads();
     }
