@@ -437,7 +437,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2, help="untimed steps served first at the same offered rate")
     ap.add_argument("--num-streams", type=int, default=128)
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
-    ap.add_argument("--extra-kernels", type=int, default=32, help="full3: kernels admitted beyond the occupancy budget")
+    ap.add_argument("--extra-kernels", type=int, default=48, help="full3: kernels admitted beyond the occupancy budget")
     ap.add_argument("--unfair", type=float, default=1e6, help="full3: deficit threshold of the headline arm (1e6 = shortest remaining work first only)")
     ap.add_argument("--no-arms", action="store_true", help="only the headline search and timed run (plus roofline and CPU baseline)")
     ap.add_argument("--no-cpu", action="store_true")
