@@ -458,6 +458,43 @@ def test_random_conv_shapes_match_the_oracle(cuda):
     assert paired >= 10 and split >= 50   # the sweep reaches both
 
 
+def test_random_transformed_input_conv_shapes_match_the_oracle(cuda):
+    """120 seeded shapes of conv(act(x * scale + shift)) in one launch: channel counts from one chunk per tap to a table of 512
+    entries, every wave count, strides with and without paired filter columns, paddings past the filter's reach, shifts of both
+    signs (a padding tap that carried act(shift) instead of 0 would show at every border)."""
+    from paella_amd import ops
+    rng = np.random.default_rng(11)
+    paired = bounded = done = 0
+    while done < 120:
+        c = int(rng.choice([8, 16, 24, 40, 64, 128, 256, 512]))
+        k = int(rng.integers(1, 130))
+        r, s = int(rng.choice([1, 3, 3])), int(rng.choice([1, 3, 3, 5]))
+        sh, sw = int(rng.choice([1, 2])), int(rng.choice([1, 2, 2]))
+        ph, pw = int(rng.integers(0, r // 2 + 2)), int(rng.integers(0, s // 2 + 2))
+        h, w = int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        if h + 2 * ph - r < 0 or w + 2 * pw - s < 0:
+            continue
+        kwlog = int(rng.integers(-1, 4))
+        in_act = int(rng.choice([orc.ACT_NONE, orc.ACT_RELU]))
+        x = rng.standard_normal((1, c, h, w)).astype(np.float32)
+        wt = (rng.standard_normal((k, c, r, s)) * (2.0 / (c * r * s)) ** 0.5).astype(np.float32)
+        b = (rng.standard_normal(k) * 0.1).astype(np.float32)
+        scale, shift = (rng.standard_normal(c) + 1.5).astype(np.float32), (rng.standard_normal(c) * 2.0).astype(np.float32)
+        conv = ops.Conv2d(wt, b, stride=(sh, sw), pad=(ph, pw), act=ops.ACT_RELU, in_hw=(h, w),
+                          tile_hint=0 if kwlog < 0 else (1 << 8) | (1 << 4) | kwlog)
+        if not conv.takes_input_transform():
+            continue
+        done += 1
+        paired += conv.plan.pair_taps != 0
+        bounded += in_act == orc.ACT_RELU
+        ref = orc.conv2d(orc.scale_shift(x, scale, shift, act=in_act), wt, b, stride=(sh, sw), pad=(ph, pw), act=orc.ACT_RELU)
+        dev = lambda a: torch.tensor(a, device=cuda)
+        got = conv(dev(x), in_scale=dev(scale), in_shift=dev(shift), in_act=in_act)
+        torch.cuda.synchronize()
+        close(got, ref)
+    assert paired >= 5 and 30 <= bounded <= 90   # the sweep reaches paired columns and both copies of the loop
+
+
 def test_random_depthwise_and_pooling_shapes_match_the_oracle(cuda):
     """150 seeded shapes each; maximum pooling bit for bit."""
     from paella_amd import ops
