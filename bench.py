@@ -122,7 +122,7 @@ def conv_roofline(models, hip, model, reps, back_to_back=200):
             "by_op": by_op, "direct_rps": direct_rps, "forward_us": sum(per_stage)}
 
 
-def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None, depth=0, only=None, burst=8):
+def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None, depth=0, only=None, burst=8, transform=False):
     """The conv kernel with the device full: every distinct conv layer of the model (groups == 1) over `images` inputs stacked
     along the height, i.e. with `images` times the pixel tiles -- what the compute units see on the serving path, where packed
     launches on four queues keep 16 to 24 problems in flight -- on the 32 x 32 tile with the layer's own waves per workgroup and
@@ -165,8 +165,12 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None
                           in_hw=(h * images, w), tile_hint=hint)
         xin = torch.randn((1, c, h * images, w), device="cuda:0")
         y = torch.empty((1, k, conv.plan.P, conv.plan.Q), device="cuda:0")
+        # transform: every layer that can apply a per-channel scale-shift to its input on the way does (batch-norm in front of a conv)
+        extra = {}
+        if transform and conv.takes_input_transform():
+            extra = {"in_scale": torch.rand(c, device="cuda:0") + 0.5, "in_shift": torch.randn(c, device="cuda:0")}
         torch.cuda.synchronize()  # the operands are written on torch's stream, the launches go to another
-        conv(xin, out=y, stream=stream.value)
+        conv(xin, out=y, stream=stream.value, **extra)
         hip.llis_hip_stream_synchronize(stream)
         us = None
         if timed:
@@ -174,7 +178,7 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None
             total = 0.0
             for _ in range(reps):
                 for _ in range(max(1, burst)):
-                    conv(xin, out=y, stream=stream.value)
+                    conv(xin, out=y, stream=stream.value, **extra)
                 hip.llis_hip_stream_synchronize(stream)
                 ms = ctypes.c_float()
                 hip.llis_hip_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms))
@@ -183,7 +187,8 @@ def full_device_pass(models, hip, model, images=16, reps=10, timed=True, kw=None
             us = total / reps * 1e3
         seen[key] = len(rows)
         rows.append({"layer": "%dx%d %d->%d %dx%d s%d" % (h, w, c, k, r, q, node["stride"][0]), "count": 1, "workgroups": conv.plan.dims.grid,
-                     "waves_per_workgroup": conv.plan.kw, "k_order": conv.plan.k_order, "flops": conv.plan.flops, "us": us})
+                     "waves_per_workgroup": conv.plan.kw, "k_order": conv.plan.k_order, "flops": conv.plan.flops, "us": us,
+                     "input_transformed": bool(extra)})
     for e in ev:
         hip.llis_hip_event_destroy(e)
     hip.llis_hip_stream_destroy(stream)
@@ -461,6 +466,8 @@ def main():
     ap.add_argument("--fd-depth", type=int, default=0, help="with --full-device: chunks of operands in flight per wave (3, 4, 6, 8, 12; default 2)")
     ap.add_argument("--fd-only", default=None, help="with --full-device: comma-separated substrings of the layers to run, e.g. '17x17 768->192'")
     ap.add_argument("--fd-images", type=int, default=16)
+    ap.add_argument("--fd-transform", action="store_true",
+                    help="with --full-device: a per-channel scale-shift applied to the input of every layer that can take one (conv_mfma_pre_kernel)")
     ap.add_argument("--fd-burst", type=int, default=8, help="with --full-device: launches enqueued back to back per sample; the last one is timed")
     ap.add_argument("--counter-pass", default=None, metavar="MODEL",
                     help="only this: three forward passes of MODEL, one launch at a time with a synchronize after each (the leg to run "
@@ -486,10 +493,13 @@ def main():
         return
     if args.full_device:
         fd = full_device_pass(models, hip, args.full_device, images=args.fd_images, timed=not under_counter_collection(), kw=args.fd_kw, depth=args.fd_depth,
-                              only=args.fd_only.split(",") if args.fd_only else None, burst=args.fd_burst)
+                              only=args.fd_only.split(",") if args.fd_only else None, burst=args.fd_burst, transform=args.fd_transform)
         for r in fd["layers"]:
-            log("[bench] %-26s x%d  %5d workgroups x %d waves  %8.1f MFLOP  %s" % (r["layer"], r["count"], r["workgroups"], r["waves_per_workgroup"], r["flops"] / 1e6,
-                "%7.2f us  %6.1f TFLOP/s" % (r["us"], r["flops"] / r["us"] / 1e6) if r["us"] else ""))
+            log("[bench] %-26s x%d  %5d workgroups x %d waves  %8.1f MFLOP  %s%s" % (r["layer"], r["count"], r["workgroups"], r["waves_per_workgroup"], r["flops"] / 1e6,
+                "%7.2f us  %6.1f TFLOP/s" % (r["us"], r["flops"] / r["us"] / 1e6) if r["us"] else "", "  (input transformed)" if r["input_transformed"] else ""))
+        if fd.get("achieved"):
+            log("[bench] %s, layers weighted by count%s: %.1f TFLOP/s = %.1f %% of the fp32 MFMA peak" %
+                (args.full_device, ", input transformed where the layer can" if args.fd_transform else "", fd["achieved"], 100 * fd["frac"]))
         print(json.dumps({"full_device": fd}), flush=True)
         return
     if args.counter_pass:
