@@ -132,7 +132,8 @@ int paella_conv2d_launch_static(const paella_conv_plan* plan, const float* x, co
  * jobs/tvm_densenet121/tvm_densenet121.cpp:41).  Only plans for which paella_conv2d_plan_takes_input_transform() returns 1
  * (MFMA plan, mi == ni == 1, C a multiple of 8); PAELLA_ENOSUP otherwise. */
 int paella_conv2d_plan_takes_input_transform(const paella_conv_plan* plan);
-/* Launch shape of that form: the plan's, with the register count of the kernel that is actually launched. */
+/* Launch shape of that form: the plan's, with the register count of the kernel that is actually launched and the LDS of its
+ * table of scales and shifts (64 bytes + 8 per input channel, on top of the plan's). */
 int paella_conv2d_transformed_dims(const paella_conv_plan* plan, paella_launch_dims* dims);
 int paella_conv2d_launch_transformed(const paella_conv_plan* plan, const float* x, const float* in_scale, const float* in_shift,
                                      int in_act, const void* blob_dev, const float* bias, const float* residual,
