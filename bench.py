@@ -615,7 +615,7 @@ def main():
             rate = 0.05 * sat
         n_timed, n_warm = args.steps * STEP_REQUESTS, args.warmup * STEP_REQUESTS
         final, attempts = None, []
-        for attempt in range(8):
+        for attempt in range(10):
             r = arm.run(1e6 / rate, n_timed, n_warm)
             p = point_of(r, tenants, rate)
             p["meets_slo"] = meets(p, tenants, slo_us)
@@ -626,7 +626,7 @@ def main():
                  "SLO met" if p["meets_slo"] else "SLO missed"))
             if p["meets_slo"]:
                 break
-            rate *= 0.97  # the longer run saw a tail the search point did not: back off and measure again
+            rate *= 0.98  # the longer run saw a tail the search point did not: back off and measure again
         main_run, main_point = final
     # a rate at which a single answer was wrong is not a rate at which the SLO was met
     value = main_run["throughput_rps"] if main_point["meets_slo"] and not main_run.get("mismatches") else None
