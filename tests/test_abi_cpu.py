@@ -64,6 +64,24 @@ def test_conv_plan_arithmetic_and_rejections():
     assert plan((8, 8, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0), hint=(3 << 8) | (1 << 4))[0] == -1  # no such tile
 
 
+def test_transformed_launch_accounts_for_its_table_in_lds():
+    """The scheduler's figure for a conv that transforms its input on the way: the plan's dynamic LDS (the partial tiles of the
+    cross-wave sum) plus the table of scales and shifts, 64 bytes of zeros and 8 bytes per input channel; without a device the
+    kernel's static LDS and register count are left as planned."""
+    from paella_amd import _abi
+    lib = _abi.ops()
+    for c in (8, 64, 512, 1024):
+        rc, p = plan((c, 14, 14, 128, 1, 1, 1, 1, 0, 0, 1, 1, 1, 0, 0, 0))
+        assert rc == 0 and lib.paella_conv2d_plan_takes_input_transform(ctypes.byref(p)) == 1
+        plain, pre = _abi.LaunchDims(), _abi.LaunchDims()
+        assert lib.paella_conv2d_dims(ctypes.byref(p), ctypes.byref(plain)) == 0
+        assert lib.paella_conv2d_transformed_dims(ctypes.byref(p), ctypes.byref(pre)) == 0
+        assert (pre.grid, pre.block) == (plain.grid, plain.block)
+        assert pre.lds_bytes - p.dims.lds_bytes in range(64 + 8 * c, 64 + 8 * c + 256)   # + the kernel's few static bytes on a device
+    rc, p = plan((3, 32, 32, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0))           # channel-major reduction order: no such form
+    assert rc == 0 and lib.paella_conv2d_transformed_dims(ctypes.byref(p), ctypes.byref(_abi.LaunchDims())) == -2
+
+
 def test_weight_packing_layout():
     """Blob = weights as [k/4][m_pad][4] with k = (c, r, s) flattened, zero padded."""
     from paella_amd import _abi
